@@ -1,0 +1,225 @@
+/*
+ * librein — C ABI of the MI355X (gfx950) quantized-weight matmul path.
+ *
+ * Drop-in boundary for sixvolts/reinstinct's `src/quant` (repacked-v2 layouts)
+ * and `src/hip` (module / launch surface) for this one path.  Plain pointers
+ * and sizes only; every `void*` that is not marked "host" is a device pointer;
+ * `rein_stream_t` is a `hipStream_t` (NULL = the default stream).
+ *
+ * Error model (reference: src/hip/mod.rs:17-22): every call returns 0 on
+ * success, a positive `hipError_t` when a HIP call failed, or a negative
+ * REIN_E_* code for argument / library errors.  `rein_last_error()` returns a
+ * thread-local message of the form "<context>: <hipGetErrorString> (code N)".
+ * Nothing throws across the boundary.  There is no CPU fallback: if the HIP
+ * runtime or the gfx950 code object cannot be loaded, every compute call fails.
+ *
+ * Format ids are the reference's GgmlType discriminants
+ * (src/gguf/types.rs:16-35).
+ */
+#ifndef REIN_H
+#define REIN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    REIN_TYPE_Q4_0   = 2,
+    REIN_TYPE_Q8_0   = 8,
+    REIN_TYPE_Q4_K   = 12,
+    REIN_TYPE_Q5_K   = 13,
+    REIN_TYPE_Q6_K   = 14,
+    REIN_TYPE_IQ4_XS = 23
+};
+
+enum {
+    REIN_OK            = 0,
+    REIN_E_NOT_LOADED  = -1,   /* libamdhip64.so or the code object is not loaded */
+    REIN_E_BAD_FORMAT  = -2,   /* unknown / unsupported format id */
+    REIN_E_BAD_SHAPE   = -3,   /* dimension not a block multiple, zero, or out of range */
+    REIN_E_BAD_POINTER = -4,   /* NULL or misaligned pointer */
+    REIN_E_NO_KERNEL   = -5,   /* symbol missing from the code object */
+    REIN_E_TOO_LARGE   = -6    /* exceeds a documented fixed limit */
+};
+
+typedef void *rein_stream_t;   /* hipStream_t   */
+typedef void *rein_event_t;    /* hipEvent_t    */
+typedef void *rein_graph_t;    /* hipGraph_t    */
+typedef void *rein_graph_exec_t; /* hipGraphExec_t */
+typedef void *rein_module_t;   /* hipModule_t   */
+typedef void *rein_function_t; /* hipFunction_t */
+
+/* ------------------------------------------------------------------ errors */
+const char *rein_last_error(void);
+
+/* ---------------------------------------------------------- runtime / init */
+/* dlopen libamdhip64.so (candidates as src/hip/sys.rs:128-135), resolve the
+ * entry points of src/hip/sys.rs:57-101, and load the gfx950 code object.
+ * `hsaco_path` NULL = "rein_gfx950.hsaco" next to librein.so.  Idempotent;
+ * thread-safe (reference: OnceLock, sys.rs:122-127). */
+int rein_init(const char *hsaco_path);
+/* 1 when rein_init has succeeded in this process */
+int rein_is_loaded(void);
+
+/* src/hip/mod.rs:25-58, 88-131 */
+int rein_device_count(int *n);
+int rein_set_device(int device);
+int rein_get_device(int *device);
+int rein_device_name(int device, char *buf, int buf_len);   /* buf: host */
+int rein_device_total_mem(int device, size_t *bytes);
+int rein_mem_info(size_t *free_bytes, size_t *total_bytes);
+int rein_device_synchronize(void);
+
+/* DeviceBuf (src/hip/mod.rs:170-330) */
+int rein_malloc(void **dptr, size_t bytes);
+int rein_free(void *dptr);
+int rein_memcpy_h2d(void *dst, const void *src_host, size_t bytes);
+int rein_memcpy_d2h(void *dst_host, const void *src, size_t bytes);
+int rein_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int rein_memcpy_h2d_async(void *dst, const void *src_host, size_t bytes, rein_stream_t s);
+int rein_memcpy_d2h_async(void *dst_host, const void *src, size_t bytes, rein_stream_t s);
+int rein_memcpy_d2d_async(void *dst, const void *src, size_t bytes, rein_stream_t s);
+
+/* Stream / Event / Graph (src/hip/mod.rs:133-168, 332-435) */
+int rein_stream_create(rein_stream_t *s);
+int rein_stream_destroy(rein_stream_t s);
+int rein_stream_synchronize(rein_stream_t s);
+int rein_stream_wait_event(rein_stream_t s, rein_event_t e);
+int rein_event_create(rein_event_t *e);
+int rein_event_record(rein_event_t e, rein_stream_t s);
+int rein_event_synchronize(rein_event_t e);
+int rein_event_elapsed_ms(float *ms, rein_event_t start, rein_event_t stop);
+int rein_event_destroy(rein_event_t e);
+int rein_stream_begin_capture(rein_stream_t s);              /* mode Global, as the reference */
+int rein_stream_end_capture(rein_stream_t s, rein_graph_t *g);
+int rein_graph_instantiate(rein_graph_exec_t *ge, rein_graph_t g);
+int rein_graph_launch(rein_graph_exec_t ge, rein_stream_t s);
+int rein_graph_destroy(rein_graph_t g);
+int rein_graph_exec_destroy(rein_graph_exec_t ge);
+
+/* Module / Function::launch (src/hip/mod.rs:437-502): load any .hsaco, look a
+ * kernel up by name, launch with an array of pointers-to-values (kernelParams). */
+int rein_module_load(rein_module_t *m, const char *path);
+int rein_module_unload(rein_module_t m);
+int rein_module_get_function(rein_function_t *f, rein_module_t m, const char *name);
+/* the code object rein_init loaded, for looking up the reference-named kernels */
+int rein_builtin_module(rein_module_t *m);
+int rein_launch_kernel(rein_function_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                       unsigned by, unsigned bz, unsigned shared_bytes, rein_stream_t s,
+                       void **args);
+
+/* ------------------------------------------------------- src/quant mirror */
+/* repacked_n_sub_padded (src/quant/q4_k.rs:92-95 and per-format twins) */
+size_t rein_repacked_n_sub_padded(size_t in_dim);
+/* <fmt>::repacked_len (q4_k.rs:98-102, q5_k.rs, q6_k.rs, q8_0.rs:74-77,
+ * q4_0.rs:66-69, iq4_xs.rs:85-88); 0 for an unknown format */
+size_t rein_repacked_len(int fmt, size_t in_dim, size_t out_dim);
+/* on-disk geometry: weights per block / bytes per block (0 = unknown format) */
+int rein_block_size(int fmt);
+int rein_bytes_per_block(int fmt);
+/* <fmt>::repack_for_matvec (q4_k.rs:126-176, q5_k.rs:97-151, q6_k.rs:86-148,
+ * q8_0.rs:93-119, q4_0.rs:86-104, iq4_xs.rs:106-136).  Host to host:
+ * `src` holds out_dim*in_dim/block on-disk blocks, `dst` rein_repacked_len
+ * bytes.  The reference asserts on a bad in_dim; this returns REIN_E_BAD_SHAPE. */
+int rein_repack_for_matvec(int fmt, const uint8_t *src, size_t in_dim, size_t out_dim,
+                           uint8_t *dst);
+/* fp32 -> on-disk blocks, host to host, for building synthetic weights.  Q8_0
+ * follows q8_0::quantize_from_f32 (q8_0.rs:45-61); the reference has no
+ * quantizer for the other five formats, these follow ggml's reference
+ * quantizers in structure and produce valid blocks. n must be a block multiple. */
+int rein_quantize_weights(int fmt, const float *src, size_t n, uint8_t *dst);
+
+/* ------------------------------------------------------------- hot path */
+/* quantize_q8_f32 (kernels/quantize_q8.cpp:23-54; launcher qwen35.rs:3202-3211):
+ * x [n_vec][in_dim] fp32 -> xq [n_vec][in_dim/32] 40-byte BlockQ8. */
+int rein_quantize_q8(const float *x, void *xq, unsigned in_dim, unsigned n_vec, rein_stream_t s);
+
+/* launch_matvec_repacked_xq8 (src/runtime/qwen35.rs:2232-2280): y[out_dim] =
+ * W . xq for one pre-quantized activation row. */
+int rein_matvec_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
+                    unsigned out_dim, rein_stream_t s);
+/* matmul_kquant_batched_into without its quantize step (src/runtime/prefill.rs:
+ * 448-508): y[n_rows][out_dim], 1 <= n_rows <= 8; the weights are streamed once. */
+int rein_matvec_batched_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
+                            unsigned out_dim, unsigned n_rows, rein_stream_t s);
+/* matmul_mmq_into without its quantize step (src/runtime/prefill.rs:512-567):
+ * Y[p_rows][out_dim] = Xq . W^T on the int8 MFMA path. */
+int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
+                 unsigned out_dim, unsigned p_rows, rein_stream_t s);
+/* PrefillGemm::matmul_into_raw (src/runtime/prefill.rs:343-384): quantize x
+ * [n_rows][in_dim] into the caller's `xq_scratch` (n_rows*in_dim/32*40 bytes),
+ * then dispatch by row count: 1 -> matvec, 2..8 -> batched matvec (the reference
+ * switches to its narrow MMQ at 5), above -> MMQ. */
+int rein_matmul(int fmt, const void *w, const float *x, float *y, unsigned in_dim,
+                unsigned out_dim, unsigned n_rows, void *xq_scratch, rein_stream_t s);
+/* Which path rein_matmul takes: 0 matvec, 1 batched matvec, 2 MMQ; <0 on error. */
+int rein_matmul_path(int fmt, unsigned n_rows);
+
+/* Debug / parity: per-block int32 dots exactly as the kernels form them.
+ * out [n_rows][out_dim][in_dim/32][parts], parts = rein_block_dot_parts(fmt)
+ * (2 for Q6_K: one per 16-weight half, each minus 32*sum(q8); Q4_0: dot minus
+ * 8*sum(q8); otherwise the raw dot).  via_mfma != 0 takes the dots from the MMQ
+ * kernel's MFMA tiles instead of the matvec's v_dot4 path. */
+int rein_block_dot_parts(int fmt);
+int rein_block_dots(int fmt, const void *w, const void *xq, int32_t *out, unsigned in_dim,
+                    unsigned out_dim, unsigned n_rows, int via_mfma, rein_stream_t s);
+
+/* ------------------------------------------------------------------- MoE */
+/* moe_topk_f32 (kernels/moe_topk.cpp:17-108; launcher qwen35.rs:2873-2886) */
+int rein_moe_topk(const float *logits, unsigned n_tok, unsigned n_expert, unsigned n_used,
+                  int32_t *out_ids, float *out_weights, rein_stream_t s);
+/* launch_moe_sort (qwen35.rs:2892-2938; kernels/moe_expert_sort.cpp:27-75):
+ * counting sort of ids [n_entries] by expert.  count/cursor: n_expert ints of
+ * scratch; perm [n_entries]; expert_off/tile_off [n_expert+1]; bn = tokens per
+ * GEMM tile used for tile_off. */
+int rein_moe_sort(const int32_t *ids, unsigned n_entries, unsigned n_expert, unsigned bn,
+                  int32_t *count, int32_t *cursor, int32_t *perm, int32_t *expert_off,
+                  int32_t *tile_off, rein_stream_t s);
+/* moe_gather_xq / moe_scatter_rows (kernels/moe_expert_sort.cpp:81-110) */
+int rein_moe_gather_xq(const void *xq_src, const int32_t *perm, void *xq_dst, unsigned nsub,
+                       unsigned n_used, unsigned n_entries, rein_stream_t s);
+int rein_moe_scatter_rows(const float *src, const int32_t *perm, float *dst, unsigned dim,
+                          unsigned n_entries, rein_stream_t s);
+/* launch_moe_grouped_gemm (qwen35.rs:3036-3064; kernels/mmq_gemm_*_grouped.cpp):
+ * rows expert_off[e]..expert_off[e+1] of the sorted xq / y against
+ * slab + e*bytes_per_expert.  n_entries = total sorted rows (upper bound for the
+ * launch). Formats: Q4_K, Q5_K, Q6_K, Q8_0. */
+int rein_moe_grouped_gemm(int fmt, const void *slab, unsigned bytes_per_expert,
+                          const int32_t *expert_off, const int32_t *tile_off, unsigned n_expert,
+                          const void *xq, float *y, unsigned in_dim, unsigned out_dim,
+                          unsigned n_entries, rein_stream_t s);
+/* swiglu_mul_f32 (kernels/swiglu.cpp:10-21) */
+int rein_swiglu_mul(const float *gate, const float *up, float *out, unsigned n, rein_stream_t s);
+/* moe_combine_f32 (kernels/moe_combine.cpp:15-38) */
+int rein_moe_combine(const float *experts, const int32_t *ids, const float *weights,
+                     const float *down_exps_s, float *out, unsigned n_tok, unsigned hidden,
+                     unsigned n_used, rein_stream_t s);
+/* tokens per grouped-GEMM tile the launcher assumes for `tile_off` (the
+ * reference's MOE_GEMM_BN, qwen35.rs:127) */
+unsigned rein_moe_gemm_bn(void);
+
+/* Workspace sizes for rein_moe_ffn, in bytes, for n_tok tokens. */
+typedef struct {
+    unsigned n_tok, hidden, n_expert, n_used, expert_ff;
+    int gate_up_fmt;    /* gate_exps / up_exps format (reference: Q4_K) */
+    int down_fmt;       /* down_exps format (reference: Q5_K or Q6_K)  */
+} rein_moe_shape;
+size_t rein_moe_workspace_bytes(const rein_moe_shape *shape);
+/* The routed-expert part of step_moe_ffn_batched (qwen35.rs:2788-2870), given
+ * router logits: top-k -> quantize -> sort -> gather -> grouped gate / up GEMM ->
+ * SwiGLU -> quantize -> grouped down GEMM -> scatter -> weighted combine.
+ * gate_exps / up_exps: n_expert slabs [hidden -> expert_ff]; down_exps:
+ * [expert_ff -> hidden]; down_exps_s [n_expert] fp32 (the reference passes
+ * ones).  `workspace` holds rein_moe_workspace_bytes; out [n_tok][hidden].
+ * No host synchronisation, no allocation. */
+int rein_moe_ffn(const rein_moe_shape *shape, const float *x, const float *logits,
+                 const void *gate_exps, const void *up_exps, const void *down_exps,
+                 const float *down_exps_s, void *workspace, float *out, rein_stream_t s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REIN_H */

@@ -1,0 +1,128 @@
+"""ctypes loader for librein.so.  Fails loudly when the library is missing."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "librein.so")
+HSACO_PATH = os.path.join(_HERE, "rein_gfx950.hsaco")
+
+
+class ReinError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"{msg} [rc={code}]")
+        self.code = code
+
+
+class MoeShape(C.Structure):
+    _fields_ = [("n_tok", C.c_uint), ("hidden", C.c_uint), ("n_expert", C.c_uint), ("n_used", C.c_uint),
+                ("expert_ff", C.c_uint), ("gate_up_fmt", C.c_int), ("down_fmt", C.c_int)]
+
+
+_vp, _u, _i, _sz = C.c_void_p, C.c_uint, C.c_int, C.c_size_t
+_P = C.POINTER
+
+# name -> (restype, argtypes); every symbol declared in include/rein.h
+SIGNATURES = {
+    "rein_last_error": (C.c_char_p, []),
+    "rein_init": (_i, [C.c_char_p]),
+    "rein_is_loaded": (_i, []),
+    "rein_device_count": (_i, [_P(_i)]),
+    "rein_set_device": (_i, [_i]),
+    "rein_get_device": (_i, [_P(_i)]),
+    "rein_device_name": (_i, [_i, C.c_char_p, _i]),
+    "rein_device_total_mem": (_i, [_i, _P(_sz)]),
+    "rein_mem_info": (_i, [_P(_sz), _P(_sz)]),
+    "rein_device_synchronize": (_i, []),
+    "rein_malloc": (_i, [_P(_vp), _sz]),
+    "rein_free": (_i, [_vp]),
+    "rein_memcpy_h2d": (_i, [_vp, _vp, _sz]),
+    "rein_memcpy_d2h": (_i, [_vp, _vp, _sz]),
+    "rein_memcpy_d2d": (_i, [_vp, _vp, _sz]),
+    "rein_memcpy_h2d_async": (_i, [_vp, _vp, _sz, _vp]),
+    "rein_memcpy_d2h_async": (_i, [_vp, _vp, _sz, _vp]),
+    "rein_memcpy_d2d_async": (_i, [_vp, _vp, _sz, _vp]),
+    "rein_stream_create": (_i, [_P(_vp)]),
+    "rein_stream_destroy": (_i, [_vp]),
+    "rein_stream_synchronize": (_i, [_vp]),
+    "rein_stream_wait_event": (_i, [_vp, _vp]),
+    "rein_event_create": (_i, [_P(_vp)]),
+    "rein_event_record": (_i, [_vp, _vp]),
+    "rein_event_synchronize": (_i, [_vp]),
+    "rein_event_elapsed_ms": (_i, [_P(C.c_float), _vp, _vp]),
+    "rein_event_destroy": (_i, [_vp]),
+    "rein_stream_begin_capture": (_i, [_vp]),
+    "rein_stream_end_capture": (_i, [_vp, _P(_vp)]),
+    "rein_graph_instantiate": (_i, [_P(_vp), _vp]),
+    "rein_graph_launch": (_i, [_vp, _vp]),
+    "rein_graph_destroy": (_i, [_vp]),
+    "rein_graph_exec_destroy": (_i, [_vp]),
+    "rein_module_load": (_i, [_P(_vp), C.c_char_p]),
+    "rein_module_unload": (_i, [_vp]),
+    "rein_module_get_function": (_i, [_P(_vp), _vp, C.c_char_p]),
+    "rein_builtin_module": (_i, [_P(_vp)]),
+    "rein_launch_kernel": (_i, [_vp, _u, _u, _u, _u, _u, _u, _u, _vp, _P(_vp)]),
+    "rein_repacked_n_sub_padded": (_sz, [_sz]),
+    "rein_repacked_len": (_sz, [_i, _sz, _sz]),
+    "rein_block_size": (_i, [_i]),
+    "rein_bytes_per_block": (_i, [_i]),
+    "rein_repack_for_matvec": (_i, [_i, _vp, _sz, _sz, _vp]),
+    "rein_quantize_weights": (_i, [_i, _vp, _sz, _vp]),
+    "rein_quantize_q8": (_i, [_vp, _vp, _u, _u, _vp]),
+    "rein_matvec_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _vp]),
+    "rein_matvec_batched_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_mmq_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_matmul": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _vp]),
+    "rein_matmul_path": (_i, [_i, _u]),
+    "rein_block_dot_parts": (_i, [_i]),
+    "rein_block_dots": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _i, _vp]),
+    "rein_moe_topk": (_i, [_vp, _u, _u, _u, _vp, _vp, _vp]),
+    "rein_moe_sort": (_i, [_vp, _u, _u, _u, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "rein_moe_gather_xq": (_i, [_vp, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_moe_scatter_rows": (_i, [_vp, _vp, _vp, _u, _u, _vp]),
+    "rein_moe_grouped_gemm": (_i, [_i, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_swiglu_mul": (_i, [_vp, _vp, _vp, _u, _vp]),
+    "rein_moe_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_moe_gemm_bn": (_u, []),
+    "rein_moe_workspace_bytes": (_sz, [_P(MoeShape)]),
+    "rein_moe_ffn": (_i, [_P(MoeShape), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """dlopen librein.so and type every entry point (no GPU needed for this)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(SO_PATH):
+        raise ReinError(-1, f"{SO_PATH} is not built: run `make -C reinstinct_amd/csrc` "
+                            "(or __graft_entry__.build()); there is no fallback path")
+    handle = C.CDLL(SO_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(handle, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = handle
+    return _lib
+
+
+class _Lazy:
+    def __getattr__(self, name):
+        return getattr(load(), name)
+
+
+lib = _Lazy()
+
+
+def check(rc):
+    """Turn a non-zero status into ReinError carrying rein_last_error()."""
+    if rc != 0:
+        msg = load().rein_last_error()
+        raise ReinError(rc, msg.decode() if msg else "unknown error")
+    return rc
+
+
+def init():
+    """Bind libamdhip64.so and load the gfx950 code object (needs a GPU)."""
+    check(load().rein_init(HSACO_PATH.encode()))

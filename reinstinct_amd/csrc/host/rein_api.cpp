@@ -1,0 +1,538 @@
+// librein C ABI: runtime (dlopen'd HIP, code-object loading, kernel lookup by
+// name) and the host-side dispatch of the quantized matmul path.  Mirrors the
+// reference's src/hip (module / launch surface) and the launch sites in
+// src/runtime/{qwen35,prefill}.rs; geometry is chosen here for MI355X
+// (256 CUs, wave64) instead of being fixed per kernel.
+#include <dlfcn.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "../../../include/rein.h"
+#include "hip_api.h"
+
+using namespace rein;
+
+namespace {
+
+struct Runtime {
+    const HipApi* api = nullptr;
+    hipModule_t   module = nullptr;
+    std::mutex    mu;
+    std::unordered_map<std::string, hipFunction_t> fns;
+    bool loaded = false;
+};
+
+Runtime g_rt;
+std::mutex g_init_mu;
+
+std::string default_hsaco_path()
+{
+    Dl_info info;
+    if (dladdr(reinterpret_cast<const void*>(&default_hsaco_path), &info) && info.dli_fname) {
+        std::string p(info.dli_fname);
+        const size_t slash = p.find_last_of('/');
+        const std::string dir = slash == std::string::npos ? std::string(".") : p.substr(0, slash);
+        return dir + "/rein_gfx950.hsaco";
+    }
+    return "rein_gfx950.hsaco";
+}
+
+int need_api(const HipApi** out)
+{
+    std::string err;
+    const HipApi* api = hip_api(&err);
+    if (!api) return fail(REIN_E_NOT_LOADED, err);
+    *out = api;
+    return 0;
+}
+
+int need_runtime()
+{
+    if (!g_rt.loaded) return fail(REIN_E_NOT_LOADED, "librein: rein_init has not succeeded; no CPU fallback exists");
+    return 0;
+}
+
+int get_fn(const std::string& name, hipFunction_t* f)
+{
+    if (int rc = need_runtime()) return rc;
+    std::lock_guard<std::mutex> lock(g_rt.mu);
+    auto it = g_rt.fns.find(name);
+    if (it != g_rt.fns.end()) {
+        *f = it->second;
+        return 0;
+    }
+    hipFunction_t fn = nullptr;
+    const hipError_t e = g_rt.api->ModuleGetFunction(&fn, g_rt.module, name.c_str());
+    if (e != 0) {
+        check_hip(g_rt.api, e, ("hipModuleGetFunction(" + name + ")").c_str());
+        return REIN_E_NO_KERNEL;
+    }
+    g_rt.fns.emplace(name, fn);
+    *f = fn;
+    return 0;
+}
+
+int launch(const std::string& name, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned shmem,
+           rein_stream_t s, void** args)
+{
+    hipFunction_t f;
+    if (int rc = get_fn(name, &f)) return rc;
+    return check_hip(g_rt.api, g_rt.api->ModuleLaunchKernel(f, gx, gy, gz, bx, 1, 1, shmem, s, args, nullptr),
+                     ("hipModuleLaunchKernel(" + name + ")").c_str());
+}
+
+const char* fmt_tag(int fmt)
+{
+    switch (fmt) {
+    case REIN_TYPE_Q4_0:   return "q4_0";
+    case REIN_TYPE_Q8_0:   return "q8_0";
+    case REIN_TYPE_Q4_K:   return "q4k";
+    case REIN_TYPE_Q5_K:   return "q5k";
+    case REIN_TYPE_Q6_K:   return "q6k";
+    case REIN_TYPE_IQ4_XS: return "iq4xs";
+    default: return nullptr;
+    }
+}
+
+int check_shape(const char* who, int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    const int bs = rein_block_size(fmt);
+    if (!bs) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": unknown format " + std::to_string(fmt));
+    if (in_dim == 0 || in_dim % (unsigned)bs != 0)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": in_dim " + std::to_string(in_dim) + " is not a non-zero multiple of " + std::to_string(bs));
+    if (out_dim == 0 || n_rows == 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": out_dim and the row count must be non-zero");
+    return 0;
+}
+
+int check_ptr(const char* who, const void* p, size_t align, const char* what)
+{
+    if (!p) return fail(REIN_E_BAD_POINTER, std::string(who) + ": " + what + " is NULL");
+    if (reinterpret_cast<uintptr_t>(p) % align != 0)
+        return fail(REIN_E_BAD_POINTER, std::string(who) + ": " + what + " must be " + std::to_string(align) + "-byte aligned");
+    return 0;
+}
+
+unsigned env_u(const char* name, unsigned dflt)
+{
+    const char* v = std::getenv(name);
+    return v && *v ? (unsigned)std::strtoul(v, nullptr, 10) : dflt;
+}
+
+constexpr unsigned kCUs = 256;    // MI355X
+
+// Rows per wavefront pass for the decode matvec.  More rows per wave amortise
+// the activation read and the cross-lane reduction; fewer rows put more waves in
+// flight.  Keep at least ~16 waves per CU unless the matrix is too small.
+unsigned pick_rows_per_wave(unsigned out_dim, unsigned batch)
+{
+    const unsigned forced = env_u("REIN_MV_ROWS", 0);
+    unsigned r = 4;
+    while (r > 1 && (r * batch > 16 || (out_dim + r - 1) / r < kCUs * 16)) r >>= 1;
+    if (forced == 1 || forced == 2 || forced == 4) r = forced;
+    while (r > 1 && r * batch > 16) r >>= 1;
+    return r;
+}
+
+unsigned batch_slot(unsigned n_rows) { return n_rows <= 1 ? 1 : n_rows <= 2 ? 2 : n_rows <= 4 ? 4 : 8; }
+
+int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
+                  unsigned out_dim, unsigned n_rows, rein_stream_t s)
+{
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_rows)) return rc;
+    if (n_rows > 8) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most 8 activation rows");
+    if (int rc = check_ptr(who, w, 16, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    const unsigned b = batch_slot(n_rows);
+    const unsigned r = pick_rows_per_wave(out_dim, b);
+    const unsigned wpb = 4;
+    const unsigned groups = (out_dim + r - 1) / r;
+    const unsigned grid = (groups + wpb - 1) / wpb;
+    const std::string name = std::string("rein_mv_") + fmt_tag(fmt) + "_r" + std::to_string(r) + "_b" + std::to_string(b);
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+    return launch(name, grid, 1, 1, wpb * 64, 0, s, args);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* rein_last_error(void) { return last_error(); }
+
+int rein_init(const char* hsaco_path)
+{
+    std::lock_guard<std::mutex> lock(g_init_mu);
+    if (g_rt.loaded) return 0;
+    const HipApi* api;
+    if (int rc = need_api(&api)) return rc;
+    const std::string path = hsaco_path && *hsaco_path ? hsaco_path : default_hsaco_path();
+    hipModule_t m = nullptr;
+    if (int rc = check_hip(api, api->ModuleLoad(&m, path.c_str()), ("hipModuleLoad(" + path + ")").c_str())) return rc;
+    g_rt.api = api;
+    g_rt.module = m;
+    g_rt.loaded = true;
+    return 0;
+}
+
+int rein_is_loaded(void) { return g_rt.loaded ? 1 : 0; }
+
+#define API_OR_RETURN() const HipApi* api; if (int rc_ = need_api(&api)) return rc_
+
+int rein_device_count(int* n) { API_OR_RETURN(); return check_hip(api, api->GetDeviceCount(n), "hipGetDeviceCount"); }
+int rein_set_device(int d) { API_OR_RETURN(); return check_hip(api, api->SetDevice(d), "hipSetDevice"); }
+int rein_get_device(int* d) { API_OR_RETURN(); return check_hip(api, api->GetDevice(d), "hipGetDevice"); }
+int rein_device_name(int d, char* buf, int len) { API_OR_RETURN(); return check_hip(api, api->DeviceGetName(buf, len, d), "hipDeviceGetName"); }
+int rein_device_total_mem(int d, size_t* b) { API_OR_RETURN(); return check_hip(api, api->DeviceTotalMem(b, d), "hipDeviceTotalMem"); }
+int rein_mem_info(size_t* f, size_t* t) { API_OR_RETURN(); return check_hip(api, api->MemGetInfo(f, t), "hipMemGetInfo"); }
+int rein_device_synchronize(void) { API_OR_RETURN(); return check_hip(api, api->DeviceSynchronize(), "hipDeviceSynchronize"); }
+
+int rein_malloc(void** p, size_t bytes) { API_OR_RETURN(); return check_hip(api, api->Malloc(p, bytes), "hipMalloc"); }
+int rein_free(void* p) { API_OR_RETURN(); return check_hip(api, api->Free(p), "hipFree"); }
+int rein_memcpy_h2d(void* d, const void* s, size_t n) { API_OR_RETURN(); return check_hip(api, api->Memcpy(d, s, n, hipMemcpyHostToDevice), "hipMemcpy H2D"); }
+int rein_memcpy_d2h(void* d, const void* s, size_t n) { API_OR_RETURN(); return check_hip(api, api->Memcpy(d, s, n, hipMemcpyDeviceToHost), "hipMemcpy D2H"); }
+int rein_memcpy_d2d(void* d, const void* s, size_t n) { API_OR_RETURN(); return check_hip(api, api->Memcpy(d, s, n, hipMemcpyDeviceToDevice), "hipMemcpy D2D"); }
+int rein_memcpy_h2d_async(void* d, const void* s, size_t n, rein_stream_t st) { API_OR_RETURN(); return check_hip(api, api->MemcpyAsync(d, s, n, hipMemcpyHostToDevice, st), "hipMemcpyAsync H2D"); }
+int rein_memcpy_d2h_async(void* d, const void* s, size_t n, rein_stream_t st) { API_OR_RETURN(); return check_hip(api, api->MemcpyAsync(d, s, n, hipMemcpyDeviceToHost, st), "hipMemcpyAsync D2H"); }
+int rein_memcpy_d2d_async(void* d, const void* s, size_t n, rein_stream_t st) { API_OR_RETURN(); return check_hip(api, api->MemcpyAsync(d, s, n, hipMemcpyDeviceToDevice, st), "hipMemcpyAsync D2D"); }
+
+int rein_stream_create(rein_stream_t* s) { API_OR_RETURN(); return check_hip(api, api->StreamCreate(s), "hipStreamCreate"); }
+int rein_stream_destroy(rein_stream_t s) { API_OR_RETURN(); return check_hip(api, api->StreamDestroy(s), "hipStreamDestroy"); }
+int rein_stream_synchronize(rein_stream_t s) { API_OR_RETURN(); return check_hip(api, api->StreamSynchronize(s), "hipStreamSynchronize"); }
+int rein_stream_wait_event(rein_stream_t s, rein_event_t e) { API_OR_RETURN(); return check_hip(api, api->StreamWaitEvent(s, e, 0), "hipStreamWaitEvent"); }
+int rein_event_create(rein_event_t* e) { API_OR_RETURN(); return check_hip(api, api->EventCreate(e), "hipEventCreate"); }
+int rein_event_record(rein_event_t e, rein_stream_t s) { API_OR_RETURN(); return check_hip(api, api->EventRecord(e, s), "hipEventRecord"); }
+int rein_event_synchronize(rein_event_t e) { API_OR_RETURN(); return check_hip(api, api->EventSynchronize(e), "hipEventSynchronize"); }
+int rein_event_elapsed_ms(float* ms, rein_event_t a, rein_event_t b) { API_OR_RETURN(); return check_hip(api, api->EventElapsedTime(ms, a, b), "hipEventElapsedTime"); }
+int rein_event_destroy(rein_event_t e) { API_OR_RETURN(); return check_hip(api, api->EventDestroy(e), "hipEventDestroy"); }
+int rein_stream_begin_capture(rein_stream_t s) { API_OR_RETURN(); return check_hip(api, api->StreamBeginCapture(s, hipStreamCaptureModeGlobal), "hipStreamBeginCapture"); }
+int rein_stream_end_capture(rein_stream_t s, rein_graph_t* g) { API_OR_RETURN(); return check_hip(api, api->StreamEndCapture(s, g), "hipStreamEndCapture"); }
+int rein_graph_instantiate(rein_graph_exec_t* ge, rein_graph_t g) { API_OR_RETURN(); return check_hip(api, api->GraphInstantiate(ge, g, nullptr, nullptr, 0), "hipGraphInstantiate"); }
+int rein_graph_launch(rein_graph_exec_t ge, rein_stream_t s) { API_OR_RETURN(); return check_hip(api, api->GraphLaunch(ge, s), "hipGraphLaunch"); }
+int rein_graph_destroy(rein_graph_t g) { API_OR_RETURN(); return check_hip(api, api->GraphDestroy(g), "hipGraphDestroy"); }
+int rein_graph_exec_destroy(rein_graph_exec_t ge) { API_OR_RETURN(); return check_hip(api, api->GraphExecDestroy(ge), "hipGraphExecDestroy"); }
+
+int rein_module_load(rein_module_t* m, const char* path)
+{
+    API_OR_RETURN();
+    if (!path) return fail(REIN_E_BAD_POINTER, "rein_module_load: path is NULL");
+    return check_hip(api, api->ModuleLoad(m, path), "hipModuleLoad");
+}
+int rein_module_unload(rein_module_t m) { API_OR_RETURN(); return check_hip(api, api->ModuleUnload(m), "hipModuleUnload"); }
+int rein_module_get_function(rein_function_t* f, rein_module_t m, const char* name)
+{
+    API_OR_RETURN();
+    if (!name) return fail(REIN_E_BAD_POINTER, "rein_module_get_function: name is NULL");
+    return check_hip(api, api->ModuleGetFunction(f, m, name), "hipModuleGetFunction");
+}
+int rein_builtin_module(rein_module_t* m)
+{
+    if (int rc = need_runtime()) return rc;
+    *m = g_rt.module;
+    return 0;
+}
+int rein_launch_kernel(rein_function_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
+                       unsigned bz, unsigned shared_bytes, rein_stream_t s, void** args)
+{
+    API_OR_RETURN();
+    return check_hip(api, api->ModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, shared_bytes, s, args, nullptr),
+                     "hipModuleLaunchKernel");
+}
+
+// ------------------------------------------------------------------ hot path
+
+int rein_quantize_q8(const float* x, void* xq, unsigned in_dim, unsigned n_vec, rein_stream_t s)
+{
+    if (in_dim == 0 || in_dim % 32 != 0 || n_vec == 0)
+        return fail(REIN_E_BAD_SHAPE, "rein_quantize_q8: in_dim must be a non-zero multiple of 32 and n_vec non-zero");
+    if (n_vec > 65535) return fail(REIN_E_TOO_LARGE, "rein_quantize_q8: at most 65535 vectors per call");
+    if (int rc = check_ptr("rein_quantize_q8", x, 4, "x")) return rc;
+    if (int rc = check_ptr("rein_quantize_q8", xq, 8, "xq")) return rc;
+    // 8 sub-blocks per 256-thread workgroup, as the reference launch (qwen35.rs:3202-3211)
+    const unsigned gx = (in_dim + 255) / 256;
+    void* args[] = {(void*)&x, (void*)&xq, (void*)&in_dim};
+    return launch("quantize_q8_f32", gx, n_vec, 1, 256, 0, s, args);
+}
+
+int rein_matvec_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                    rein_stream_t s)
+{
+    return launch_matvec("rein_matvec_xq8", fmt, w, xq, y, in_dim, out_dim, 1, s);
+}
+
+int rein_matvec_batched_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
+                            unsigned out_dim, unsigned n_rows, rein_stream_t s)
+{
+    return launch_matvec("rein_matvec_batched_xq8", fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+}
+
+int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                 unsigned p_rows, rein_stream_t s)
+{
+    const char* who = "rein_mmq_xq8";
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
+    if (int rc = check_ptr(who, w, 16, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    // token tile: 32 for a handful of rows, wider once the batch can fill it
+    unsigned tm = p_rows <= 32 ? 32 : p_rows <= 64 ? 64 : 128;
+    const unsigned forced = env_u("REIN_MMQ_TM", 0);
+    if (forced == 32 || forced == 64 || forced == 128) tm = forced;
+    const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + tm - 1) / tm;
+    if (n_tt > 65535) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many token tiles");
+    const std::string name = std::string("rein_mmq_") + fmt_tag(fmt) + "_t" + std::to_string(tm);
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
+    return launch(name, n_rb, n_tt, 1, 256, 0, s, args);
+}
+
+int rein_matmul_path(int fmt, unsigned n_rows)
+{
+    if (!rein_block_size(fmt)) return fail(REIN_E_BAD_FORMAT, "rein_matmul_path: unknown format " + std::to_string(fmt));
+    if (n_rows == 0) return fail(REIN_E_BAD_SHAPE, "rein_matmul_path: n_rows is zero");
+    if (n_rows == 1) return 0;
+    return n_rows <= 8 ? 1 : 2;
+}
+
+int rein_matmul(int fmt, const void* w, const float* x, float* y, unsigned in_dim, unsigned out_dim,
+                unsigned n_rows, void* xq_scratch, rein_stream_t s)
+{
+    if (int rc = check_shape("rein_matmul", fmt, in_dim, out_dim, n_rows)) return rc;
+    if (int rc = rein_quantize_q8(x, xq_scratch, in_dim, n_rows, s)) return rc;
+    switch (rein_matmul_path(fmt, n_rows)) {
+    case 0:  return rein_matvec_xq8(fmt, w, xq_scratch, y, in_dim, out_dim, s);
+    case 1:  return rein_matvec_batched_xq8(fmt, w, xq_scratch, y, in_dim, out_dim, n_rows, s);
+    default: return rein_mmq_xq8(fmt, w, xq_scratch, y, in_dim, out_dim, n_rows, s);
+    }
+}
+
+int rein_block_dot_parts(int fmt) { return fmt == REIN_TYPE_Q6_K ? 2 : (rein_block_size(fmt) ? 1 : 0); }
+
+int rein_block_dots(int fmt, const void* w, const void* xq, int32_t* out, unsigned in_dim, unsigned out_dim,
+                    unsigned n_rows, int via_mfma, rein_stream_t s)
+{
+    const char* who = "rein_block_dots";
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_rows)) return rc;
+    if (int rc = check_ptr(who, w, 16, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, out, 4, "out")) return rc;
+    if (n_rows > 65535) return fail(REIN_E_TOO_LARGE, "rein_block_dots: at most 65535 rows");
+    if (via_mfma) {
+        const std::string name = std::string("rein_mmq_dots_") + fmt_tag(fmt);
+        void* args[] = {(void*)&w, (void*)&xq, (void*)&out, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+        return launch(name, (out_dim + 127) / 128, (n_rows + 31) / 32, 1, 256, 0, s, args);
+    }
+    const std::string name = std::string("rein_block_dots_") + fmt_tag(fmt);
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&out, (void*)&in_dim, (void*)&out_dim};
+    return launch(name, out_dim < 4096 ? out_dim : 4096, n_rows, 1, 64, 0, s, args);
+}
+
+// ------------------------------------------------------------------------ MoE
+
+unsigned rein_moe_gemm_bn(void) { return 32; }
+
+int rein_moe_topk(const float* logits, unsigned n_tok, unsigned n_expert, unsigned n_used, int32_t* out_ids,
+                  float* out_weights, rein_stream_t s)
+{
+    if (n_tok == 0 || n_expert == 0 || n_used == 0 || n_used > 64 || n_used > n_expert)
+        return fail(REIN_E_BAD_SHAPE, "rein_moe_topk: need n_tok > 0 and 1 <= n_used <= min(64, n_expert)");
+    if (n_expert > 12288) return fail(REIN_E_TOO_LARGE, "rein_moe_topk: at most 12288 experts (LDS)");
+    if (int rc = check_ptr("rein_moe_topk", logits, 4, "logits")) return rc;
+    if (int rc = check_ptr("rein_moe_topk", out_ids, 4, "out_ids")) return rc;
+    if (int rc = check_ptr("rein_moe_topk", out_weights, 4, "out_weights")) return rc;
+    int ne = (int)n_expert, nu = (int)n_used;
+    void* args[] = {(void*)&logits, (void*)&ne, (void*)&nu, (void*)&out_ids, (void*)&out_weights};
+    return launch("moe_topk_f32", n_tok, 1, 1, 128, n_expert * 4, s, args);
+}
+
+int rein_moe_sort(const int32_t* ids, unsigned n_entries, unsigned n_expert, unsigned bn, int32_t* count,
+                  int32_t* cursor, int32_t* perm, int32_t* expert_off, int32_t* tile_off, rein_stream_t s)
+{
+    if (n_entries == 0 || n_expert == 0 || bn == 0)
+        return fail(REIN_E_BAD_SHAPE, "rein_moe_sort: n_entries, n_expert and bn must be non-zero");
+    const void* ptrs[] = {ids, count, cursor, perm, expert_off, tile_off};
+    for (const void* p : ptrs)
+        if (int rc = check_ptr("rein_moe_sort", p, 4, "buffer")) return rc;
+    const unsigned ge = (n_expert + 255) / 256, gn = (n_entries + 255) / 256;
+    {
+        void* a[] = {(void*)&count, (void*)&n_expert};
+        if (int rc = launch("moe_sort_zero", ge, 1, 1, 256, 0, s, a)) return rc;
+    }
+    {
+        void* a[] = {(void*)&ids, (void*)&count, (void*)&n_entries, (void*)&n_expert};
+        if (int rc = launch("moe_sort_histogram", gn, 1, 1, 256, 0, s, a)) return rc;
+    }
+    {
+        void* a[] = {(void*)&count, (void*)&expert_off, (void*)&tile_off, (void*)&n_expert, (void*)&bn};
+        if (int rc = launch("moe_sort_scan", 1, 1, 1, 64, 0, s, a)) return rc;
+    }
+    {
+        void* a[] = {(void*)&cursor, (void*)&n_expert};
+        if (int rc = launch("moe_sort_zero", ge, 1, 1, 256, 0, s, a)) return rc;
+    }
+    void* a[] = {(void*)&ids, (void*)&expert_off, (void*)&cursor, (void*)&perm, (void*)&n_entries, (void*)&n_expert};
+    return launch("moe_sort_scatter", gn, 1, 1, 256, 0, s, a);
+}
+
+int rein_moe_gather_xq(const void* xq_src, const int32_t* perm, void* xq_dst, unsigned nsub, unsigned n_used,
+                       unsigned n_entries, rein_stream_t s)
+{
+    if (nsub == 0 || n_used == 0 || n_entries == 0) return fail(REIN_E_BAD_SHAPE, "rein_moe_gather_xq: zero dimension");
+    if (int rc = check_ptr("rein_moe_gather_xq", xq_src, 8, "xq_src")) return rc;
+    if (int rc = check_ptr("rein_moe_gather_xq", xq_dst, 8, "xq_dst")) return rc;
+    if (int rc = check_ptr("rein_moe_gather_xq", perm, 4, "perm")) return rc;
+    const unsigned gx = (nsub * 5 + 255) / 256, gy = n_entries < 65535 ? n_entries : 65535;
+    void* a[] = {(void*)&xq_src, (void*)&perm, (void*)&xq_dst, (void*)&nsub, (void*)&n_used, (void*)&n_entries};
+    return launch("moe_gather_xq", gx, gy, 1, 256, 0, s, a);
+}
+
+int rein_moe_scatter_rows(const float* src, const int32_t* perm, float* dst, unsigned dim, unsigned n_entries,
+                          rein_stream_t s)
+{
+    if (dim == 0 || n_entries == 0) return fail(REIN_E_BAD_SHAPE, "rein_moe_scatter_rows: zero dimension");
+    if (int rc = check_ptr("rein_moe_scatter_rows", src, 4, "src")) return rc;
+    if (int rc = check_ptr("rein_moe_scatter_rows", dst, 4, "dst")) return rc;
+    if (int rc = check_ptr("rein_moe_scatter_rows", perm, 4, "perm")) return rc;
+    const unsigned gx = (dim + 255) / 256, gy = n_entries < 65535 ? n_entries : 65535;
+    void* a[] = {(void*)&src, (void*)&perm, (void*)&dst, (void*)&dim, (void*)&n_entries};
+    return launch("moe_scatter_rows", gx, gy, 1, 256, 0, s, a);
+}
+
+int rein_moe_grouped_gemm(int fmt, const void* slab, unsigned bytes_per_expert, const int32_t* expert_off,
+                          const int32_t* tile_off, unsigned n_expert, const void* xq, float* y, unsigned in_dim,
+                          unsigned out_dim, unsigned n_entries, rein_stream_t s)
+{
+    const char* who = "rein_moe_grouped_gemm";
+    if (fmt != REIN_TYPE_Q4_K && fmt != REIN_TYPE_Q5_K && fmt != REIN_TYPE_Q6_K && fmt != REIN_TYPE_Q8_0)
+        return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_entries)) return rc;
+    if (n_expert == 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_expert is zero");
+    if (bytes_per_expert % 16 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert must be a multiple of 16");
+    if (int rc = check_ptr(who, slab, 16, "slab")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    if (int rc = check_ptr(who, expert_off, 4, "expert_off")) return rc;
+    if (int rc = check_ptr(who, tile_off, 4, "tile_off")) return rc;
+    // the tile count lives on the device; launch its upper bound (qwen35.rs:3051)
+    const unsigned bn = rein_moe_gemm_bn();
+    unsigned tile_ub = (n_entries + bn - 1) / bn + n_expert;
+    if (tile_ub > 65535) tile_ub = 65535;       // the kernel strides over tiles
+    const std::string name = std::string("mmq_gemm_") + fmt_tag(fmt) + "_grouped_f32";
+    void* a[] = {(void*)&slab, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off, (void*)&n_expert,
+                 (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim};
+    return launch(name, (out_dim + 127) / 128, tile_ub, 1, 256, 0, s, a);
+}
+
+int rein_swiglu_mul(const float* gate, const float* up, float* out, unsigned n, rein_stream_t s)
+{
+    if (n == 0) return fail(REIN_E_BAD_SHAPE, "rein_swiglu_mul: n is zero");
+    if (int rc = check_ptr("rein_swiglu_mul", gate, 4, "gate")) return rc;
+    if (int rc = check_ptr("rein_swiglu_mul", up, 4, "up")) return rc;
+    if (int rc = check_ptr("rein_swiglu_mul", out, 4, "out")) return rc;
+    unsigned g = (n + 255) / 256;
+    if (g > kCUs * 32) g = kCUs * 32;
+    void* a[] = {(void*)&gate, (void*)&up, (void*)&out, (void*)&n};
+    return launch("swiglu_mul_f32", g, 1, 1, 256, 0, s, a);
+}
+
+int rein_moe_combine(const float* experts, const int32_t* ids, const float* weights, const float* down_exps_s,
+                     float* out, unsigned n_tok, unsigned hidden, unsigned n_used, rein_stream_t s)
+{
+    if (n_tok == 0 || hidden == 0 || n_used == 0) return fail(REIN_E_BAD_SHAPE, "rein_moe_combine: zero dimension");
+    if (n_tok > 65535) return fail(REIN_E_TOO_LARGE, "rein_moe_combine: at most 65535 tokens per call");
+    const void* ptrs[] = {experts, ids, weights, down_exps_s, out};
+    for (const void* p : ptrs)
+        if (int rc = check_ptr("rein_moe_combine", p, 4, "buffer")) return rc;
+    void* a[] = {(void*)&experts, (void*)&ids, (void*)&weights, (void*)&down_exps_s, (void*)&out, (void*)&hidden, (void*)&n_used};
+    return launch("moe_combine_f32", (hidden + 255) / 256, n_tok, 1, 256, 0, s, a);
+}
+
+// Workspace carve-up for rein_moe_ffn (all offsets 256-byte aligned).
+namespace {
+struct MoeWs {
+    size_t ids, weights, count, cursor, perm, eoff, toff, xq_in, g_in, e_gate, e_up, xq_exp, g_out, e_out, total;
+};
+size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+MoeWs moe_ws(const rein_moe_shape& sh)
+{
+    const size_t ne = (size_t)sh.n_tok * sh.n_used;
+    MoeWs w;
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o += up256(bytes); return at; };
+    w.ids     = take(ne * 4);
+    w.weights = take(ne * 4);
+    w.count   = take((size_t)sh.n_expert * 4);
+    w.cursor  = take((size_t)sh.n_expert * 4);
+    w.perm    = take(ne * 4);
+    w.eoff    = take(((size_t)sh.n_expert + 1) * 4);
+    w.toff    = take(((size_t)sh.n_expert + 1) * 4);
+    w.xq_in   = take((size_t)sh.n_tok * (sh.hidden / 32) * 40);
+    w.g_in    = take(ne * (sh.hidden / 32) * 40);
+    w.e_gate  = take(ne * sh.expert_ff * 4);
+    w.e_up    = take(ne * sh.expert_ff * 4);
+    w.xq_exp  = take(ne * (sh.expert_ff / 32) * 40);
+    w.g_out   = take(ne * sh.hidden * 4);
+    w.e_out   = take(ne * sh.hidden * 4);
+    w.total   = o;
+    return w;
+}
+}  // namespace
+
+size_t rein_moe_workspace_bytes(const rein_moe_shape* sh)
+{
+    if (!sh) return 0;
+    return moe_ws(*sh).total;
+}
+
+int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits, const void* gate_exps,
+                 const void* up_exps, const void* down_exps, const float* down_exps_s, void* workspace,
+                 float* out, rein_stream_t s)
+{
+    const char* who = "rein_moe_ffn";
+    if (!shp) return fail(REIN_E_BAD_POINTER, std::string(who) + ": shape is NULL");
+    const rein_moe_shape sh = *shp;
+    if (sh.n_tok == 0 || sh.hidden == 0 || sh.n_expert == 0 || sh.n_used == 0 || sh.expert_ff == 0)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": zero dimension");
+    if (int rc = check_shape(who, sh.gate_up_fmt, sh.hidden, sh.expert_ff, sh.n_tok)) return rc;
+    if (int rc = check_shape(who, sh.down_fmt, sh.expert_ff, sh.hidden, sh.n_tok)) return rc;
+    if (int rc = check_ptr(who, workspace, 256, "workspace")) return rc;
+    const size_t bpe_gu = rein_repacked_len(sh.gate_up_fmt, sh.hidden, sh.expert_ff);
+    const size_t bpe_dn = rein_repacked_len(sh.down_fmt, sh.expert_ff, sh.hidden);
+    if (bpe_gu > 0xFFFFFFFFull || bpe_dn > 0xFFFFFFFFull)
+        return fail(REIN_E_TOO_LARGE, std::string(who) + ": an expert slab must stay below 4 GiB");   // u32, qwen35.rs:3052
+
+    const MoeWs w = moe_ws(sh);
+    char* base = static_cast<char*>(workspace);
+    int32_t* ids = (int32_t*)(base + w.ids);
+    float* weights = (float*)(base + w.weights);
+    int32_t* perm = (int32_t*)(base + w.perm);
+    int32_t* eoff = (int32_t*)(base + w.eoff);
+    int32_t* toff = (int32_t*)(base + w.toff);
+    const unsigned ne = sh.n_tok * sh.n_used;
+
+    if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
+    if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
+    if (int rc = rein_moe_sort(ids, ne, sh.n_expert, rein_moe_gemm_bn(), (int32_t*)(base + w.count),
+                               (int32_t*)(base + w.cursor), perm, eoff, toff, s)) return rc;
+    if (int rc = rein_moe_gather_xq(base + w.xq_in, perm, base + w.g_in, sh.hidden / 32, sh.n_used, ne, s)) return rc;
+    if (int rc = rein_moe_grouped_gemm(sh.gate_up_fmt, gate_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
+                                       base + w.g_in, (float*)(base + w.e_gate), sh.hidden, sh.expert_ff, ne, s)) return rc;
+    if (int rc = rein_moe_grouped_gemm(sh.gate_up_fmt, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
+                                       base + w.g_in, (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;
+    if (int rc = rein_swiglu_mul((float*)(base + w.e_gate), (float*)(base + w.e_up), (float*)(base + w.e_gate),
+                                 ne * sh.expert_ff, s)) return rc;
+    // the quantizer's grid.y carries the row count: split long batches
+    for (unsigned r0 = 0; r0 < ne; r0 += 32768) {
+        const unsigned nr = ne - r0 < 32768 ? ne - r0 : 32768;
+        if (int rc = rein_quantize_q8((float*)(base + w.e_gate) + (size_t)r0 * sh.expert_ff,
+                                      base + w.xq_exp + (size_t)r0 * (sh.expert_ff / 32) * 40, sh.expert_ff, nr, s)) return rc;
+    }
+    if (int rc = rein_moe_grouped_gemm(sh.down_fmt, down_exps, (unsigned)bpe_dn, eoff, toff, sh.n_expert,
+                                       base + w.xq_exp, (float*)(base + w.g_out), sh.expert_ff, sh.hidden, ne, s)) return rc;
+    if (int rc = rein_moe_scatter_rows((float*)(base + w.g_out), perm, (float*)(base + w.e_out), sh.hidden, ne, s)) return rc;
+    return rein_moe_combine((float*)(base + w.e_out), ids, weights, down_exps_s, out, sh.n_tok, sh.hidden, sh.n_used, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,14 @@
+// Prefill MMQ GEMM, repacked Q4K weights, on the int8 matrix cores.  Entry
+// points the reference host looks up by name (kernels/mmq_gemm_q4k_repacked.cpp):
+//   _f32         wide tile   (reference launch: grid (ceil(out/64), ceil(P/64)) x 256)
+//   _narrow_f32  <= 16 rows  (reference launch: grid (ceil(out/16), ceil(P/16)) x 64)
+// plus the tuned token-tile variants the C-ABI launcher picks from and the MFMA
+// block-dot dump used by the parity tests.
+#include "mmq_gemm.h"
+
+REIN_DEFINE_MMQ(mmq_gemm_q4k_repacked_f32, REIN_Q4_K, 64)
+REIN_DEFINE_MMQ(mmq_gemm_q4k_repacked_narrow_f32, REIN_Q4_K, 32)
+REIN_DEFINE_MMQ(rein_mmq_q4k_t32, REIN_Q4_K, 32)
+REIN_DEFINE_MMQ(rein_mmq_q4k_t64, REIN_Q4_K, 64)
+REIN_DEFINE_MMQ(rein_mmq_q4k_t128, REIN_Q4_K, 128)
+REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q4k, REIN_Q4_K)

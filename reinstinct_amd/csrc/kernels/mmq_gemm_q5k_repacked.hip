@@ -1,0 +1,14 @@
+// Prefill MMQ GEMM, repacked Q5K weights, on the int8 matrix cores.  Entry
+// points the reference host looks up by name (kernels/mmq_gemm_q5k_repacked.cpp):
+//   _f32         wide tile   (reference launch: grid (ceil(out/64), ceil(P/64)) x 256)
+//   _narrow_f32  <= 16 rows  (reference launch: grid (ceil(out/16), ceil(P/16)) x 64)
+// plus the tuned token-tile variants the C-ABI launcher picks from and the MFMA
+// block-dot dump used by the parity tests.
+#include "mmq_gemm.h"
+
+REIN_DEFINE_MMQ(mmq_gemm_q5k_repacked_f32, REIN_Q5_K, 64)
+REIN_DEFINE_MMQ(mmq_gemm_q5k_repacked_narrow_f32, REIN_Q5_K, 32)
+REIN_DEFINE_MMQ(rein_mmq_q5k_t32, REIN_Q5_K, 32)
+REIN_DEFINE_MMQ(rein_mmq_q5k_t64, REIN_Q5_K, 64)
+REIN_DEFINE_MMQ(rein_mmq_q5k_t128, REIN_Q5_K, 128)
+REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q5k, REIN_Q5_K)

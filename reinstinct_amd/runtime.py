@@ -1,0 +1,102 @@
+"""Launch sites of the path, as thin wrappers over the C ABI.  Arguments are
+device pointers (ints or DeviceBuf) exactly as the C functions take them."""
+import ctypes as C
+
+from ._lib import MoeShape, check, lib
+from .hip import DeviceBuf
+
+
+def _p(x):
+    if isinstance(x, DeviceBuf):
+        return x.ptr
+    return x
+
+
+def _s(stream):
+    return stream.raw if stream is not None else None
+
+
+def quantize_q8(x, xq, in_dim, n_vec=1, stream=None):
+    """launch_quantize_q8 (src/runtime/qwen35.rs:3202-3211)"""
+    check(lib.rein_quantize_q8(_p(x), _p(xq), in_dim, n_vec, _s(stream)))
+
+
+def matvec_xq8(fmt, w, xq, y, in_dim, out_dim, stream=None):
+    """launch_matvec_repacked_xq8 (src/runtime/qwen35.rs:2232-2280)"""
+    check(lib.rein_matvec_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, _s(stream)))
+
+
+def matvec_batched_xq8(fmt, w, xq, y, in_dim, out_dim, n_rows, stream=None):
+    """matmul_kquant_batched_into minus its quantize (src/runtime/prefill.rs:448-508)"""
+    check(lib.rein_matvec_batched_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, n_rows, _s(stream)))
+
+
+def mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, stream=None):
+    """matmul_mmq_into minus its quantize (src/runtime/prefill.rs:512-567)"""
+    check(lib.rein_mmq_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _s(stream)))
+
+
+def matmul(fmt, w, x, y, in_dim, out_dim, n_rows, xq_scratch, stream=None):
+    """PrefillGemm::matmul_into_raw (src/runtime/prefill.rs:343-384)"""
+    check(lib.rein_matmul(fmt, _p(w), _p(x), _p(y), in_dim, out_dim, n_rows, _p(xq_scratch), _s(stream)))
+
+
+def matmul_path(fmt, n_rows):
+    rc = lib.rein_matmul_path(fmt, n_rows)
+    if rc < 0:
+        check(rc)
+    return ("matvec", "batched_matvec", "mmq")[rc]
+
+
+def block_dots(fmt, w, xq, out, in_dim, out_dim, n_rows, via_mfma=False, stream=None):
+    check(lib.rein_block_dots(fmt, _p(w), _p(xq), _p(out), in_dim, out_dim, n_rows, int(via_mfma), _s(stream)))
+
+
+def moe_topk(logits, n_tok, n_expert, n_used, out_ids, out_weights, stream=None):
+    check(lib.rein_moe_topk(_p(logits), n_tok, n_expert, n_used, _p(out_ids), _p(out_weights), _s(stream)))
+
+
+def moe_sort(ids, n_entries, n_expert, bn, count, cursor, perm, expert_off, tile_off, stream=None):
+    check(lib.rein_moe_sort(_p(ids), n_entries, n_expert, bn, _p(count), _p(cursor), _p(perm),
+                            _p(expert_off), _p(tile_off), _s(stream)))
+
+
+def moe_gather_xq(xq_src, perm, xq_dst, nsub, n_used, n_entries, stream=None):
+    check(lib.rein_moe_gather_xq(_p(xq_src), _p(perm), _p(xq_dst), nsub, n_used, n_entries, _s(stream)))
+
+
+def moe_scatter_rows(src, perm, dst, dim, n_entries, stream=None):
+    check(lib.rein_moe_scatter_rows(_p(src), _p(perm), _p(dst), dim, n_entries, _s(stream)))
+
+
+def moe_grouped_gemm(fmt, slab, bytes_per_expert, expert_off, tile_off, n_expert, xq, y, in_dim, out_dim,
+                     n_entries, stream=None):
+    check(lib.rein_moe_grouped_gemm(fmt, _p(slab), bytes_per_expert, _p(expert_off), _p(tile_off), n_expert,
+                                    _p(xq), _p(y), in_dim, out_dim, n_entries, _s(stream)))
+
+
+def swiglu_mul(gate, up, out, n, stream=None):
+    check(lib.rein_swiglu_mul(_p(gate), _p(up), _p(out), n, _s(stream)))
+
+
+def moe_combine(experts, ids, weights, down_exps_s, out, n_tok, hidden, n_used, stream=None):
+    check(lib.rein_moe_combine(_p(experts), _p(ids), _p(weights), _p(down_exps_s), _p(out), n_tok, hidden,
+                               n_used, _s(stream)))
+
+
+def moe_gemm_bn():
+    return lib.rein_moe_gemm_bn()
+
+
+def moe_shape(n_tok, hidden, n_expert, n_used, expert_ff, gate_up_fmt, down_fmt):
+    return MoeShape(n_tok, hidden, n_expert, n_used, expert_ff, gate_up_fmt, down_fmt)
+
+
+def moe_workspace_bytes(shape):
+    return lib.rein_moe_workspace_bytes(C.byref(shape))
+
+
+def moe_ffn(shape, x, logits, gate_exps, up_exps, down_exps, down_exps_s, workspace, out, stream=None):
+    """routed-expert part of step_moe_ffn_batched (src/runtime/qwen35.rs:2788-2870)"""
+    check(lib.rein_moe_ffn(C.byref(shape), _p(x), _p(logits), _p(gate_exps), _p(up_exps), _p(down_exps),
+                           _p(down_exps_s), _p(workspace), _p(out), _s(stream)))

@@ -1,0 +1,134 @@
+"""CPU-side tests of the product's host code: the C ABI loads and exports every
+symbol include/rein.h declares, the src/quant mirror reproduces the oracle's
+repack byte for byte, the synthetic quantizers emit valid blocks, the dispatch
+thresholds and the error model.  No compute call is made (no GPU here)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import reinstinct_amd as rein
+from reinstinct_amd import _lib, quant, runtime
+from oracle import orc
+from helpers import random_raw_weights, rel_l2
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ALL = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS]
+
+
+def test_header_symbols_all_exported_and_typed():
+    text = open(os.path.join(ROOT, "include", "rein.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(rein_[a-z0-9_]+)\s*\(", text))
+    declared -= {"rein_moe_shape"}
+    assert len(declared) > 55
+    lib = _lib.load()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in rein.h but not exported by librein.so"
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+
+
+def test_format_ids_match_reference_enum():  # src/gguf/types.rs:16-35
+    assert (rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS) == (2, 8, 12, 13, 14, 23)
+    for fmt in ALL:
+        assert quant.block_size(fmt) == orc.block_size(fmt)
+        assert quant.bytes_per_block(fmt) == orc.bytes_per_block(fmt)
+    assert quant.block_size(99) == 0
+
+
+@pytest.mark.parametrize("fmt", ALL)
+@pytest.mark.parametrize("in_dim,out_dim", [(256, 1), (512, 3), (768, 5), (2048, 4), (5120, 2)])
+def test_repack_matches_oracle_bytes(fmt, in_dim, out_dim):
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt * 7 + in_dim)
+    got = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    want = orc.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    assert quant.repacked_len(fmt, in_dim, out_dim) == want.size
+    assert quant.repacked_n_sub_padded(in_dim) == orc.repacked_n_sub_padded(in_dim)
+    assert np.array_equal(got, want)
+
+
+def test_repack_threaded_path_matches_oracle():
+    fmt, in_dim, out_dim = rein.Q5_K, 4096, 1100       # above the threading threshold, ragged split
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=3)
+    assert np.array_equal(quant.repack_for_matvec(fmt, raw, in_dim, out_dim),
+                          orc.repack_for_matvec(fmt, raw, in_dim, out_dim))
+
+
+def test_repack_small_blocks_odd_counts():
+    for fmt in (rein.Q4_0, rein.Q8_0):
+        for in_dim in (32, 96, 128, 160):
+            raw = random_raw_weights(fmt, in_dim, 3, seed=in_dim)
+            assert np.array_equal(quant.repack_for_matvec(fmt, raw, in_dim, 3),
+                                  orc.repack_for_matvec(fmt, raw, in_dim, 3))
+
+
+def test_repack_errors():
+    raw = np.zeros(144, np.uint8)
+    with pytest.raises(rein.ReinError) as e:
+        quant.repack_for_matvec(rein.Q4_K, raw, 200, 1)        # the reference asserts (q4_k.rs:127)
+    assert e.value.code == -3 and "multiple of 256" in str(e.value)
+    with pytest.raises(rein.ReinError) as e:
+        quant.repack_for_matvec(99, raw, 256, 1)
+    assert e.value.code == -2
+
+
+@pytest.mark.parametrize("fmt,tol", [(rein.Q8_0, 6e-3), (rein.Q6_K, 2e-2), (rein.Q5_K, 4e-2), (rein.Q4_K, 8e-2),
+                                     (rein.Q4_0, 1.2e-1), (rein.IQ4_XS, 1.2e-1)])
+def test_quantize_weights_valid_and_close(fmt, tol):
+    rng = np.random.default_rng(fmt)
+    w = (rng.standard_normal((16, 1024)) * 0.02).astype(np.float32)
+    raw = quant.quantize_weights(fmt, w)
+    assert raw.size == w.size // quant.block_size(fmt) * quant.bytes_per_block(fmt)
+    deq = orc.dequantize_to_f32(fmt, raw, w.size).reshape(w.shape)
+    assert np.all(np.isfinite(deq))
+    assert rel_l2(deq, w) < tol
+    # all-zero input stays zero and finite
+    z = quant.quantize_weights(fmt, np.zeros(512, np.float32))
+    assert np.all(orc.dequantize_to_f32(fmt, z, 512) == 0)
+
+
+def test_quantize_weights_q8_0_matches_reference_quantizer():
+    w = (np.random.default_rng(0).standard_normal(4096) * 0.02).astype(np.float32)
+    assert np.array_equal(quant.quantize_weights(rein.Q8_0, w), orc.q8_0_quantize_from_f32(w))
+
+
+def test_matmul_dispatch_thresholds():
+    # 1 row -> matvec; 2..8 -> weight-streaming batched matvec (the reference
+    # switches to its narrow MMQ at 5, prefill.rs:358,383); above -> MMQ.
+    # Row counts are the reference's own sweep (prefill.rs:579-682).
+    want = {1: "matvec", 4: "batched_matvec", 5: "batched_matvec", 8: "batched_matvec",
+            15: "mmq", 16: "mmq", 20: "mmq"}
+    for fmt in ALL:
+        for n, path in want.items():
+            assert runtime.matmul_path(fmt, n) == path
+    with pytest.raises(rein.ReinError):
+        runtime.matmul_path(99, 1)
+    with pytest.raises(rein.ReinError):
+        runtime.matmul_path(rein.Q4_K, 0)
+
+
+def test_compute_calls_fail_loudly_without_runtime():
+    lib = _lib.load()
+    if lib.rein_is_loaded():
+        pytest.skip("a GPU runtime is loaded in this process")
+    rc = lib.rein_matvec_xq8(rein.Q4_K, 16, 16, 16, 256, 8, None)
+    assert rc == -1 and b"no CPU fallback" in lib.rein_last_error()
+    # argument errors are reported before anything touches the device
+    assert lib.rein_matvec_xq8(rein.Q4_K, 16, 16, 16, 200, 8, None) == -3
+    assert lib.rein_matvec_xq8(99, 16, 16, 16, 256, 8, None) == -2
+    assert lib.rein_matvec_xq8(rein.Q4_K, 8, 16, 16, 256, 8, None) == -4 and b"16-byte aligned" in lib.rein_last_error()
+    assert lib.rein_matvec_batched_xq8(rein.Q4_K, 16, 16, 16, 256, 8, 9, None) == -6
+    assert lib.rein_quantize_q8(16, 16, 48, 1, None) == -3
+    assert lib.rein_moe_grouped_gemm(rein.Q4_0, 16, 16, 16, 16, 1, 16, 16, 256, 8, 1, None) == -2
+
+
+def test_moe_workspace_layout():
+    sh = runtime.moe_shape(512, 2048, 128, 8, 768, rein.Q4_K, rein.Q6_K)
+    n = runtime.moe_workspace_bytes(sh)
+    ne = 512 * 8
+    need = ne * 4 * 3 + 128 * 4 * 2 + 129 * 4 * 2 + 512 * 64 * 40 + ne * 64 * 40 + ne * 768 * 4 * 2 + ne * 24 * 40 \
+        + ne * 2048 * 4 * 2
+    assert need <= n <= need + 14 * 256
+    assert runtime.moe_gemm_bn() == 32
