@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+
+Headline workload (BASELINE.json configs[1], first shape): Q4_K repacked-v2 decode
+matvec, batch 1, K=5120 -> N=5120, weights ~N(0,0.02) quantized to Q4_K, activation
+~N(0,1) quantized to BlockQ8.  One *step* is one pass of the matvec over a rotation
+of distinct weight buffers (together larger than L2 + Infinity Cache, so every
+launch streams its weights from HBM), captured in a hipGraph.  Everything is
+resident in HBM before the timed region.  Prints ONE JSON line.
+
+The same line carries the MMQ prefill GEMM (Q4_K, 512 x 5120 x 17408) in "mmq",
+the roofline object of the dominant kernel and the CPU baseline (the oracle's
+restatement of the reference CPU path: dequantize once, then the f32 matvec of
+src/cpu/ops.rs:108-140 over all host cores) timed on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import reinstinct_amd as rein  # noqa: E402
+from reinstinct_amd import hip, quant, runtime  # noqa: E402
+from reinstinct_amd._lib import init  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
+CACHE_BYTES = 512 << 20        # rotate over more than L2 (32 MB) + Infinity Cache (256 MB)
+
+FMT_NAME = {rein.Q4_0: "q4_0", rein.Q4_K: "q4_k", rein.Q5_K: "q5_k", rein.Q6_K: "q6_k", rein.Q8_0: "q8_0",
+            rein.IQ4_XS: "iq4_xs"}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def synth_weights(fmt, in_dim, out_dim, seed):
+    """fp32 ~N(0,0.02) -> on-disk blocks -> repacked-v2 slab (host)."""
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((out_dim, in_dim), dtype=np.float32) * np.float32(0.02))
+    raw = quant.quantize_weights(fmt, w)
+    return raw, quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+
+
+def matvec_bytes(fmt, in_dim, out_dim, batch):
+    """algorithmic bytes of one launch: weights + BlockQ8 activations + fp32 outputs"""
+    return quant.repacked_len(fmt, in_dim, out_dim) + batch * (in_dim // 32) * 40 + batch * out_dim * 4
+
+
+class MatvecCase:
+    """A rotation of weight buffers and a captured graph of one pass over them."""
+
+    def __init__(self, fmt, in_dim, out_dim, batch, stream, seed=0, min_bytes=CACHE_BYTES, packed=None):
+        self.fmt, self.in_dim, self.out_dim, self.batch, self.stream = fmt, in_dim, out_dim, batch, stream
+        if packed is None:
+            _, packed = synth_weights(fmt, in_dim, out_dim, seed)
+        self.packed = packed
+        self.n_buf = max(2, -(-min_bytes // packed.nbytes))
+        first = hip.DeviceBuf.from_host(packed)
+        self.weights = [first]
+        for _ in range(self.n_buf - 1):
+            b = hip.DeviceBuf(packed.nbytes)
+            rein.lib.rein_memcpy_d2d(b.ptr, first.ptr, packed.nbytes)
+            self.weights.append(b)
+        x = np.random.default_rng(seed + 1).standard_normal((batch, in_dim)).astype(np.float32)
+        self.x = x
+        self.dx = hip.DeviceBuf.from_host(x)
+        self.dq = hip.DeviceBuf(batch * (in_dim // 32) * 40)
+        self.dy = hip.DeviceBuf(batch * out_dim * 4)
+        runtime.quantize_q8(self.dx, self.dq, in_dim, batch, stream)
+        stream.synchronize()
+        self.bytes_per_launch = matvec_bytes(fmt, in_dim, out_dim, batch)
+        stream.begin_capture()
+        for wbuf in self.weights:
+            self.launch(wbuf)
+        self.graph = stream.end_capture()
+        self.exe = self.graph.instantiate()
+
+    def launch(self, wbuf):
+        if self.batch == 1:
+            runtime.matvec_xq8(self.fmt, wbuf, self.dq, self.dy, self.in_dim, self.out_dim, self.stream)
+        else:
+            runtime.matvec_batched_xq8(self.fmt, wbuf, self.dq, self.dy, self.in_dim, self.out_dim, self.batch,
+                                       self.stream)
+
+    def step(self):
+        self.exe.launch(self.stream)
+
+    def time(self, steps, warmup):
+        """-> (seconds per step, seconds per launch), events on the launch stream"""
+        for _ in range(warmup):
+            self.step()
+        self.stream.synchronize()
+        e0, e1 = hip.Event(), hip.Event()
+        e0.record(self.stream)
+        for _ in range(steps):
+            self.step()
+        e1.record(self.stream)
+        e1.synchronize()
+        sec = e0.elapsed_ms(e1) * 1e-3
+        return sec / steps, sec / (steps * self.n_buf)
+
+
+class MmqCase:
+    def __init__(self, fmt, p_rows, in_dim, out_dim, stream, seed=0):
+        self.fmt, self.p, self.in_dim, self.out_dim, self.stream = fmt, p_rows, in_dim, out_dim, stream
+        _, packed = synth_weights(fmt, in_dim, out_dim, seed)
+        self.n_buf = 4                                  # 4 x 89 MB of weights > Infinity Cache
+        self.weights = [hip.DeviceBuf.from_host(packed)]
+        for _ in range(self.n_buf - 1):
+            b = hip.DeviceBuf(packed.nbytes)
+            rein.lib.rein_memcpy_d2d(b.ptr, self.weights[0].ptr, packed.nbytes)
+            self.weights.append(b)
+        x = np.random.default_rng(seed + 1).standard_normal((p_rows, in_dim)).astype(np.float32)
+        self.dx = hip.DeviceBuf.from_host(x)
+        self.dq = hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
+        self.dy = hip.DeviceBuf(p_rows * out_dim * 4)
+        runtime.quantize_q8(self.dx, self.dq, in_dim, p_rows, stream)
+        stream.synchronize()
+        self.ops = 2.0 * p_rows * in_dim * out_dim      # reference convention, kernels.rs:2917
+
+    def time(self, launches, warmup):
+        for i in range(warmup):
+            runtime.mmq_xq8(self.fmt, self.weights[i % self.n_buf], self.dq, self.dy, self.in_dim, self.out_dim,
+                            self.p, self.stream)
+        self.stream.synchronize()
+        e0, e1 = hip.Event(), hip.Event()
+        e0.record(self.stream)
+        for i in range(launches):
+            runtime.mmq_xq8(self.fmt, self.weights[i % self.n_buf], self.dq, self.dy, self.in_dim, self.out_dim,
+                            self.p, self.stream)
+        e1.record(self.stream)
+        e1.synchronize()
+        return e0.elapsed_ms(e1) * 1e-3 / launches
+
+
+def cpu_baseline(fmt, in_dim, out_dim, seed, budget_s=12.0):
+    """The reference CPU path (dequantize once, untimed; then f32 matvec over all
+    cores) on the headline shape, repeated for about `budget_s` seconds."""
+    from oracle import orc          # the checker, used here only as the timed CPU baseline
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else int(os.environ["OMP_NUM_THREADS"])
+    raw, _ = synth_weights(fmt, in_dim, out_dim, seed)
+    w = orc.dequantize_to_f32(fmt, raw, in_dim * out_dim).reshape(out_dim, in_dim)
+    x = np.random.default_rng(seed + 1).standard_normal(in_dim).astype(np.float32)
+    orc.matvec_f32(x, w, n_threads=cores)
+    best, reps, t_start = 1e30, 0, time.perf_counter()
+    while time.perf_counter() - t_start < budget_s and reps < 2000:
+        t0 = time.perf_counter()
+        orc.matvec_f32(x, w, n_threads=cores)
+        best = min(best, time.perf_counter() - t0)
+        reps += 1
+    return {"value": round(matvec_bytes(fmt, in_dim, out_dim, 1) / best / 1e9, 3), "unit": "GB/s",
+            "cores": cores, "kind": "port",
+            "sample": f"dequantize_to_f32 once (untimed) + f32 matvec {in_dim}->{out_dim}, best of {reps} runs, "
+                      f"algorithmic (repacked) bytes / time; {round(in_dim * out_dim * 4 / best / 1e9, 2)} GB/s of f32 traffic"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--sweep", action="store_true", help="also time the format x shape x batch sweep of configs[1]")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-mmq", action="store_true")
+    ap.add_argument("--fmt", default="q4_k")
+    ap.add_argument("--shape", default="5120x5120", help="KxN of the headline matvec")
+    ap.add_argument("--batch", type=int, default=1)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path has no collectives",
+              file=sys.stderr)
+        sys.exit(2)
+
+    init()
+    hip.set_device(0)
+    stream = hip.Stream()
+    fmt = rein.FORMATS[args.fmt]
+    in_dim, out_dim = (int(v) for v in args.shape.lower().split("x"))
+
+    case = MatvecCase(fmt, in_dim, out_dim, args.batch, stream, seed=1234)
+    sec_step, sec_launch = case.time(args.steps, args.warmup)
+    gbs = case.bytes_per_launch / sec_launch / 1e9
+    log(f"matvec {args.fmt} {in_dim}->{out_dim} b{args.batch}: {sec_launch * 1e6:.2f} us/launch, {gbs:.0f} GB/s "
+        f"({case.n_buf} buffers/step)")
+
+    out = {
+        "metric": "Q4_K decode matvec HBM GB/s (% of peak) + MMQ pp512 int8 TOPS, 1 MI355X",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec_step * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 dot4 / fp32 accumulate", "data": "synthetic",
+        "config": {"workload": f"{args.fmt} repacked-v2 decode matvec K={in_dim} N={out_dim} batch={args.batch} "
+                               f"(BASELINE configs[1]); step = one pass over {case.n_buf} distinct weight buffers",
+                   "launches_per_step": case.n_buf, "bytes_per_launch": case.bytes_per_launch,
+                   "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": f"rein_mv_{'q4k' if fmt == rein.Q4_K else args.fmt}", "us_per_launch": round(sec_launch * 1e6, 3)},
+    }
+
+    if not args.no_mmq:
+        mm = MmqCase(rein.Q4_K, 512, 5120, 17408, stream, seed=77)
+        sec = mm.time(max(4, min(args.steps, 20)), 2)
+        tops = mm.ops / sec / 1e12
+        log(f"mmq q4_k 512x5120x17408: {sec * 1e6:.1f} us, {tops:.1f} TOPS")
+        out["mmq"] = {"workload": "Q4_K MMQ prefill GEMM 512x5120x17408 (BASELINE configs[2])",
+                      "us_per_launch": round(sec * 1e6, 2), "value": round(tops, 2), "unit": "int8 TOPS",
+                      "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+
+    if args.sweep:
+        sweep = []
+        for f in (rein.Q4_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.IQ4_XS):
+            for (k, n) in ((5120, 5120), (5120, 34816), (17408, 5120)):
+                _, packed = synth_weights(f, k, n, seed=5)
+                for b in (1, 2, 4, 8):
+                    c = MatvecCase(f, k, n, b, stream, seed=5, packed=packed)
+                    _, sl = c.time(max(3, args.steps // 4), 1)
+                    g = c.bytes_per_launch / sl / 1e9
+                    sweep.append({"fmt": FMT_NAME[f], "K": k, "N": n, "batch": b, "us": round(sl * 1e6, 2),
+                                  "GBs": round(g, 0), "frac": round(g / HBM_PEAK_GBS, 3)})
+                    log(sweep[-1])
+                    del c
+        out["sweep"] = sweep
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(fmt, in_dim, out_dim, seed=1234)
+        log("cpu baseline:", out["cpu_baseline"])
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,409 @@
+"""GPU parity tests: every kernel of the path, through the C ABI, against the
+CPU oracle on the same seeded inputs.
+
+Bars: quantize_q8 bytes and per-block int32 dots bit-exact; fp32 outputs within
+1e-3 relative / 1e-4 absolute of the oracle's int8 path, and within the
+reference's own rel_l2 < 1.5e-2 (src/runtime/kernels.rs:1598-1601) of its
+dequantize -> f32 matvec CPU path.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import reinstinct_amd as rein
+from reinstinct_amd import hip, quant, runtime
+from reinstinct_amd._lib import init
+from oracle import orc
+from helpers import Lcg, assert_close_f32, random_raw_weights, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+ALL = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS]
+NAME = {rein.Q4_0: "q4_0", rein.Q8_0: "q8_0", rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k",
+        rein.IQ4_XS: "iq4xs"}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def gpu():
+    init()                      # raises if librein / the code object / the GPU is missing
+    hip.set_device(0)
+    print("device:", hip.device_name(0), flush=True)
+    yield
+    hip.synchronize()
+
+
+def dev(a):
+    return hip.DeviceBuf.from_host(a)
+
+
+def make_weights(fmt, in_dim, out_dim, seed, gaussian=False):
+    if gaussian:
+        w = (np.random.default_rng(seed).standard_normal((out_dim, in_dim)) * 0.02).astype(np.float32)
+        raw = quant.quantize_weights(fmt, w)
+    else:
+        raw = random_raw_weights(fmt, in_dim, out_dim, seed)
+    return raw, quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+
+
+def gpu_quantize(x):
+    n_vec, k = x.shape
+    dx, dq = dev(x), hip.DeviceBuf(n_vec * (k // 32) * 40)
+    runtime.quantize_q8(dx, dq, k, n_vec)
+    hip.synchronize()
+    return dq
+
+
+# ------------------------------------------------------------------ quantize_q8
+@pytest.mark.parametrize("n_vec,k", [(1, 4096), (3, 5120), (8, 17408), (1, 32), (5, 96)])
+def test_quantize_q8_bit_exact(n_vec, k):
+    rng = np.random.default_rng(k + n_vec)
+    x = (rng.standard_normal((n_vec, k)) * rng.uniform(0.01, 50, (n_vec, 1))).astype(np.float32)
+    got = gpu_quantize(x).to_host(np.uint8)
+    assert np.array_equal(got, orc.quantize_q8(x))
+
+
+def test_quantize_q8_edge_blocks_bit_exact():
+    x = np.zeros((2, 256), np.float32)
+    x[0, 32:64] = 1e-30                      # tiny but normal
+    x[0, 64 + 3] = 3.0e38                    # near the top of the range
+    x[0, 96:128] = np.linspace(-127, 127, 32)
+    x[0, 128:160] = 0.5                      # all equal: every quant 127
+    x[1, :] = np.random.default_rng(1).standard_normal(256) * 1e-3
+    x[1, 7] = -4.0
+    got = gpu_quantize(x).to_host(np.uint8)
+    assert np.array_equal(got, orc.quantize_q8(x))
+
+
+def test_quantize_q8_reference_launch_geometry():
+    # grid (ceil(in_dim/256), n_vec) x 256, as qwen35.rs:3202-3211 launches it
+    x = np.random.default_rng(9).standard_normal((4, 5120)).astype(np.float32)
+    dx, dq = dev(x), hip.DeviceBuf(4 * 160 * 40)
+    f = hip.Module.builtin().function("quantize_q8_f32")
+    f.launch((20, 4, 1), (256, 1, 1), 0, None, [C.c_void_p(dx.ptr), C.c_void_p(dq.ptr), C.c_uint(5120)])
+    hip.synchronize()
+    assert np.array_equal(dq.to_host(np.uint8), orc.quantize_q8(x))
+
+
+# ------------------------------------------------------------------ decode matvec
+def check_matvec_outputs(fmt, raw, packed, xq_host, in_dim, out_dim, y, n_rows, x=None):
+    want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq_host, n_rows)
+    assert_close_f32(y, want, what=f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}")
+    if x is not None:
+        w = orc.dequantize_to_f32(fmt, raw, in_dim * out_dim).reshape(out_dim, in_dim)
+        for t in range(n_rows):
+            assert rel_l2(y[t], orc.matvec_f32(x[t], w)) < 1.5e-2
+
+
+SHAPES = [(2048, 384), (4096, 37), (768, 130), (5120, 64)]
+
+
+@pytest.mark.parametrize("fmt", ALL)
+@pytest.mark.parametrize("in_dim,out_dim", SHAPES)
+def test_matvec_parity(fmt, in_dim, out_dim):
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=fmt + in_dim)
+    x = Lcg(0x13579BDF + fmt).acts(in_dim)[None, :]
+    dq = gpu_quantize(x)
+    xq_host = dq.to_host(np.uint8)
+    assert np.array_equal(xq_host, orc.quantize_q8(x))
+    dw, dy = dev(packed), hip.DeviceBuf(out_dim * 4)
+    runtime.matvec_xq8(fmt, dw, dq, dy, in_dim, out_dim)
+    hip.synchronize()
+    y = dy.to_host(np.float32)[None, :]
+    check_matvec_outputs(fmt, raw, packed, xq_host, in_dim, out_dim, y, 1, x)
+    # per-block int32 dots, bit-exact, from the v_dot4 path and from the MFMA path
+    parts = orc.block_dots(fmt, packed, in_dim, out_dim, xq_host, 1)
+    for via_mfma in (False, True):
+        dd = hip.DeviceBuf(parts.nbytes)
+        runtime.block_dots(fmt, dw, dq, dd, in_dim, out_dim, 1, via_mfma)
+        hip.synchronize()
+        got = dd.to_host(np.int32).reshape(parts.shape)
+        assert np.array_equal(got, parts), f"block dots differ (via_mfma={via_mfma})"
+
+
+@pytest.mark.parametrize("fmt", ALL)
+def test_matvec_gaussian_weights_config1_shape(fmt):
+    # BASELINE config 1: 4096x4096 ~N(0,0.02) quantized, x ~N(0,1) (pad path nsp = 129);
+    # a 256-row slice of it keeps the CPU side quick
+    in_dim, out_dim = 4096, 256
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=100 + fmt, gaussian=True)
+    x = np.random.default_rng(5).standard_normal((1, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    dw, dy = dev(packed), hip.DeviceBuf(out_dim * 4)
+    runtime.matvec_xq8(fmt, dw, dq, dy, in_dim, out_dim)
+    hip.synchronize()
+    check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim,
+                         dy.to_host(np.float32)[None, :], 1, x)
+
+
+REF_MATVEC = [  # (kernel symbol, rows per workgroup, threads) exactly as qwen35.rs:2232-2280 launches them
+    ("matvec_{}_repacked_f32", 8, 256), ("matvec_{}_repacked_r1_f32", 4, 256), ("matvec_{}_repacked_r4_f32", 16, 256)]
+
+
+@pytest.mark.parametrize("fmt", ALL)
+def test_matvec_reference_symbols_and_geometry(fmt):
+    in_dim, out_dim = 2048, 389
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=31 + fmt)
+    x = Lcg(0x2468ACE0 + fmt).acts(in_dim)[None, :]
+    dq = gpu_quantize(x)
+    want = orc.matvec_q8(fmt, packed, in_dim, out_dim, dq.to_host(np.uint8), 1)
+    dw = dev(packed)
+    mod = hip.Module.builtin()
+    if fmt == rein.Q8_0:   # 64-thread workgroups, 2 rows (1 for _r1) per workgroup
+        launches = [("matvec_q8_0_repacked_f32", 2, 64), ("matvec_q8_0_repacked_r1_f32", 1, 64)]
+    elif fmt in (rein.Q5_K, rein.Q6_K):
+        launches = [(REF_MATVEC[0][0].format(NAME[fmt]), 8, 256)]
+    else:
+        launches = [(n.format(NAME[fmt]), r, t) for n, r, t in REF_MATVEC]
+    for name, rows, threads in launches:
+        dy = dev(np.full(out_dim, np.nan, np.float32))
+        mod.function(name).launch(((out_dim + rows - 1) // rows, 1, 1), (threads, 1, 1), 0, None,
+                                  [C.c_void_p(dw.ptr), C.c_void_p(dq.ptr), C.c_void_p(dy.ptr),
+                                   C.c_uint(in_dim), C.c_uint(out_dim)])
+        hip.synchronize()
+        assert_close_f32(dy.to_host(np.float32)[None, :], want, what=name)
+
+
+@pytest.mark.parametrize("fmt", ALL)
+@pytest.mark.parametrize("n_rows", [1, 2, 3, 4, 5, 8])
+def test_batched_matvec_parity(fmt, n_rows):
+    in_dim, out_dim = 1024, 203
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=57 + fmt)
+    x = np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    dw, dy = dev(packed), hip.DeviceBuf(n_rows * out_dim * 4)
+    runtime.matvec_batched_xq8(fmt, dw, dq, dy, in_dim, out_dim, n_rows)
+    hip.synchronize()
+    y = dy.to_host(np.float32).reshape(n_rows, out_dim)
+    check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim, y, n_rows, x)
+
+
+@pytest.mark.parametrize("fmt", ALL)
+def test_batched_reference_symbols(fmt):
+    # matvec_<fmt>_repacked_batched{,16}_f32 under the reference launch (prefill.rs:461-506)
+    in_dim, out_dim = 1024, 77
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=77 + fmt)
+    mod = hip.Module.builtin()
+    dw = dev(packed)
+    for name, rows_per_wg, n_rows in [("matvec_{}_repacked_batched_f32", 8, 4),
+                                      ("matvec_{}_repacked_batched_f32", 8, 3),
+                                      ("matvec_{}_repacked_batched16_f32", 4, 16),
+                                      ("matvec_{}_repacked_batched16_f32", 4, 9)]:
+        x = np.random.default_rng(n_rows + 40).standard_normal((n_rows, in_dim)).astype(np.float32)
+        dq = gpu_quantize(x)
+        dy = dev(np.full(n_rows * out_dim, np.nan, np.float32))
+        mod.function(name.format(NAME[fmt])).launch(
+            ((out_dim + rows_per_wg - 1) // rows_per_wg, 1, 1), (256, 1, 1), 0, None,
+            [C.c_void_p(dw.ptr), C.c_void_p(dq.ptr), C.c_void_p(dy.ptr), C.c_uint(in_dim), C.c_uint(out_dim),
+             C.c_uint(n_rows)])
+        hip.synchronize()
+        want = orc.matvec_q8(fmt, packed, in_dim, out_dim, dq.to_host(np.uint8), n_rows)
+        assert_close_f32(dy.to_host(np.float32).reshape(n_rows, out_dim), want, what=name)
+
+
+# ------------------------------------------------------------------ MMQ / matmul dispatch
+@pytest.mark.parametrize("fmt", ALL)
+@pytest.mark.parametrize("p_rows", [70, 24, 1, 129])
+def test_mmq_parity(fmt, p_rows):
+    # P = 70 exercises the token tail as the reference test does (kernels.rs:3176-3178)
+    in_dim, out_dim = 1024, 200
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=0x9494 + fmt)
+    x = Lcg(0x2468ACE0).acts(p_rows * in_dim).reshape(p_rows, in_dim)
+    dq = gpu_quantize(x)
+    xq_host = dq.to_host(np.uint8)
+    dw = dev(packed)
+    dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    runtime.mmq_xq8(fmt, dw, dq, dy, in_dim, out_dim, p_rows)
+    hip.synchronize()
+    y = dy.to_host(np.float32).reshape(p_rows, out_dim)
+    check_matvec_outputs(fmt, raw, packed, xq_host, in_dim, out_dim, y, p_rows, x)
+    parts = orc.block_dots(fmt, packed, in_dim, out_dim, xq_host, p_rows)
+    dd = hip.DeviceBuf(parts.nbytes)
+    runtime.block_dots(fmt, dw, dq, dd, in_dim, out_dim, p_rows, True)
+    hip.synchronize()
+    assert np.array_equal(dd.to_host(np.int32).reshape(parts.shape), parts)
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])
+def test_mmq_odd_sub_block_count(fmt):
+    in_dim, out_dim, p_rows = 32 * 11, 50, 40          # 11 sub-blocks: ragged last chunk and pair
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=5)
+    x = np.random.default_rng(8).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    runtime.mmq_xq8(fmt, dev(packed), dq, dy, in_dim, out_dim, p_rows)
+    hip.synchronize()
+    check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim,
+                         dy.to_host(np.float32).reshape(p_rows, out_dim), p_rows, x)
+
+
+@pytest.mark.parametrize("fmt", ALL)
+def test_mmq_reference_symbols_and_geometry(fmt):
+    in_dim, out_dim = 512, 150
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=3 + fmt)
+    mod = hip.Module.builtin()
+    dw = dev(packed)
+    for name, tile, threads, p_rows in [("mmq_gemm_{}_repacked_f32", 64, 256, 70),
+                                        ("mmq_gemm_{}_repacked_narrow_f32", 16, 64, 16),
+                                        ("mmq_gemm_{}_repacked_narrow_f32", 16, 64, 5)]:
+        x = np.random.default_rng(p_rows).standard_normal((p_rows, in_dim)).astype(np.float32)
+        dq = gpu_quantize(x)
+        dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+        mod.function(name.format(NAME[fmt])).launch(
+            ((out_dim + tile - 1) // tile, (p_rows + tile - 1) // tile, 1), (threads, 1, 1), 0, None,
+            [C.c_void_p(dw.ptr), C.c_void_p(dq.ptr), C.c_void_p(dy.ptr), C.c_uint(in_dim), C.c_uint(out_dim),
+             C.c_uint(p_rows)])
+        hip.synchronize()
+        want = orc.matvec_q8(fmt, packed, in_dim, out_dim, dq.to_host(np.uint8), p_rows)
+        assert_close_f32(dy.to_host(np.float32).reshape(p_rows, out_dim), want, what=name)
+
+
+@pytest.mark.parametrize("fmt", ALL)
+@pytest.mark.parametrize("n_rows", [1, 4, 5, 8, 15, 16, 20])
+def test_matmul_dispatch_row_sweep(fmt, n_rows):
+    # the reference's row-count sweep over every dtype (prefill.rs:579-682)
+    in_dim, out_dim = 512, 96
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=11 + fmt)
+    x = np.random.default_rng(n_rows * 3).standard_normal((n_rows, in_dim)).astype(np.float32)
+    dxq = hip.DeviceBuf(n_rows * (in_dim // 32) * 40)
+    dy = dev(np.full(n_rows * out_dim, np.nan, np.float32))
+    runtime.matmul(fmt, dev(packed), dev(x), dy, in_dim, out_dim, n_rows, dxq)
+    hip.synchronize()
+    xq_host = dxq.to_host(np.uint8)
+    assert np.array_equal(xq_host, orc.quantize_q8(x))
+    check_matvec_outputs(fmt, raw, packed, xq_host, in_dim, out_dim,
+                         dy.to_host(np.float32).reshape(n_rows, out_dim), n_rows, x)
+
+
+# ------------------------------------------------------------------ MoE
+def test_moe_topk_parity():
+    rng = np.random.default_rng(0)
+    for n_tok, n_expert, n_used in [(64, 128, 8), (5, 200, 4), (3, 16, 2)]:
+        logits = rng.standard_normal((n_tok, n_expert)).astype(np.float32)
+        d_ids, d_w = hip.DeviceBuf(n_tok * n_used * 4), hip.DeviceBuf(n_tok * n_used * 4)
+        runtime.moe_topk(dev(logits), n_tok, n_expert, n_used, d_ids, d_w)
+        hip.synchronize()
+        ids, w = orc.moe_topk(logits, n_used)
+        assert np.array_equal(d_ids.to_host(np.int32).reshape(ids.shape), ids)
+        assert np.allclose(d_w.to_host(np.float32).reshape(w.shape), w, rtol=1e-5, atol=1e-7)
+    # ties resolve through the same halving tree on both sides
+    logits = np.zeros((2, 128), np.float32)
+    d_ids, d_w = hip.DeviceBuf(2 * 8 * 4), hip.DeviceBuf(2 * 8 * 4)
+    runtime.moe_topk(dev(logits), 2, 128, 8, d_ids, d_w)
+    hip.synchronize()
+    ids, w = orc.moe_topk(logits, 8)
+    assert np.array_equal(d_ids.to_host(np.int32).reshape(ids.shape), ids)
+
+
+def gpu_sort(ids, n_expert, bn):
+    n = ids.size
+    bufs = [hip.DeviceBuf(n_expert * 4), hip.DeviceBuf(n_expert * 4), dev(np.full(n, -1, np.int32)),
+            hip.DeviceBuf((n_expert + 1) * 4), hip.DeviceBuf((n_expert + 1) * 4)]
+    runtime.moe_sort(dev(ids), n, n_expert, bn, *bufs)
+    hip.synchronize()
+    return bufs[2], bufs[3], bufs[4]
+
+
+def test_moe_sort_invariants():
+    rng = np.random.default_rng(1)
+    for n_tok, n_used, n_expert, bn in [(512, 8, 128, 32), (7, 2, 200, 16), (300, 4, 3, 32)]:
+        ids = rng.integers(0, n_expert, (n_tok, n_used)).astype(np.int32)
+        if n_tok > 10:
+            ids[0, 0], ids[3, 1] = -1, n_expert      # dropped (moe_expert_sort.cpp:38-40,71)
+        d_perm, d_eoff, d_toff = gpu_sort(ids, n_expert, bn)
+        perm, eoff, toff = d_perm.to_host(np.int32), d_eoff.to_host(np.int32), d_toff.to_host(np.int32)
+        _, want_eoff, want_toff = orc.moe_sort(ids, n_expert, bn)
+        assert np.array_equal(eoff, want_eoff) and np.array_equal(toff, want_toff)
+        flat = ids.ravel()
+        valid = perm[: eoff[-1]]
+        assert len(set(valid.tolist())) == valid.size and valid.min() >= 0 and valid.max() < flat.size
+        for e in range(n_expert):     # the order inside one expert is free (qwen35.rs:2956-2987)
+            assert np.all(flat[perm[eoff[e]: eoff[e + 1]]] == e)
+
+
+def test_moe_gather_scatter_swiglu_combine():
+    rng = np.random.default_rng(2)
+    n_tok, n_used, nsub, dim = 37, 8, 64, 300
+    n = n_tok * n_used
+    xq = rng.integers(0, 256, n_tok * nsub * 40, dtype=np.uint8)
+    perm = rng.permutation(n).astype(np.int32)
+    d_dst = hip.DeviceBuf(n * nsub * 40)
+    runtime.moe_gather_xq(dev(xq), dev(perm), d_dst, nsub, n_used, n)
+    rows = rng.standard_normal((n, dim)).astype(np.float32)
+    d_sc = hip.DeviceBuf(n * dim * 4)
+    runtime.moe_scatter_rows(dev(rows), dev(perm), d_sc, dim, n)
+    gate = (rng.standard_normal(5000) * 4).astype(np.float32)
+    up = rng.standard_normal(5000).astype(np.float32)
+    d_sw = hip.DeviceBuf(5000 * 4)
+    runtime.swiglu_mul(dev(gate), dev(up), d_sw, 5000)
+    experts = rng.standard_normal((n_tok, n_used, dim)).astype(np.float32)
+    ids = rng.integers(0, 16, (n_tok, n_used)).astype(np.int32)
+    w = rng.random((n_tok, n_used)).astype(np.float32)
+    s = rng.random(16).astype(np.float32)
+    d_out = hip.DeviceBuf(n_tok * dim * 4)
+    runtime.moe_combine(dev(experts), dev(ids), dev(w), dev(s), d_out, n_tok, dim, n_used)
+    hip.synchronize()
+    assert np.array_equal(d_dst.to_host(np.uint8), orc.moe_gather_xq(xq, perm, nsub, n_used))
+    assert np.array_equal(d_sc.to_host(np.float32).reshape(n, dim), orc.moe_scatter_rows(rows, perm, dim))
+    # __expf vs expf: the reference's own tolerance (kernels.rs:1468-1473)
+    assert np.allclose(d_sw.to_host(np.float32), orc.swiglu_mul(gate, up), rtol=1e-5, atol=1e-5)
+    assert np.array_equal(d_out.to_host(np.float32).reshape(n_tok, dim), orc.moe_combine(experts, ids, w, s))
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0])
+def test_grouped_gemm_parity(fmt):
+    in_dim, out_dim, n_expert, n_tok, n_used = 512, 136, 6, 40, 2
+    bpe = quant.repacked_len(fmt, in_dim, out_dim)
+    slabs = [make_weights(fmt, in_dim, out_dim, seed=200 + e)[1] for e in range(n_expert)]
+    slab = np.concatenate(slabs)
+    rng = np.random.default_rng(4)
+    ids = rng.integers(0, n_expert, (n_tok, n_used)).astype(np.int32)
+    ids[ids == 2] = 3                                   # expert 2 gets no tokens
+    d_perm, d_eoff, d_toff = gpu_sort(ids, n_expert, runtime.moe_gemm_bn())
+    perm, eoff = d_perm.to_host(np.int32), d_eoff.to_host(np.int32)
+    x = rng.standard_normal((n_tok, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    n = n_tok * n_used
+    d_gin = hip.DeviceBuf(n * (in_dim // 32) * 40)
+    runtime.moe_gather_xq(dq, d_perm, d_gin, in_dim // 32, n_used, n)
+    dy = dev(np.full(n * out_dim, np.nan, np.float32))
+    runtime.moe_grouped_gemm(fmt, dev(slab), bpe, d_eoff, d_toff, n_expert, d_gin, dy, in_dim, out_dim, n)
+    hip.synchronize()
+    gin = d_gin.to_host(np.uint8)
+    assert np.array_equal(gin, orc.moe_gather_xq(dq.to_host(np.uint8), perm, in_dim // 32, n_used))
+    want = orc.grouped_gemm(fmt, slab, bpe, eoff, gin, in_dim, out_dim)
+    assert_close_f32(dy.to_host(np.float32).reshape(n, out_dim), want, what=f"grouped fmt {fmt}")
+
+
+def test_moe_ffn_end_to_end_small():
+    # config 4 in miniature: top-k -> sort -> gather -> gate/up (Q4_K) -> SwiGLU ->
+    # quantize -> down (Q6_K) -> scatter -> combine, against the same chain on the CPU
+    n_tok, hidden, n_expert, n_used, ff = 48, 512, 16, 4, 256
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((n_tok, hidden)).astype(np.float32)
+    logits = rng.standard_normal((n_tok, n_expert)).astype(np.float32)
+    gate = np.concatenate([make_weights(rein.Q4_K, hidden, ff, 300 + e, True)[1] for e in range(n_expert)])
+    up = np.concatenate([make_weights(rein.Q4_K, hidden, ff, 400 + e, True)[1] for e in range(n_expert)])
+    down = np.concatenate([make_weights(rein.Q6_K, ff, hidden, 500 + e, True)[1] for e in range(n_expert)])
+    ones = np.ones(n_expert, np.float32)
+    sh = runtime.moe_shape(n_tok, hidden, n_expert, n_used, ff, rein.Q4_K, rein.Q6_K)
+    ws = hip.DeviceBuf(runtime.moe_workspace_bytes(sh))
+    d_out = dev(np.full(n_tok * hidden, np.nan, np.float32))
+    runtime.moe_ffn(sh, dev(x), dev(logits), dev(gate), dev(up), dev(down), dev(ones), ws, d_out)
+    hip.synchronize()
+    got = d_out.to_host(np.float32).reshape(n_tok, hidden)
+
+    ids, wts = orc.moe_topk(logits, n_used)
+    perm, eoff, _ = orc.moe_sort(ids, n_expert, 32)
+    gin = orc.moe_gather_xq(orc.quantize_q8(x), perm, hidden // 32, n_used)
+    bpe_gu, bpe_dn = orc.repacked_len(orc.Q4_K, hidden, ff), orc.repacked_len(orc.Q6_K, ff, hidden)
+    eg = orc.grouped_gemm(orc.Q4_K, gate, bpe_gu, eoff, gin, hidden, ff)
+    eu = orc.grouped_gemm(orc.Q4_K, up, bpe_gu, eoff, gin, hidden, ff)
+    act = orc.swiglu_mul(eg, eu)
+    gout = orc.grouped_gemm(orc.Q6_K, down, bpe_dn, eoff, orc.quantize_q8(act), ff, hidden)
+    eout = orc.moe_scatter_rows(gout, perm, hidden).reshape(n_tok, n_used, hidden)
+    want = orc.moe_combine(eout, ids, wts, ones)
+    # the intermediate is re-quantized after SwiGLU, so fp32 noise in gate/up can flip a
+    # quant by one step: compare at the reference's rel_l2 bar plus a loose element bound
+    assert rel_l2(got, want) < 2e-3
+    assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what="moe_ffn")
