@@ -86,13 +86,13 @@ def test_quantize_q8_reference_launch_geometry():
 
 
 # ------------------------------------------------------------------ decode matvec
-def check_matvec_outputs(fmt, raw, packed, xq_host, in_dim, out_dim, y, n_rows, x=None):
+def check_matvec_outputs(fmt, raw, packed, xq_host, in_dim, out_dim, y, n_rows, x=None, f32_tol=1.5e-2):
     want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq_host, n_rows)
     assert_close_f32(y, want, what=f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}")
     if x is not None:
         w = orc.dequantize_to_f32(fmt, raw, in_dim * out_dim).reshape(out_dim, in_dim)
         for t in range(n_rows):
-            assert rel_l2(y[t], orc.matvec_f32(x[t], w)) < 1.5e-2
+            assert rel_l2(y[t], orc.matvec_f32(x[t], w)) < f32_tol
 
 
 SHAPES = [(2048, 384), (4096, 37), (768, 130), (5120, 64)]
@@ -132,8 +132,13 @@ def test_matvec_gaussian_weights_config1_shape(fmt):
     dw, dy = dev(packed), hip.DeviceBuf(out_dim * 4)
     runtime.matvec_xq8(fmt, dw, dq, dy, in_dim, out_dim)
     hip.synchronize()
+    # Against the f32 path the bar is looser here than the reference's 1.5e-2, which it
+    # quotes for weights with scales of both signs: Q4_K/Q5_K pair the *exact* xsum with
+    # *quantized* activations in the dot, so with real (all-positive d*sc) weights the
+    # activation rounding error enters every row with the same sign (~2.5e-2 at K=4096).
+    # That is a property of the reference's formula; the int8 oracle above matches to 1e-3.
     check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim,
-                         dy.to_host(np.float32)[None, :], 1, x)
+                         dy.to_host(np.float32)[None, :], 1, x, f32_tol=5e-2)
 
 
 REF_MATVEC = [  # (kernel symbol, rows per workgroup, threads) exactly as qwen35.rs:2232-2280 launches them
