@@ -278,14 +278,18 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     // token tile: 32 for a handful of rows, wider once the batch can fill it
-    unsigned tm = p_rows <= 32 ? 32 : p_rows <= 64 ? 64 : 128;
+    unsigned tm = p_rows <= 32 ? 32 : 64;
     const unsigned forced = env_u("REIN_MMQ_TM", 0);
-    if (forced == 32 || forced == 64 || forced == 128) tm = forced;
+    if (forced == 32 || forced == 64) tm = forced;
+    if (fmt == REIN_TYPE_Q6_K) tm = 32;          // two int8 MFMAs per sub-block: the 64-token tile does not fit the register file
     const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + tm - 1) / tm;
-    if (n_tt > 65535) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many token tiles");
+    // 1-D grid; workgroup i runs on XCD i % 8 and the kernel maps it to
+    // (row block, token tile) so that one weight block stays on one XCD
+    const unsigned long long grid = 8ull * ((n_rb + 7) / 8) * n_tt;
+    if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many tiles for one launch");
     const std::string name = std::string("rein_mmq_") + fmt_tag(fmt) + "_t" + std::to_string(tm);
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
-    return launch(name, n_rb, n_tt, 1, 256, 0, s, args);
+    return launch(name, (unsigned)grid, 1, 1, 256, 0, s, args);
 }
 
 int rein_matmul_path(int fmt, unsigned n_rows)

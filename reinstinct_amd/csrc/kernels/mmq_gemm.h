@@ -55,169 +55,156 @@ __device__ __forceinline__ int rein_sub_bytes(uint32_t x, uint32_t c4)
     return (int)(((x | 0x80808080u) - c4) ^ 0x80808080u);
 }
 
-// Weight side of one superblock chunk for lane (row, half h):
-//   b[s]     int8 operand (quants 16h..16h+15 of sub-block s, offsets folded)
-//   sc[u]    fp32 scale feeding the outer-product MFMA, mn[u] the (negated) min
-// One-scale formats: u = p (pair index), value for sub-block 2p+h.
-// Q6_K: u = s, value = d*sc_h for this lane's half.
+// Weight side of one superblock chunk (8 sub-blocks) for lane (row, half h).
+//   fetch()   raw plane words HBM/L2 -> registers (so the next chunk can be in
+//             flight while this one is multiplied)
+//   expand()  raw -> b[s]: int8 operand (quants 16h..16h+15 of sub-block s, offsets
+//             folded), sc[u]: fp32 scale feeding the outer-product MFMA, mn[u]:
+//             negated min term
+// One-scale formats: u = pair index p, value for sub-block 2p+h.
+// Q6_K: u = s, value = d*sc_h for this lane's 16-weight half.
 template <int FMT> struct MmqChunk;
 
-#define REIN_MMQ_COMMON                                                                         \
-    rein_v4i b[8];                                                                              \
-    __device__ __forceinline__ static unsigned clamp_sb(unsigned sb, unsigned n_sub)            \
-    {                                                                                           \
-        return sb < n_sub ? sb : n_sub - 1;                                                     \
-    }
+__device__ __forceinline__ unsigned rein_clamp_sb(unsigned sb, unsigned n_sub) { return sb < n_sub ? sb : n_sub - 1; }
 
 template <> struct MmqChunk<REIN_Q4_K> {
     static constexpr bool kTwoScales = false, kHasMin = true;
-    REIN_MMQ_COMMON
+    struct Raw { uint4 q[8]; ReinU16x8 sm; uint32_t dd; };
+    rein_v4i b[8];
     float sc[4], mn[4];
-    __device__ __forceinline__ void load(const Fmt<REIN_Q4_K>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q4_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
     {
-        const size_t i = (size_t)row * f.nsp + sb0;      // K-quants: n_sub % 8 == 0, whole chunk valid
-        const ReinU16x8 sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
-        const uint32_t dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
-        const float d = rein_h2f((uint16_t)(dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(dd >> 16));
+        const size_t i = (size_t)row * f.nsp + sb0;      // K-quants: n_sub % 8 == 0, the whole chunk is valid
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
+        r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
+        r.dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
+    }
+    __device__ __forceinline__ void expand(const Raw& r, unsigned, unsigned, unsigned h)
+    {
+        const float d = rein_h2f((uint16_t)(r.dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(r.dd >> 16));
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const uint4 q = f.nib[i + s];
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) b[s][j] = (int)((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
         }
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            const uint16_t v = h ? sm.v[2 * p + 1] : sm.v[2 * p];
+            const uint16_t v = h ? r.sm.v[2 * p + 1] : r.sm.v[2 * p];
             sc[p] = d * (float)(v & 0xFFu);
             mn[p] = -(dmin * (float)(v >> 8));
         }
-        (void)n_sub;
     }
 };
 
 template <> struct MmqChunk<REIN_Q5_K> {
     static constexpr bool kTwoScales = false, kHasMin = true;
-    REIN_MMQ_COMMON
+    struct Raw { uint4 q[8]; ReinU32x8 qh; ReinU16x8 sm; uint32_t dd; };
+    rein_v4i b[8];
     float sc[4], mn[4];
-    __device__ __forceinline__ void load(const Fmt<REIN_Q5_K>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q5_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
     {
         const size_t i = (size_t)row * f.nsp + sb0;
-        const ReinU16x8 sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
-        const ReinU32x8 qh = *reinterpret_cast<const ReinU32x8*>(f.qhp + i);
-        const uint32_t dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
-        const float d = rein_h2f((uint16_t)(dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(dd >> 16));
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
+        r.qh = *reinterpret_cast<const ReinU32x8*>(f.qhp + i);
+        r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
+        r.dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
+    }
+    __device__ __forceinline__ void expand(const Raw& r, unsigned, unsigned, unsigned h)
+    {
+        const float d = rein_h2f((uint16_t)(r.dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(r.dd >> 16));
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const uint4 q = f.nib[i + s];
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                b[s][j] = (int)(((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | (rein_spread4(qh.v[s] >> (8 * j + 4 * h)) << 4));
+                b[s][j] = (int)(((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | (rein_spread4(r.qh.v[s] >> (8 * j + 4 * h)) << 4));
         }
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            const uint16_t v = h ? sm.v[2 * p + 1] : sm.v[2 * p];
+            const uint16_t v = h ? r.sm.v[2 * p + 1] : r.sm.v[2 * p];
             sc[p] = d * (float)(v & 0xFFu);
             mn[p] = -(dmin * (float)(v >> 8));
         }
-        (void)n_sub;
     }
 };
 
 template <> struct MmqChunk<REIN_Q6_K> {
     static constexpr bool kTwoScales = true, kHasMin = false;
-    REIN_MMQ_COMMON
+    struct Raw { uint4 q[8]; ReinU64x8 h2; ReinU16x8 sm; uint16_t d; };
+    rein_v4i b[8];
     float sc[8];
-    __device__ __forceinline__ void load(const Fmt<REIN_Q6_K>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q6_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
     {
         const size_t i = (size_t)row * f.nsp + sb0;
-        const ReinU16x8 sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
-        const ReinU64x8 h2 = *reinterpret_cast<const ReinU64x8*>(f.h2p + i);
-        const float d = rein_h2f(f.dp[(size_t)row * f.n_super + (sb0 >> 3)]);
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
+        r.h2 = *reinterpret_cast<const ReinU64x8*>(f.h2p + i);
+        r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
+        r.d  = f.dp[(size_t)row * f.n_super + (sb0 >> 3)];
+    }
+    __device__ __forceinline__ void expand(const Raw& r, unsigned, unsigned, unsigned h)
+    {
+        const float d = rein_h2f(r.d);
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const uint4 q = f.nib[i + s];
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 // hi2 byte 2j+h holds the 2-bit fields of this half's word j
-                const uint32_t hw = j < 2 ? h2.v[s].x : h2.v[s].y;
+                const uint32_t hw = j < 2 ? r.h2.v[s].x : r.h2.v[s].y;
                 const uint32_t hb = (hw >> (16 * (j & 1) + 8 * h)) & 0xFFu;
                 const uint32_t q6 = ((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | rein_spread2(hb);
                 b[s][j] = rein_sub_bytes(q6, 0x20202020u);
             }
-            const uint16_t v = sm.v[s];
+            const uint16_t v = r.sm.v[s];
             sc[s] = d * (float)(int)(int8_t)(h ? (v >> 8) : (v & 0xFFu));
         }
-        (void)n_sub;
     }
 };
 
-template <> struct MmqChunk<REIN_Q8_0> {
+// Q8_0 / Q4_0 / IQ4_XS: one fp16 scale per sub-block, the chunk may be ragged
+// (in_dim is only a multiple of 32): sub-blocks past the end are clamped and
+// their scale is forced to zero.
+template <int FMT> struct MmqChunkD16 {
     static constexpr bool kTwoScales = false, kHasMin = false;
-    REIN_MMQ_COMMON
+    struct Raw { uint4 q[8]; uint16_t d[4]; };
+    rein_v4i b[8];
     float sc[4], mn[4];
-    __device__ __forceinline__ void load(const Fmt<REIN_Q8_0>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<FMT>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
     {
-        const uint4* plane = h ? f.hip_ : f.lop;
+        const uint4* plane;
+        if constexpr (FMT == REIN_Q8_0) plane = h ? f.hip_ : f.lop;     // this lane's 16 quants are one plane entry
+        else plane = f.nib;
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = plane[(size_t)row * f.nsp + rein_clamp_sb(sb0 + s, n_sub)];
+#pragma unroll
+        for (int p = 0; p < 4; p++) r.d[p] = f.dp[(size_t)row * f.nsp + rein_clamp_sb(sb0 + 2 * p + h, n_sub)];
+    }
+    __device__ __forceinline__ void expand(const Raw& r, unsigned sb0, unsigned n_sub, unsigned h)
+    {
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const uint4 q = plane[(size_t)row * f.nsp + clamp_sb(sb0 + s, n_sub)];
-            b[s][0] = (int)q.x; b[s][1] = (int)q.y; b[s][2] = (int)q.z; b[s][3] = (int)q.w;
+            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if constexpr (FMT == REIN_Q8_0) b[s][j] = (int)w[j];
+                else if constexpr (FMT == REIN_Q4_0) b[s][j] = rein_sub_bytes((w[j] >> (4 * h)) & 0x0F0F0F0Fu, 0x08080808u);
+                else b[s][j] = rein_iq4_lut4((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
+            }
         }
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            const unsigned sb = sb0 + 2 * p + h;
-            sc[p] = sb < n_sub ? rein_h2f(f.dp[(size_t)row * f.nsp + sb]) : 0.0f;
+            sc[p] = sb0 + 2 * p + h < n_sub ? rein_h2f(r.d[p]) : 0.0f;
             mn[p] = 0.0f;
         }
     }
 };
-
-template <> struct MmqChunk<REIN_Q4_0> {
-    static constexpr bool kTwoScales = false, kHasMin = false;
-    REIN_MMQ_COMMON
-    float sc[4], mn[4];
-    __device__ __forceinline__ void load(const Fmt<REIN_Q4_0>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
-    {
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const uint4 q = f.nib[(size_t)row * f.nsp + clamp_sb(sb0 + s, n_sub)];
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[s][j] = rein_sub_bytes((w[j] >> (4 * h)) & 0x0F0F0F0Fu, 0x08080808u);
-        }
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const unsigned sb = sb0 + 2 * p + h;
-            sc[p] = sb < n_sub ? rein_h2f(f.dp[(size_t)row * f.nsp + sb]) : 0.0f;
-            mn[p] = 0.0f;
-        }
-    }
-};
-
-template <> struct MmqChunk<REIN_IQ4_XS> {
-    static constexpr bool kTwoScales = false, kHasMin = false;
-    REIN_MMQ_COMMON
-    float sc[4], mn[4];
-    __device__ __forceinline__ void load(const Fmt<REIN_IQ4_XS>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
-    {
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const uint4 q = f.nib[(size_t)row * f.nsp + clamp_sb(sb0 + s, n_sub)];
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[s][j] = rein_iq4_lut4((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
-        }
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const unsigned sb = sb0 + 2 * p + h;
-            sc[p] = sb < n_sub ? rein_h2f(f.dp[(size_t)row * f.nsp + sb]) : 0.0f;
-            mn[p] = 0.0f;
-        }
-    }
-};
+template <> struct MmqChunk<REIN_Q8_0> : MmqChunkD16<REIN_Q8_0> {};
+template <> struct MmqChunk<REIN_Q4_0> : MmqChunkD16<REIN_Q4_0> {};
+template <> struct MmqChunk<REIN_IQ4_XS> : MmqChunkD16<REIN_IQ4_XS> {};
 
 // LDS image of one activation chunk: TM tokens x 8 sub-blocks.
 template <int TM>
@@ -280,7 +267,11 @@ __device__ __forceinline__ void rein_mmq_tile(const uint8_t* __restrict__ w, con
 
     for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 8) {
         C ck;
-        ck.load(fmt, rowc, sb0, n_sub, h);        // HBM/L2 -> registers, overlaps the staging below
+        {
+            typename C::Raw raw;
+            C::fetch(raw, fmt, rowc, sb0, n_sub, h);   // HBM/L2 -> registers, overlaps the staging below
+            ck.expand(raw, sb0, n_sub, h);
+        }
         __syncthreads();                           // previous chunk's LDS reads are done
         rein_mmq_stage<TM>(lds, xq, n_sub, tok_base, tok_end, sb0);
         __syncthreads();
@@ -380,6 +371,180 @@ __device__ __forceinline__ void rein_mmq_tile(const uint8_t* __restrict__ w, con
     }
 }
 
+// ---------------------------------------------------------------------------
+// Pipelined dense MMQ (the tuned launch).  Same math and layouts as
+// rein_mmq_tile, plus:
+//   * the next chunk's weight words and activation blocks are fetched into
+//     registers before the current chunk is multiplied, the LDS image is
+//     double-buffered, and there is one barrier per chunk;
+//   * a fixed workgroup of 4 wavefronts (128 rows x TM tokens);
+//   * a 1-D grid whose workgroup -> tile map keeps all token tiles of one
+//     128-row weight block on the same XCD (workgroups are dealt round-robin
+//     over the 8 XCDs, each with its own L2), so a weight block is pulled from
+//     HBM once and re-read from that L2.
+// Grid: 8 * ceil(n_row_blocks / 8) * n_token_tiles workgroups of 256 threads.
+template <int TM>
+struct MmqXRegs {
+    static constexpr int kPer = TM * 8 / 256;            // activation blocks per thread per chunk
+    uint2 hdr[kPer];
+    uint4 lo[kPer], hi[kPer];
+};
+
+template <int TM>
+__device__ __forceinline__ void rein_mmq_xfetch(MmqXRegs<TM>& r, const BlockQ8* __restrict__ xq, unsigned n_sub,
+                                                unsigned tok_base, unsigned tok_end, unsigned sb0)
+{
+#pragma unroll
+    for (int k = 0; k < MmqXRegs<TM>::kPer; k++) {
+        const unsigned e = threadIdx.x + k * 256;
+        const unsigned tl = e >> 3, s = e & 7;
+        const unsigned tok = tok_base + tl, sb = sb0 + s;
+        const bool ok = tok < tok_end && sb < n_sub;
+        const BlockQ8* p = xq + (size_t)(tok < tok_end ? tok : tok_end - 1) * n_sub + (sb < n_sub ? sb : n_sub - 1);
+        const float d = p->d, xs = p->xsum;
+        r.hdr[k].x = ok ? __builtin_bit_cast(unsigned, d) : 0u;
+        r.hdr[k].y = ok ? __builtin_bit_cast(unsigned, xs) : 0u;
+        r.lo[k].x = p->qs[0]; r.lo[k].y = p->qs[1]; r.lo[k].z = p->qs[2]; r.lo[k].w = p->qs[3];
+        r.hi[k].x = p->qs[4]; r.hi[k].y = p->qs[5]; r.hi[k].z = p->qs[6]; r.hi[k].w = p->qs[7];
+    }
+}
+
+template <int TM>
+__device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM>& r)
+{
+#pragma unroll
+    for (int k = 0; k < MmqXRegs<TM>::kPer; k++) {
+        const unsigned e = threadIdx.x + k * 256;
+        const unsigned tl = e >> 3, s = e & 7;
+        l.qs[0][s][tl] = r.lo[k];
+        l.qs[1][s][tl] = r.hi[k];
+        l.dx[s][tl]    = __builtin_bit_cast(float, r.hdr[k].x);
+        l.xsum[s][tl]  = __builtin_bit_cast(float, r.hdr[k].y);
+    }
+}
+
+// multiply one staged chunk into the accumulators
+template <int FMT, int TM>
+__device__ __forceinline__ void rein_mmq_chunk_math(const MmqLds<TM>& lds, const MmqChunk<FMT>& ck,
+                                                    rein_v16f (&acc)[TM / 32], unsigned j, unsigned h)
+{
+    using C = MmqChunk<FMT>;
+    constexpr int NT = TM / 32;
+    rein_v16i z;
+#pragma unroll
+    for (int v = 0; v < 16; v++) z[v] = 0;
+    rein_v32f z32;
+#pragma unroll
+    for (int v = 0; v < 32; v++) z32[v] = 0.0f;
+
+    if constexpr (C::kTwoScales) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            rein_v4i blo, bhi;
+#pragma unroll
+            for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : ck.b[s][k]; bhi[k] = h ? ck.b[s][k] : 0; }
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 a4 = lds.qs[h][s][t * 32 + j];
+                rein_v4i a;
+                a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
+                const rein_v16i clo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, z, 0, 0, 0);
+                const rein_v16i chi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, z, 0, 0, 0);
+                const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    acc[t][v] = fmaf((float)clo[v], sx[v], acc[t][v]);
+                    acc[t][v] = fmaf((float)chi[v], sx[16 + v], acc[t][v]);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 a40 = lds.qs[h][2 * p][t * 32 + j];
+                const uint4 a41 = lds.qs[h][2 * p + 1][t * 32 + j];
+                rein_v4i a0, a1;
+                a0[0] = (int)a40.x; a0[1] = (int)a40.y; a0[2] = (int)a40.z; a0[3] = (int)a40.w;
+                a1[0] = (int)a41.x; a1[1] = (int)a41.y; a1[2] = (int)a41.z; a1[3] = (int)a41.w;
+                const rein_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, ck.b[2 * p], z, 0, 0, 0);
+                const rein_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, ck.b[2 * p + 1], z, 0, 0, 0);
+                const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[p], z32, 0, 0, 0);
+                if constexpr (C::kHasMin)
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(lds.xsum[2 * p + h][t * 32 + j], ck.mn[p], acc[t], 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    acc[t][v] = fmaf((float)c0[v], sx[v], acc[t][v]);
+                    acc[t][v] = fmaf((float)c1[v], sx[16 + v], acc[t][v]);
+                }
+            }
+        }
+    }
+}
+
+template <int FMT, int TM>
+__device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                   float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                   unsigned p_rows)
+{
+    using F = Fmt<FMT>;
+    using C = MmqChunk<FMT>;
+    constexpr int NT = TM / 32;
+    __shared__ MmqLds<TM> lds[2];
+
+    // workgroup -> (row block, token tile), XCD-aware
+    const unsigned n_rb = (out_dim + 127u) / 128u;
+    const unsigned n_tt = (p_rows + TM - 1) / TM;
+    const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
+    const unsigned rb = (k / n_tt) * 8u + xcd, tt = k % n_tt;
+    if (rb >= n_rb) return;
+
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned j = lane & 31u, h = lane >> 5;
+    const unsigned n_sub = in_dim >> 5;
+    const F fmt(w, n_sub, out_dim);
+    const unsigned row = rb * 128u + wave * 32u + j;
+    const unsigned rowc = row < out_dim ? row : out_dim - 1;
+    const unsigned tok_base = tt * TM;
+    const unsigned tok_end = min(p_rows, tok_base + TM);
+
+    rein_v16f acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
+
+    typename C::Raw raw;
+    MmqXRegs<TM> xr;
+    C::fetch(raw, fmt, rowc, 0, n_sub, h);
+    rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 0);
+    rein_mmq_xstore<TM>(lds[0], xr);
+    __syncthreads();
+
+    unsigned buf = 0;
+    for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 8, buf ^= 1u) {
+        C ck;
+        ck.expand(raw, sb0, n_sub, h);
+        const bool more = sb0 + 8 < n_sub;
+        if (more) {                                  // next chunk goes out before the math
+            C::fetch(raw, fmt, rowc, sb0 + 8, n_sub, h);
+            rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, sb0 + 8);
+        }
+        rein_mmq_chunk_math<FMT, TM>(lds[buf], ck, acc, j, h);
+        if (more) rein_mmq_xstore<TM>(lds[buf ^ 1u], xr);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const unsigned tok = tok_base + t * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+            if (tok < tok_end && row < out_dim) y[(size_t)tok * out_dim + row] = acc[t][v];
+        }
+}
+
 // Dense GEMM: grid-stride over (row block, token tile).
 template <int FMT, int TM, int DOTS>
 __device__ __forceinline__ void rein_mmq_dense(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
@@ -433,6 +598,13 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     extern "C" __global__ __launch_bounds__(256) void name(REIN_MMQ_ARGS)                        \
     {                                                                                            \
         rein_mmq_dense<FMT, TM, 0>(w, xq, y, nullptr, in_dim, out_dim, p_rows);                  \
+    }
+
+// tuned entry: fixed 256-thread workgroups, 1-D XCD-aware grid
+#define REIN_DEFINE_MMQ_PIPE(name, FMT, TM)                                                      \
+    extern "C" __global__ __launch_bounds__(256) void name(REIN_MMQ_ARGS)                        \
+    {                                                                                            \
+        rein_mmq_pipelined<FMT, TM>(w, xq, y, in_dim, out_dim, p_rows);                          \
     }
 
 #define REIN_DEFINE_MMQ_DOTS(name, FMT)                                                          \

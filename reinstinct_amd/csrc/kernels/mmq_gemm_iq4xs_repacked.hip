@@ -8,7 +8,6 @@
 
 REIN_DEFINE_MMQ(mmq_gemm_iq4xs_repacked_f32, REIN_IQ4_XS, 64)
 REIN_DEFINE_MMQ(mmq_gemm_iq4xs_repacked_narrow_f32, REIN_IQ4_XS, 32)
-REIN_DEFINE_MMQ(rein_mmq_iq4xs_t32, REIN_IQ4_XS, 32)
-REIN_DEFINE_MMQ(rein_mmq_iq4xs_t64, REIN_IQ4_XS, 64)
-REIN_DEFINE_MMQ(rein_mmq_iq4xs_t128, REIN_IQ4_XS, 128)
+REIN_DEFINE_MMQ_PIPE(rein_mmq_iq4xs_t32, REIN_IQ4_XS, 32)
+REIN_DEFINE_MMQ_PIPE(rein_mmq_iq4xs_t64, REIN_IQ4_XS, 64)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_iq4xs, REIN_IQ4_XS)

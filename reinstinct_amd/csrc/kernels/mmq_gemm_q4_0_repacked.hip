@@ -8,7 +8,6 @@
 
 REIN_DEFINE_MMQ(mmq_gemm_q4_0_repacked_f32, REIN_Q4_0, 64)
 REIN_DEFINE_MMQ(mmq_gemm_q4_0_repacked_narrow_f32, REIN_Q4_0, 32)
-REIN_DEFINE_MMQ(rein_mmq_q4_0_t32, REIN_Q4_0, 32)
-REIN_DEFINE_MMQ(rein_mmq_q4_0_t64, REIN_Q4_0, 64)
-REIN_DEFINE_MMQ(rein_mmq_q4_0_t128, REIN_Q4_0, 128)
+REIN_DEFINE_MMQ_PIPE(rein_mmq_q4_0_t32, REIN_Q4_0, 32)
+REIN_DEFINE_MMQ_PIPE(rein_mmq_q4_0_t64, REIN_Q4_0, 64)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q4_0, REIN_Q4_0)

@@ -8,7 +8,6 @@
 
 REIN_DEFINE_MMQ(mmq_gemm_q4k_repacked_f32, REIN_Q4_K, 64)
 REIN_DEFINE_MMQ(mmq_gemm_q4k_repacked_narrow_f32, REIN_Q4_K, 32)
-REIN_DEFINE_MMQ(rein_mmq_q4k_t32, REIN_Q4_K, 32)
-REIN_DEFINE_MMQ(rein_mmq_q4k_t64, REIN_Q4_K, 64)
-REIN_DEFINE_MMQ(rein_mmq_q4k_t128, REIN_Q4_K, 128)
+REIN_DEFINE_MMQ_PIPE(rein_mmq_q4k_t32, REIN_Q4_K, 32)
+REIN_DEFINE_MMQ_PIPE(rein_mmq_q4k_t64, REIN_Q4_K, 64)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q4k, REIN_Q4_K)
