@@ -1,19 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-weight matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu] [--no-mmq]
 
-Headline workload (BASELINE.json configs[1], first shape): Q4_K repacked-v2 decode
-matvec, batch 1, K=5120 -> N=5120, weights ~N(0,0.02) quantized to Q4_K, activation
-~N(0,1) quantized to BlockQ8.  One *step* is one pass of the matvec over a rotation
-of distinct weight buffers (together larger than L2 + Infinity Cache, so every
-launch streams its weights from HBM), captured in a hipGraph.  Everything is
-resident in HBM before the timed region.  Prints ONE JSON line.
+Headline workload (BASELINE.json configs[1], Q4_K, batch 1): the three decode
+matvec shapes of the 27B-class layer -- K=5120 -> N=5120, the fused gate+up
+K=5120 -> N=34816 and down K=17408 -> N=5120 -- with weights ~N(0,0.02) quantized
+to Q4_K and repacked, activations ~N(0,1) quantized to BlockQ8.  One *step* is one
+pass of each shape over a rotation of distinct weight buffers (each rotation larger
+than L2 + Infinity Cache, so every launch streams its weights from HBM), captured
+in one hipGraph per shape.  `value` is total algorithmic bytes / total time over
+the three shapes; everything is resident in HBM before the timed region.  Prints
+ONE JSON line.
 
-The same line carries the MMQ prefill GEMM (Q4_K, 512 x 5120 x 17408) in "mmq",
-the roofline object of the dominant kernel and the CPU baseline (the oracle's
-restatement of the reference CPU path: dequantize once, then the f32 matvec of
-src/cpu/ops.rs:108-140 over all host cores) timed on a bounded sample.
+The same line carries the per-shape figures, the roofline object of the dominant
+kernel (the gate+up launch), the MMQ prefill GEMM (Q4_K, 512 x 5120 x 17408) in
+"mmq" and the CPU baseline (the oracle's restatement of the reference CPU path:
+dequantize once, then the f32 matvec of src/cpu/ops.rs:108-140 over the host
+cores) timed on a bounded sample.
 """
 import argparse
 import json
@@ -165,6 +169,14 @@ def cpu_baseline(fmt, in_dim, out_dim, seed, budget_s=12.0):
                       f"algorithmic (repacked) bytes / time; {round(in_dim * out_dim * 4 / best / 1e9, 2)} GB/s of f32 traffic"}
 
 
+HEADLINE_SHAPES = ((5120, 5120), (5120, 34816), (17408, 5120))      # (K, N) of configs[1]
+# HBM bytes per launch of the dominant kernel (Q4_K 5120 -> 34816, batch 1) from rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by the same counter's reading for the
+# set-up device-to-device copies of known size (fetch x1.99905, write x1.0); it cannot be read
+# live, so it is the recorded figure and only reported for the configuration it was taken on
+DOMINANT_TRAFFIC_BYTES = 104054700
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -174,7 +186,6 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mmq", action="store_true")
     ap.add_argument("--fmt", default="q4_k")
-    ap.add_argument("--shape", default="5120x5120", help="KxN of the headline matvec")
     ap.add_argument("--batch", type=int, default=1)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -186,26 +197,53 @@ def main():
     hip.set_device(0)
     stream = hip.Stream()
     fmt = rein.FORMATS[args.fmt]
-    in_dim, out_dim = (int(v) for v in args.shape.lower().split("x"))
 
-    case = MatvecCase(fmt, in_dim, out_dim, args.batch, stream, seed=1234)
-    sec_step, sec_launch = case.time(args.steps, args.warmup)
-    gbs = case.bytes_per_launch / sec_launch / 1e9
-    log(f"matvec {args.fmt} {in_dim}->{out_dim} b{args.batch}: {sec_launch * 1e6:.2f} us/launch, {gbs:.0f} GB/s "
-        f"({case.n_buf} buffers/step)")
+    cases = [MatvecCase(fmt, k, n, args.batch, stream, seed=1234 + i) for i, (k, n) in enumerate(HEADLINE_SHAPES)]
+    for c in cases:
+        for _ in range(args.warmup):
+            c.step()
+    stream.synchronize()
+    # K steps, each = one pass of every shape; one event pair per shape and step so
+    # the per-kernel launch time is measured on the launch stream itself
+    marks = [[(hip.Event(), hip.Event()) for _ in cases] for _ in range(args.steps)]
+    t0, t1 = hip.Event(), hip.Event()
+    t0.record(stream)
+    for k in range(args.steps):
+        for c, (e0, e1) in zip(cases, marks[k]):
+            e0.record(stream)
+            c.step()
+            e1.record(stream)
+    t1.record(stream)
+    t1.synchronize()
+    total_s = t0.elapsed_ms(t1) * 1e-3
+    shapes = []
+    for i, c in enumerate(cases):
+        sec = sum(marks[k][i][0].elapsed_ms(marks[k][i][1]) for k in range(args.steps)) * 1e-3
+        per_launch = sec / (args.steps * c.n_buf)
+        gbs = c.bytes_per_launch / per_launch / 1e9
+        shapes.append({"K": c.in_dim, "N": c.out_dim, "us_per_launch": round(per_launch * 1e6, 3),
+                       "GBs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                       "bytes_per_launch": c.bytes_per_launch, "launches_per_step": c.n_buf})
+        log(f"matvec {args.fmt} {c.in_dim}->{c.out_dim} b{args.batch}: {per_launch * 1e6:.2f} us/launch, {gbs:.0f} GB/s "
+            f"({c.n_buf} buffers/step)")
+    step_bytes = sum(c.bytes_per_launch * c.n_buf for c in cases)
+    value = step_bytes * args.steps / total_s / 1e9
+    is_headline = fmt == rein.Q4_K and args.batch == 1
+    dom = shapes[1]                                   # gate+up: most bytes, its own kernel variant
 
     out = {
         "metric": "Q4_K decode matvec HBM GB/s (% of peak) + MMQ pp512 int8 TOPS, 1 MI355X",
-        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(sec_step * 1e3, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "int8 dot4 / fp32 accumulate", "data": "synthetic",
-        "config": {"workload": f"{args.fmt} repacked-v2 decode matvec K={in_dim} N={out_dim} batch={args.batch} "
-                               f"(BASELINE configs[1]); step = one pass over {case.n_buf} distinct weight buffers",
-                   "launches_per_step": case.n_buf, "bytes_per_launch": case.bytes_per_launch,
-                   "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2)},
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": f"rein_mv_{'q4k' if fmt == rein.Q4_K else args.fmt}", "us_per_launch": round(sec_launch * 1e6, 3)},
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(total_s / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8 (int8 dot4, fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"{args.fmt} repacked-v2 decode matvec, batch {args.batch}, BASELINE configs[1] shapes "
+                               "5120->5120, 5120->34816 (fused gate+up), 17408->5120; value = total algorithmic bytes "
+                               "/ total time; step = one pass of each shape over its rotation of distinct weight buffers",
+                   "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2), "shapes": shapes},
+        "roofline": {"bound": "hbm", "achieved": dom["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": dom["frac_of_hbm_peak"], "traffic": DOMINANT_TRAFFIC_BYTES if is_headline else None,
+                     "kernel": "rein_mv_q4k_r4_b1 (K=5120 -> N=34816)", "us_per_launch": dom["us_per_launch"],
+                     "algorithmic_bytes_per_launch": dom["bytes_per_launch"]},
     }
 
     if not args.no_mmq:
@@ -215,12 +253,14 @@ def main():
         log(f"mmq q4_k 512x5120x17408: {sec * 1e6:.1f} us, {tops:.1f} TOPS")
         out["mmq"] = {"workload": "Q4_K MMQ prefill GEMM 512x5120x17408 (BASELINE configs[2])",
                       "us_per_launch": round(sec * 1e6, 2), "value": round(tops, 2), "unit": "int8 TOPS",
-                      "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+                      "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                   "frac": round(tops / INT8_PEAK_TOPS, 4)}}
+        del mm
 
     if args.sweep:
         sweep = []
         for f in (rein.Q4_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.IQ4_XS):
-            for (k, n) in ((5120, 5120), (5120, 34816), (17408, 5120)):
+            for (k, n) in HEADLINE_SHAPES:
                 _, packed = synth_weights(f, k, n, seed=5)
                 for b in (1, 2, 4, 8):
                     c = MatvecCase(f, k, n, b, stream, seed=5, packed=packed)
@@ -233,7 +273,7 @@ def main():
         out["sweep"] = sweep
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(fmt, in_dim, out_dim, seed=1234)
+        out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)
         log("cpu baseline:", out["cpu_baseline"])
     print(json.dumps(out), flush=True)
 

@@ -126,12 +126,15 @@ constexpr unsigned kCUs = 256;    // MI355X
 
 // Rows per wavefront pass for the decode matvec.  More rows per wave amortise
 // the activation read and the cross-lane reduction; fewer rows put more waves in
-// flight.  Keep at least ~16 waves per CU unless the matrix is too small.
+// flight.  Measured on MI355X (Q4_K, batch 1): 4 rows win once that still leaves
+// ~32 waves per CU (N = 34816), 2 rows down to ~8 waves per CU (N = 5120), 1 row
+// below that.
 unsigned pick_rows_per_wave(unsigned out_dim, unsigned batch)
 {
     const unsigned forced = env_u("REIN_MV_ROWS", 0);
-    unsigned r = 4;
-    while (r > 1 && (r * batch > 16 || (out_dim + r - 1) / r < kCUs * 16)) r >>= 1;
+    unsigned r = 1;
+    if ((out_dim + 3) / 4 >= kCUs * 32) r = 4;
+    else if ((out_dim + 1) / 2 >= kCUs * 8) r = 2;
     if (forced == 1 || forced == 2 || forced == 4) r = forced;
     while (r > 1 && r * batch > 16) r >>= 1;
     return r;

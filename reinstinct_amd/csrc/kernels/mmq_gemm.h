@@ -394,32 +394,36 @@ template <int TM>
 __device__ __forceinline__ void rein_mmq_xfetch(MmqXRegs<TM>& r, const BlockQ8* __restrict__ xq, unsigned n_sub,
                                                 unsigned tok_base, unsigned tok_end, unsigned sb0)
 {
+    // loads only: nothing here may consume a loaded value, or the wait for it
+    // lands in front of the chunk's math and the prefetch is lost
 #pragma unroll
     for (int k = 0; k < MmqXRegs<TM>::kPer; k++) {
         const unsigned e = threadIdx.x + k * 256;
         const unsigned tl = e >> 3, s = e & 7;
         const unsigned tok = tok_base + tl, sb = sb0 + s;
-        const bool ok = tok < tok_end && sb < n_sub;
-        const BlockQ8* p = xq + (size_t)(tok < tok_end ? tok : tok_end - 1) * n_sub + (sb < n_sub ? sb : n_sub - 1);
-        const float d = p->d, xs = p->xsum;
-        r.hdr[k].x = ok ? __builtin_bit_cast(unsigned, d) : 0u;
-        r.hdr[k].y = ok ? __builtin_bit_cast(unsigned, xs) : 0u;
-        r.lo[k].x = p->qs[0]; r.lo[k].y = p->qs[1]; r.lo[k].z = p->qs[2]; r.lo[k].w = p->qs[3];
-        r.hi[k].x = p->qs[4]; r.hi[k].y = p->qs[5]; r.hi[k].z = p->qs[6]; r.hi[k].w = p->qs[7];
+        const uint2* p = reinterpret_cast<const uint2*>(
+            xq + (size_t)(tok < tok_end ? tok : tok_end - 1) * n_sub + (sb < n_sub ? sb : n_sub - 1));
+        const uint2 w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];   // 8-byte aligned words
+        r.hdr[k] = w0;
+        r.lo[k].x = w1.x; r.lo[k].y = w1.y; r.lo[k].z = w2.x; r.lo[k].w = w2.y;
+        r.hi[k].x = w3.x; r.hi[k].y = w3.y; r.hi[k].z = w4.x; r.hi[k].w = w4.y;
     }
 }
 
+// rows past tok_end / sub-blocks past n_sub get zero scales here
 template <int TM>
-__device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM>& r)
+__device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM>& r, unsigned n_sub,
+                                                unsigned tok_base, unsigned tok_end, unsigned sb0)
 {
 #pragma unroll
     for (int k = 0; k < MmqXRegs<TM>::kPer; k++) {
         const unsigned e = threadIdx.x + k * 256;
         const unsigned tl = e >> 3, s = e & 7;
+        const bool ok = tok_base + tl < tok_end && sb0 + s < n_sub;
         l.qs[0][s][tl] = r.lo[k];
         l.qs[1][s][tl] = r.hi[k];
-        l.dx[s][tl]    = __builtin_bit_cast(float, r.hdr[k].x);
-        l.xsum[s][tl]  = __builtin_bit_cast(float, r.hdr[k].y);
+        l.dx[s][tl]    = ok ? __builtin_bit_cast(float, r.hdr[k].x) : 0.0f;
+        l.xsum[s][tl]  = ok ? __builtin_bit_cast(float, r.hdr[k].y) : 0.0f;
     }
 }
 
@@ -519,7 +523,7 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
     MmqXRegs<TM> xr;
     C::fetch(raw, fmt, rowc, 0, n_sub, h);
     rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 0);
-    rein_mmq_xstore<TM>(lds[0], xr);
+    rein_mmq_xstore<TM>(lds[0], xr, n_sub, tok_base, tok_end, 0);
     __syncthreads();
 
     unsigned buf = 0;
@@ -532,7 +536,7 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
             rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, sb0 + 8);
         }
         rein_mmq_chunk_math<FMT, TM>(lds[buf], ck, acc, j, h);
-        if (more) rein_mmq_xstore<TM>(lds[buf ^ 1u], xr);
+        if (more) rein_mmq_xstore<TM>(lds[buf ^ 1u], xr, n_sub, tok_base, tok_end, sb0 + 8);
         __syncthreads();
     }
 
