@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <algorithm>
 #include <string>
 #include <unordered_map>
 
@@ -142,6 +143,48 @@ unsigned pick_rows_per_wave(unsigned out_dim, unsigned batch)
 
 unsigned batch_slot(unsigned n_rows) { return n_rows <= 1 ? 1 : n_rows <= 2 ? 2 : n_rows <= 4 ? 4 : 8; }
 
+// Skinny MMQ (rein_mmqs_<fmt>_v<NV>): up to 16 activation rows per token group on
+// the matrix cores; KS wavefronts of a workgroup (the block size) split the
+// contraction over the same 32 weight rows.  The kernel hides latency with resident
+// wavefronts, so KS is the smallest split that fills the machine: waves_per_cu is
+// what LDS and the 128-register budget allow (at most 16), a CU holds
+// floor(waves_per_cu / KS) workgroups, and a choice costs
+// rounds x (chunks per wavefront + about two chunks of pipeline fill), with a
+// penalty when fewer than about 12 wavefronts per CU are resident.
+int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                  unsigned n_rows, rein_stream_t s)
+{
+    const unsigned nv = n_rows <= 8 ? 4 : 8, tok = 2 * nv;
+    const unsigned tiles = ((out_dim + 31) / 32) * ((n_rows + tok - 1) / tok);
+    const unsigned n_chunks = (in_dim / 32 + 7) / 8;
+    const unsigned planes = fmt == REIN_TYPE_Q8_0 ? 2 : 1;
+    const unsigned small_lds = fmt == REIN_TYPE_Q4_K ? 640 : fmt == REIN_TYPE_Q5_K ? 1664 : fmt == REIN_TYPE_Q6_K ? 2688 : 512;
+    const unsigned lds_per_wave = planes * 4096 + 2 * (320 * tok + small_lds);    // sizeof(SkinnyWaveLds<FMT, TOK>)
+    const unsigned waves_per_cu = std::min(16u, 160u * 1024u / lds_per_wave);
+    const unsigned ks_max = std::min(std::min(16u, waves_per_cu), n_chunks);
+    unsigned ks = 1;
+    double best = 1e30;
+    for (unsigned k = 1; k <= ks_max; k++) {
+        const unsigned wg_per_cu = waves_per_cu / k;
+        const unsigned rounds = (tiles + kCUs * wg_per_cu - 1) / (kCUs * wg_per_cu);
+        // wavefronts resident per CU in a typical round
+        const double resident = std::min((double)wg_per_cu * k, (double)tiles * k / (kCUs * rounds));
+        const double cost = rounds * ((n_chunks + k - 1) / k + 2.0) * std::max(1.0, 12.0 / resident);
+        if (cost < best) { best = cost; ks = k; }
+    }
+    const unsigned forced = env_u("REIN_SKINNY_KS", 0);
+    if (forced >= 1 && forced <= ks_max) ks = forced;
+    const std::string name = std::string("rein_mmqs_") + fmt_tag(fmt) + "_v" + std::to_string(nv);
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+    return launch(name, (out_dim + 31) / 32, (n_rows + tok - 1) / tok, 1, ks * 64, ks * lds_per_wave, s, args);
+}
+
+// Activation rows from which the batched decode leaves the dot4 kernels for the
+// skinny MMQ (v_dot4 issues at a quarter of the fp32 rate on this part, so eight
+// dot4 chains per weight row cost more than one MFMA tile).  Measured on MI355X,
+// Q4_K: at 4 rows the two are level, at 8 rows the skinny MMQ is 1.7-2.3x faster.
+unsigned skinny_from_rows() { return env_u("REIN_SKINNY_FROM", 5); }
+
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
                   unsigned out_dim, unsigned n_rows, rein_stream_t s)
 {
@@ -150,6 +193,8 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
+    if (n_rows >= skinny_from_rows() && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(out_dim, b);
     const unsigned wpb = 4;
@@ -280,6 +325,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows() <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // token tile: 32 for a handful of rows, wider once the batch can fill it
     unsigned tm = p_rows <= 32 ? 32 : 64;
     const unsigned forced = env_u("REIN_MMQ_TM", 0);

@@ -8,7 +8,7 @@
 //
 //   * activations: the TM x 8 BlockQ8 of the chunk are staged in LDS, split into
 //     the two 16-quant halves (so an MFMA operand is one conflict-free
-//     ds_read_b128) plus planes of dx and xsum;
+//     ds_read_b128) plus planes of dx and of the bf16 splits of xsum;
 //   * weights: lane (j = lane%32, h = lane/32) streams row j's eight sub-blocks
 //     straight from HBM/L2 (8 x 16 B contiguous = one cache line, scales as one
 //     16 B load), expands half h of each to int8 in registers, and keeps them
@@ -20,9 +20,10 @@
 //     operands;
 //   * scales: v_mfma_f32_32x32x1_2b forms the outer products dx[token] *
 //     dsc[row] for two sub-blocks at once in the accumulator layout, so the
-//     combine is one convert and one fma per element; the -deff*xsum term of
-//     Q4_K/Q5_K is a v_mfma_f32_32x32x2 (K = the two sub-blocks) straight into
-//     the fp32 accumulators;
+//     combine is one subtract (the int32 dots come out biased so that their bits
+//     read as fp32) and one fma per element; the -dmin*m*xsum term of Q4_K/Q5_K
+//     is one superblock-wide pair of bf16 MFMAs on the three-way bf16 split of
+//     xsum against the integer mins (exact products), scaled by -dmin;
 //   * Q6_K has one scale per 16 weights: two int8 MFMAs per sub-block with the
 //     other half of the weight operand zeroed, and the 2-block outer product
 //     holds dx*dsc_lo and dx*dsc_hi.  The -32 (Q6_K) and -8 (Q4_0) offsets are
@@ -44,6 +45,23 @@ typedef int   rein_v4i  __attribute__((ext_vector_type(4)));
 typedef int   rein_v16i __attribute__((ext_vector_type(16)));
 typedef float rein_v16f __attribute__((ext_vector_type(16)));
 typedef float rein_v32f __attribute__((ext_vector_type(32)));
+typedef __bf16 rein_v8bf __attribute__((ext_vector_type(8)));
+
+// The int8 MFMA accumulates on top of this bias, so its int32 result read as
+// fp32 is exactly 12582912 + dot (|dot| < 2^22), and one v_sub_f32 replaces the
+// slower v_cvt_f32_i32.
+#define REIN_MMQ_MAGIC_I 0x4B400000
+#define REIN_MMQ_MAGIC_F 12582912.0f
+
+// Whole-vector form on purpose: written per element (bit_cast of c[v], then the
+// subtract) hipcc 7.2 reuses element 0 for all sixteen lanes of the tile.
+__device__ __forceinline__ rein_v16f rein_mmq_unbias(rein_v16i c)
+{
+    return __builtin_bit_cast(rein_v16f, c) - REIN_MMQ_MAGIC_F;
+}
+
+// bf16 bit pattern of a small non-negative integer (exact below 256)
+__device__ __forceinline__ uint32_t rein_bf16_of_u8(uint32_t v) { return __builtin_bit_cast(uint32_t, (float)v) >> 16; }
 
 struct __attribute__((packed, aligned(2))) ReinU16x8 { uint16_t v[8]; };
 struct __attribute__((packed, aligned(4))) ReinU32x8 { uint32_t v[8]; };
@@ -56,164 +74,258 @@ __device__ __forceinline__ int rein_sub_bytes(uint32_t x, uint32_t c4)
 }
 
 // Weight side of one superblock chunk (8 sub-blocks) for lane (row, half h).
-//   fetch()   raw plane words HBM/L2 -> registers (so the next chunk can be in
-//             flight while this one is multiplied)
-//   expand()  raw -> b[s]: int8 operand (quants 16h..16h+15 of sub-block s, offsets
-//             folded), sc[u]: fp32 scale feeding the outer-product MFMA, mn[u]:
-//             negated min term
+// The 16-byte-per-sub-block plane (nibbles; Q8_0: the lane half's quant plane) is
+// kept apart from the small words (aux bits, scales, fp16 pair), because the tuned
+// kernel moves the former through LDS and only the latter through registers:
+//   Small / fetch_small()  aux + scale words HBM/L2 -> registers
+//   prepare()   Small -> sc[u]: fp32 scale feeding the outer-product MFMA; Q4_K/Q5_K
+//               also mb: the eight 6-bit mins as bf16 and ndmin = -dmin
+//   operand()   16 plane bytes of sub-block s -> int8 MFMA operand (quants
+//               16h..16h+15, offsets folded)
+//   plane()     which 16-byte plane this lane half reads
 // One-scale formats: u = pair index p, value for sub-block 2p+h.
 // Q6_K: u = s, value = d*sc_h for this lane's 16-weight half.
+// The plain kernels use Raw / fetch() / expand(): everything through registers.
 template <int FMT> struct MmqChunk;
 
 __device__ __forceinline__ unsigned rein_clamp_sb(unsigned sb, unsigned n_sub) { return sb < n_sub ? sb : n_sub - 1; }
 
-template <> struct MmqChunk<REIN_Q4_K> {
-    static constexpr bool kTwoScales = false, kHasMin = true;
-    struct Raw { uint4 q[8]; ReinU16x8 sm; uint32_t dd; };
+template <int FMT, class Self> struct MmqChunkBase {
     rein_v4i b[8];
-    float sc[4], mn[4];
-    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q4_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
+    template <class Raw>
+    __device__ __forceinline__ void expand(const Raw& r, unsigned sb0, unsigned n_sub, unsigned h)
     {
-        const size_t i = (size_t)row * f.nsp + sb0;      // K-quants: n_sub % 8 == 0, the whole chunk is valid
+        Self& self = *static_cast<Self*>(this);
+        self.prepare(r.sm, sb0, n_sub, h);
 #pragma unroll
-        for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
-        r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
-        r.dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
-    }
-    __device__ __forceinline__ void expand(const Raw& r, unsigned, unsigned, unsigned h)
-    {
-        const float d = rein_h2f((uint16_t)(r.dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(r.dd >> 16));
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[s][j] = (int)((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
-        }
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const uint16_t v = h ? r.sm.v[2 * p + 1] : r.sm.v[2 * p];
-            sc[p] = d * (float)(v & 0xFFu);
-            mn[p] = -(dmin * (float)(v >> 8));
-        }
+        for (int s = 0; s < 8; s++) b[s] = Self::operand(r.q[s], r.sm, s, h);
     }
 };
 
-template <> struct MmqChunk<REIN_Q5_K> {
+template <> struct MmqChunk<REIN_Q4_K> : MmqChunkBase<REIN_Q4_K, MmqChunk<REIN_Q4_K>> {
     static constexpr bool kTwoScales = false, kHasMin = true;
-    struct Raw { uint4 q[8]; ReinU32x8 qh; ReinU16x8 sm; uint32_t dd; };
-    rein_v4i b[8];
-    float sc[4], mn[4];
-    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q5_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
+    struct Small { ReinU16x8 sm; uint32_t dd; };
+    struct Raw { uint4 q[8]; Small sm; };
+    float sc[4], ndmin;
+    rein_v8bf mb;
+    static __device__ __forceinline__ const uint4* plane(const Fmt<REIN_Q4_K>& f, unsigned) { return f.nib; }
+    static __device__ __forceinline__ void fetch_small(Small& r, const Fmt<REIN_Q4_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
+    {
+        const size_t i = (size_t)row * f.nsp + sb0;      // K-quants: n_sub % 8 == 0, the whole chunk is valid
+        r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
+        r.dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
+    }
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q4_K>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
     {
         const size_t i = (size_t)row * f.nsp + sb0;
 #pragma unroll
         for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
+        fetch_small(r.sm, f, row, sb0, n_sub, h);
+    }
+    __device__ __forceinline__ void prepare(const Small& r, unsigned, unsigned, unsigned h)
+    {
+        const float d = rein_h2f((uint16_t)(r.dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(r.dd >> 16));
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint16_t v = h ? r.sm.v[2 * p + 1] : r.sm.v[2 * p];
+            sc[p] = d * (float)(v & 0xFFu);
+        }
+        uint4 m4;                                   // the eight 6-bit mins as bf16, sub-block order
+        m4.x = rein_bf16_of_u8(r.sm.v[0] >> 8) | (rein_bf16_of_u8(r.sm.v[1] >> 8) << 16);
+        m4.y = rein_bf16_of_u8(r.sm.v[2] >> 8) | (rein_bf16_of_u8(r.sm.v[3] >> 8) << 16);
+        m4.z = rein_bf16_of_u8(r.sm.v[4] >> 8) | (rein_bf16_of_u8(r.sm.v[5] >> 8) << 16);
+        m4.w = rein_bf16_of_u8(r.sm.v[6] >> 8) | (rein_bf16_of_u8(r.sm.v[7] >> 8) << 16);
+        mb = __builtin_bit_cast(rein_v8bf, m4);
+        ndmin = -dmin;
+    }
+    static __device__ __forceinline__ rein_v4i operand(const uint4& q, const Small&, int, unsigned h)
+    {
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        rein_v4i o;
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[j] = (int)((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
+        return o;
+    }
+    // next sub-block pair to the front (the rolled loop of the tuned kernel only
+    // ever indexes entries 0 and 1)
+    __device__ __forceinline__ void rotate(Small&) { sc[0] = sc[1]; sc[1] = sc[2]; sc[2] = sc[3]; }
+};
+
+template <> struct MmqChunk<REIN_Q5_K> : MmqChunkBase<REIN_Q5_K, MmqChunk<REIN_Q5_K>> {
+    static constexpr bool kTwoScales = false, kHasMin = true;
+    struct Small { ReinU32x8 qh; ReinU16x8 sm; uint32_t dd; };
+    struct Raw { uint4 q[8]; Small sm; };
+    float sc[4], ndmin;
+    rein_v8bf mb;
+    static __device__ __forceinline__ const uint4* plane(const Fmt<REIN_Q5_K>& f, unsigned) { return f.nib; }
+    static __device__ __forceinline__ void fetch_small(Small& r, const Fmt<REIN_Q5_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
+    {
+        const size_t i = (size_t)row * f.nsp + sb0;
         r.qh = *reinterpret_cast<const ReinU32x8*>(f.qhp + i);
         r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
         r.dd = f.ddp[(size_t)row * f.n_super + (sb0 >> 3)];
     }
-    __device__ __forceinline__ void expand(const Raw& r, unsigned, unsigned, unsigned h)
-    {
-        const float d = rein_h2f((uint16_t)(r.dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(r.dd >> 16));
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                b[s][j] = (int)(((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | (rein_spread4(r.qh.v[s] >> (8 * j + 4 * h)) << 4));
-        }
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const uint16_t v = h ? r.sm.v[2 * p + 1] : r.sm.v[2 * p];
-            sc[p] = d * (float)(v & 0xFFu);
-            mn[p] = -(dmin * (float)(v >> 8));
-        }
-    }
-};
-
-template <> struct MmqChunk<REIN_Q6_K> {
-    static constexpr bool kTwoScales = true, kHasMin = false;
-    struct Raw { uint4 q[8]; ReinU64x8 h2; ReinU16x8 sm; uint16_t d; };
-    rein_v4i b[8];
-    float sc[8];
-    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q6_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q5_K>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
     {
         const size_t i = (size_t)row * f.nsp + sb0;
 #pragma unroll
         for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
+        fetch_small(r.sm, f, row, sb0, n_sub, h);
+    }
+    __device__ __forceinline__ void prepare(const Small& r, unsigned, unsigned, unsigned h)
+    {
+        const float d = rein_h2f((uint16_t)(r.dd & 0xFFFFu)), dmin = rein_h2f((uint16_t)(r.dd >> 16));
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint16_t v = h ? r.sm.v[2 * p + 1] : r.sm.v[2 * p];
+            sc[p] = d * (float)(v & 0xFFu);
+        }
+        uint4 m4;
+        m4.x = rein_bf16_of_u8(r.sm.v[0] >> 8) | (rein_bf16_of_u8(r.sm.v[1] >> 8) << 16);
+        m4.y = rein_bf16_of_u8(r.sm.v[2] >> 8) | (rein_bf16_of_u8(r.sm.v[3] >> 8) << 16);
+        m4.z = rein_bf16_of_u8(r.sm.v[4] >> 8) | (rein_bf16_of_u8(r.sm.v[5] >> 8) << 16);
+        m4.w = rein_bf16_of_u8(r.sm.v[6] >> 8) | (rein_bf16_of_u8(r.sm.v[7] >> 8) << 16);
+        mb = __builtin_bit_cast(rein_v8bf, m4);
+        ndmin = -dmin;
+    }
+    static __device__ __forceinline__ rein_v4i operand(const uint4& q, const Small& r, int s, unsigned h)
+    {
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        rein_v4i o;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            o[j] = (int)(((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | (rein_spread4(r.qh.v[s] >> (8 * j + 4 * h)) << 4));
+        return o;
+    }
+    __device__ __forceinline__ void rotate(Small& r)
+    {
+        sc[0] = sc[1]; sc[1] = sc[2]; sc[2] = sc[3];
+#pragma unroll
+        for (int i = 0; i < 6; i++) r.qh.v[i] = r.qh.v[i + 2];
+    }
+};
+
+template <> struct MmqChunk<REIN_Q6_K> : MmqChunkBase<REIN_Q6_K, MmqChunk<REIN_Q6_K>> {
+    static constexpr bool kTwoScales = true, kHasMin = false;
+    struct Small { ReinU64x8 h2; ReinU16x8 sm; uint16_t d; };
+    struct Raw { uint4 q[8]; Small sm; };
+    float sc[8];
+    static __device__ __forceinline__ const uint4* plane(const Fmt<REIN_Q6_K>& f, unsigned) { return f.nib; }
+    static __device__ __forceinline__ void fetch_small(Small& r, const Fmt<REIN_Q6_K>& f, unsigned row, unsigned sb0, unsigned, unsigned)
+    {
+        const size_t i = (size_t)row * f.nsp + sb0;
         r.h2 = *reinterpret_cast<const ReinU64x8*>(f.h2p + i);
         r.sm = *reinterpret_cast<const ReinU16x8*>(f.smp + i);
         r.d  = f.dp[(size_t)row * f.n_super + (sb0 >> 3)];
     }
-    __device__ __forceinline__ void expand(const Raw& r, unsigned, unsigned, unsigned h)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q6_K>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    {
+        const size_t i = (size_t)row * f.nsp + sb0;
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = f.nib[i + s];
+        fetch_small(r.sm, f, row, sb0, n_sub, h);
+    }
+    __device__ __forceinline__ void prepare(const Small& r, unsigned, unsigned, unsigned h)
     {
         const float d = rein_h2f(r.d);
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                // hi2 byte 2j+h holds the 2-bit fields of this half's word j
-                const uint32_t hw = j < 2 ? r.h2.v[s].x : r.h2.v[s].y;
-                const uint32_t hb = (hw >> (16 * (j & 1) + 8 * h)) & 0xFFu;
-                const uint32_t q6 = ((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | rein_spread2(hb);
-                b[s][j] = rein_sub_bytes(q6, 0x20202020u);
-            }
             const uint16_t v = r.sm.v[s];
             sc[s] = d * (float)(int)(int8_t)(h ? (v >> 8) : (v & 0xFFu));
         }
+    }
+    static __device__ __forceinline__ rein_v4i operand(const uint4& q, const Small& r, int s, unsigned h)
+    {
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        rein_v4i o;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            // hi2 byte 2j+h holds the 2-bit fields of this half's word j
+            const uint32_t hw = j < 2 ? r.h2.v[s].x : r.h2.v[s].y;
+            const uint32_t hb = (hw >> (16 * (j & 1) + 8 * h)) & 0xFFu;
+            const uint32_t q6 = ((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | rein_spread2(hb);
+            o[j] = rein_sub_bytes(q6, 0x20202020u);
+        }
+        return o;
+    }
+    __device__ __forceinline__ void rotate(Small& r)
+    {
+#pragma unroll
+        for (int i = 0; i < 6; i++) { sc[i] = sc[i + 2]; r.h2.v[i] = r.h2.v[i + 2]; }
     }
 };
 
 // Q8_0 / Q4_0 / IQ4_XS: one fp16 scale per sub-block, the chunk may be ragged
 // (in_dim is only a multiple of 32): sub-blocks past the end are clamped and
 // their scale is forced to zero.
-template <int FMT> struct MmqChunkD16 {
+template <int FMT> struct MmqChunkD16 : MmqChunkBase<FMT, MmqChunk<FMT>> {
     static constexpr bool kTwoScales = false, kHasMin = false;
-    struct Raw { uint4 q[8]; uint16_t d[4]; };
-    rein_v4i b[8];
-    float sc[4], mn[4];
-    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<FMT>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    struct Small { uint16_t d[4]; };
+    struct Raw { uint4 q[8]; Small sm; };
+    float sc[4];
+    static __device__ __forceinline__ const uint4* plane(const Fmt<FMT>& f, unsigned h)
     {
-        const uint4* plane;
-        if constexpr (FMT == REIN_Q8_0) plane = h ? f.hip_ : f.lop;     // this lane's 16 quants are one plane entry
-        else plane = f.nib;
-#pragma unroll
-        for (int s = 0; s < 8; s++) r.q[s] = plane[(size_t)row * f.nsp + rein_clamp_sb(sb0 + s, n_sub)];
+        if constexpr (FMT == REIN_Q8_0) return h ? f.hip_ : f.lop;      // this lane's 16 quants are one plane entry
+        else return f.nib;
+    }
+    static __device__ __forceinline__ void fetch_small(Small& r, const Fmt<FMT>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    {
 #pragma unroll
         for (int p = 0; p < 4; p++) r.d[p] = f.dp[(size_t)row * f.nsp + rein_clamp_sb(sb0 + 2 * p + h, n_sub)];
     }
-    __device__ __forceinline__ void expand(const Raw& r, unsigned sb0, unsigned n_sub, unsigned h)
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<FMT>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    {
+        const uint4* pl = plane(f, h);
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = pl[(size_t)row * f.nsp + rein_clamp_sb(sb0 + s, n_sub)];
+        fetch_small(r.sm, f, row, sb0, n_sub, h);
+    }
+    __device__ __forceinline__ void prepare(const Small& r, unsigned sb0, unsigned n_sub, unsigned h)
     {
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const uint32_t w[4] = {r.q[s].x, r.q[s].y, r.q[s].z, r.q[s].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if constexpr (FMT == REIN_Q8_0) b[s][j] = (int)w[j];
-                else if constexpr (FMT == REIN_Q4_0) b[s][j] = rein_sub_bytes((w[j] >> (4 * h)) & 0x0F0F0F0Fu, 0x08080808u);
-                else b[s][j] = rein_iq4_lut4((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
-            }
-        }
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            sc[p] = sb0 + 2 * p + h < n_sub ? rein_h2f(r.d[p]) : 0.0f;
-            mn[p] = 0.0f;
-        }
+        for (int p = 0; p < 4; p++) sc[p] = sb0 + 2 * p + h < n_sub ? rein_h2f(r.d[p]) : 0.0f;
     }
+    static __device__ __forceinline__ rein_v4i operand(const uint4& q, const Small&, int, unsigned h)
+    {
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        rein_v4i o;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if constexpr (FMT == REIN_Q8_0) o[j] = (int)w[j];
+            else if constexpr (FMT == REIN_Q4_0) o[j] = rein_sub_bytes((w[j] >> (4 * h)) & 0x0F0F0F0Fu, 0x08080808u);
+            else o[j] = rein_iq4_lut4((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
+        }
+        return o;
+    }
+    __device__ __forceinline__ void rotate(Small&) { sc[0] = sc[1]; sc[1] = sc[2]; sc[2] = sc[3]; }
 };
 template <> struct MmqChunk<REIN_Q8_0> : MmqChunkD16<REIN_Q8_0> {};
 template <> struct MmqChunk<REIN_Q4_0> : MmqChunkD16<REIN_Q4_0> {};
 template <> struct MmqChunk<REIN_IQ4_XS> : MmqChunkD16<REIN_IQ4_XS> {};
 
-// LDS image of one activation chunk: TM tokens x 8 sub-blocks.
+// LDS image of one activation chunk: TM tokens x 8 sub-blocks.  xsb holds each
+// block's xsum split into three bf16 (truncated head, then the exact remainders),
+// which together carry all 24 significand bits: the -dmin*m*xsum term of
+// Q4_K/Q5_K is then one superblock-wide bf16 MFMA against the integer mins with
+// exact products and fp32 accumulation.
 template <int TM>
 struct MmqLds {
     static constexpr int kPlane = TM + 1;                 // +1 entry: sub-block planes land on different banks
     uint4 qs[2][8][kPlane];                               // [half][sub-block][token]
     float dx[8][kPlane];
-    float xsum[8][kPlane];
+    uint16_t xsb[3][TM][8];                               // [split][token][sub-block]
 };
+
+__device__ __forceinline__ void rein_mmq_split_xsum(float xs, uint16_t out[3])
+{
+    const uint32_t b0 = __builtin_bit_cast(uint32_t, xs) & 0xFFFF0000u;
+    const float r1 = xs - __builtin_bit_cast(float, b0);
+    const uint32_t b1 = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
+    const float r2 = r1 - __builtin_bit_cast(float, b1);
+    out[0] = (uint16_t)(b0 >> 16);
+    out[1] = (uint16_t)(b1 >> 16);
+    out[2] = (uint16_t)(__builtin_bit_cast(uint32_t, r2) >> 16);
+}
 
 // Stage xq rows tok_base .. tok_base+TM (rows >= tok_end are zero-scaled) for
 // sub-blocks sb0..sb0+8 into LDS, all threads of the workgroup.
@@ -234,7 +346,125 @@ __device__ __forceinline__ void rein_mmq_stage(MmqLds<TM>& l, const BlockQ8* __r
         l.qs[0][s][tl] = lo;
         l.qs[1][s][tl] = hi;
         l.dx[s][tl]   = ok ? d : 0.0f;
-        l.xsum[s][tl] = ok ? xs : 0.0f;
+        uint16_t sp[3];
+        rein_mmq_split_xsum(ok ? xs : 0.0f, sp);
+        l.xsb[0][tl][s] = sp[0];
+        l.xsb[1][tl][s] = sp[1];
+        l.xsb[2][tl][s] = sp[2];
+    }
+}
+
+// Multiply one staged chunk (8 sub-blocks) into the accumulators of this
+// wavefront's TM/32 tiles.  DOTS != 0: store the raw int32 block dots instead.
+template <int FMT, int TM, int DOTS, class BSrc>
+__device__ __forceinline__ void rein_mmq_chunk_math(const MmqLds<TM>& lds, const MmqChunk<FMT>& ck, const BSrc& bsrc,
+                                                    rein_v16f (&acc)[TM / 32], unsigned j, unsigned h,
+                                                    int* __restrict__ dots, unsigned row, unsigned out_dim,
+                                                    unsigned tok_base, unsigned tok_end, unsigned sb0, unsigned n_sub)
+{
+    using C = MmqChunk<FMT>;
+    constexpr int NT = TM / 32;
+    rein_v16i cinit;
+#pragma unroll
+    for (int v = 0; v < 16; v++) cinit[v] = DOTS ? 0 : REIN_MMQ_MAGIC_I;
+    rein_v32f z32;
+#pragma unroll
+    for (int v = 0; v < 32; v++) z32[v] = 0.0f;
+
+    if constexpr (C::kTwoScales) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const rein_v4i bs = bsrc(s);
+            rein_v4i blo, bhi;
+#pragma unroll
+            for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : bs[k]; bhi[k] = h ? bs[k] : 0; }
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 a4 = lds.qs[h][s][t * 32 + j];
+                rein_v4i a;
+                a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
+                const rein_v16i clo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, cinit, 0, 0, 0);
+                const rein_v16i chi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, cinit, 0, 0, 0);
+                if constexpr (DOTS != 0) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const unsigned tok = tok_base + t * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+                        if (tok < tok_end && row < out_dim && sb0 + s < n_sub) {
+                            int* o = dots + (((size_t)tok * out_dim + row) * n_sub + sb0 + s) * 2;
+                            o[0] = clo[v];
+                            o[1] = chi[v];
+                        }
+                    }
+                } else {
+                    // block 0 (lanes 0-31 of both operands): dx * dsc_lo, block 1: dx * dsc_hi
+                    const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
+                    const rein_v16f flo = rein_mmq_unbias(clo), fhi = rein_mmq_unbias(chi);
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        acc[t][v] = fmaf(flo[v], sx[v], acc[t][v]);
+                        acc[t][v] = fmaf(fhi[v], sx[16 + v], acc[t][v]);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const rein_v4i b0 = bsrc(2 * p), b1 = bsrc(2 * p + 1);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 a40 = lds.qs[h][2 * p][t * 32 + j];
+                const uint4 a41 = lds.qs[h][2 * p + 1][t * 32 + j];
+                rein_v4i a0, a1;
+                a0[0] = (int)a40.x; a0[1] = (int)a40.y; a0[2] = (int)a40.z; a0[3] = (int)a40.w;
+                a1[0] = (int)a41.x; a1[1] = (int)a41.y; a1[2] = (int)a41.z; a1[3] = (int)a41.w;
+                const rein_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0, cinit, 0, 0, 0);
+                const rein_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1, cinit, 0, 0, 0);
+                if constexpr (DOTS != 0) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const unsigned tok = tok_base + t * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+                        if (tok < tok_end && row < out_dim) {
+                            int* o = dots + ((size_t)tok * out_dim + row) * n_sub + sb0 + 2 * p;
+                            if (sb0 + 2 * p < n_sub) o[0] = c0[v];
+                            if (sb0 + 2 * p + 1 < n_sub) o[1] = c1[v];
+                        }
+                    }
+                } else {
+                    // lane half h feeds sub-block 2p+h: block 0 = sub-block 2p, block 1 = 2p+1
+                    const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[p], z32, 0, 0, 0);
+                    const rein_v16f f0 = rein_mmq_unbias(c0), f1 = rein_mmq_unbias(c1);
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        acc[t][v] = fmaf(f0[v], sx[v], acc[t][v]);
+                        acc[t][v] = fmaf(f1[v], sx[16 + v], acc[t][v]);
+                    }
+                }
+            }
+            // keep the pairs apart: interleaving them buys nothing (MFMA and VALU of
+            // a SIMD do not overlap) and costs a second set of 96 live registers
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (C::kHasMin && DOTS == 0) {
+            // sum over the 8 sub-blocks of m * xsum: lane half 0 carries the heads of
+            // the xsum splits, half 1 the first remainders, a second MFMA the last
+            // remainders (its half 1 multiplies zeros)
+            const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
+            const rein_v8bf mb2 = h ? __builtin_bit_cast(rein_v8bf, z4) : ck.mb;
+            rein_v16f z16;
+#pragma unroll
+            for (int v = 0; v < 16; v++) z16[v] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 x01 = *reinterpret_cast<const uint4*>(lds.xsb[h][t * 32 + j]);
+                const uint4 x2  = *reinterpret_cast<const uint4*>(lds.xsb[2][t * 32 + j]);
+                rein_v16f m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x01), ck.mb, z16, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x2), mb2, m, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[t][v] = fmaf(m[v], ck.ndmin, acc[t][v]);
+            }
+        }
     }
 }
 
@@ -275,89 +505,8 @@ __device__ __forceinline__ void rein_mmq_tile(const uint8_t* __restrict__ w, con
         __syncthreads();                           // previous chunk's LDS reads are done
         rein_mmq_stage<TM>(lds, xq, n_sub, tok_base, tok_end, sb0);
         __syncthreads();
-
-        if constexpr (C::kTwoScales) {
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                rein_v4i blo, bhi;
-#pragma unroll
-                for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : ck.b[s][k]; bhi[k] = h ? ck.b[s][k] : 0; }
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const uint4 a4 = lds.qs[h][s][t * 32 + j];
-                    rein_v4i a;
-                    a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
-                    rein_v16i z;
-#pragma unroll
-                    for (int v = 0; v < 16; v++) z[v] = 0;
-                    const rein_v16i clo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, z, 0, 0, 0);
-                    const rein_v16i chi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, z, 0, 0, 0);
-                    if (DOTS) {
-#pragma unroll
-                        for (int v = 0; v < 16; v++) {
-                            const unsigned tok = tok_base + t * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-                            if (tok < tok_end && row < out_dim && sb0 + s < n_sub) {
-                                int* o = dots + (((size_t)tok * out_dim + row) * n_sub + sb0 + s) * 2;
-                                o[0] = clo[v];
-                                o[1] = chi[v];
-                            }
-                        }
-                    } else {
-                        rein_v32f z32;
-#pragma unroll
-                        for (int v = 0; v < 32; v++) z32[v] = 0.0f;
-                        // block 0 (lanes 0-31 of both operands): dx * dsc_lo, block 1: dx * dsc_hi
-                        const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
-#pragma unroll
-                        for (int v = 0; v < 16; v++) {
-                            acc[t][v] = fmaf((float)clo[v], sx[v], acc[t][v]);
-                            acc[t][v] = fmaf((float)chi[v], sx[16 + v], acc[t][v]);
-                        }
-                    }
-                }
-            }
-        } else {
-#pragma unroll
-            for (int p = 0; p < 4; p++) {
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const uint4 a40 = lds.qs[h][2 * p][t * 32 + j];
-                    const uint4 a41 = lds.qs[h][2 * p + 1][t * 32 + j];
-                    rein_v4i a0, a1;
-                    a0[0] = (int)a40.x; a0[1] = (int)a40.y; a0[2] = (int)a40.z; a0[3] = (int)a40.w;
-                    a1[0] = (int)a41.x; a1[1] = (int)a41.y; a1[2] = (int)a41.z; a1[3] = (int)a41.w;
-                    rein_v16i z;
-#pragma unroll
-                    for (int v = 0; v < 16; v++) z[v] = 0;
-                    const rein_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, ck.b[2 * p], z, 0, 0, 0);
-                    const rein_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, ck.b[2 * p + 1], z, 0, 0, 0);
-                    if (DOTS) {
-#pragma unroll
-                        for (int v = 0; v < 16; v++) {
-                            const unsigned tok = tok_base + t * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-                            if (tok < tok_end && row < out_dim) {
-                                int* o = dots + ((size_t)tok * out_dim + row) * n_sub + sb0 + 2 * p;
-                                if (sb0 + 2 * p < n_sub) o[0] = c0[v];
-                                if (sb0 + 2 * p + 1 < n_sub) o[1] = c1[v];
-                            }
-                        }
-                    } else {
-                        rein_v32f z32;
-#pragma unroll
-                        for (int v = 0; v < 32; v++) z32[v] = 0.0f;
-                        // lane half h feeds sub-block 2p+h: block 0 = sub-block 2p, block 1 = 2p+1
-                        const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[p], z32, 0, 0, 0);
-                        if constexpr (C::kHasMin)
-                            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(lds.xsum[2 * p + h][t * 32 + j], ck.mn[p], acc[t], 0, 0, 0);
-#pragma unroll
-                        for (int v = 0; v < 16; v++) {
-                            acc[t][v] = fmaf((float)c0[v], sx[v], acc[t][v]);
-                            acc[t][v] = fmaf((float)c1[v], sx[16 + v], acc[t][v]);
-                        }
-                    }
-                }
-            }
-        }
+        rein_mmq_chunk_math<FMT, TM, DOTS>(lds, ck, [&](int s) { return ck.b[s]; }, acc, j, h, dots, row, out_dim,
+                                           tok_base, tok_end, sb0, n_sub);
     }
 
     if (!DOTS) {
@@ -374,9 +523,13 @@ __device__ __forceinline__ void rein_mmq_tile(const uint8_t* __restrict__ w, con
 // ---------------------------------------------------------------------------
 // Pipelined dense MMQ (the tuned launch).  Same math and layouts as
 // rein_mmq_tile, plus:
-//   * the next chunk's weight words and activation blocks are fetched into
-//     registers before the current chunk is multiplied, the LDS image is
-//     double-buffered, and there is one barrier per chunk;
+//   * the 16-byte weight plane travels HBM -> LDS directly
+//     (global_load_lds_dwordx4, no registers), each wavefront into its own ring
+//     of two half-chunk slots, so it needs no barrier; a slot is refilled with
+//     the next chunk's half as soon as it has been read;
+//   * the next chunk's small weight words and activation blocks are fetched into
+//     registers before the current chunk is multiplied, the activation LDS image
+//     is double-buffered, and there is one barrier per chunk;
 //   * a fixed workgroup of 4 wavefronts (128 rows x TM tokens);
 //   * a 1-D grid whose workgroup -> tile map keeps all token tiles of one
 //     128-row weight block on the same XCD (workgroups are dealt round-robin
@@ -423,48 +576,133 @@ __device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM
         l.qs[0][s][tl] = r.lo[k];
         l.qs[1][s][tl] = r.hi[k];
         l.dx[s][tl]    = ok ? __builtin_bit_cast(float, r.hdr[k].x) : 0.0f;
-        l.xsum[s][tl]  = ok ? __builtin_bit_cast(float, r.hdr[k].y) : 0.0f;
+        uint16_t sp[3];
+        rein_mmq_split_xsum(ok ? __builtin_bit_cast(float, r.hdr[k].y) : 0.0f, sp);
+        l.xsb[0][tl][s] = sp[0];
+        l.xsb[1][tl][s] = sp[1];
+        l.xsb[2][tl][s] = sp[2];
     }
 }
 
-// multiply one staged chunk into the accumulators
-template <int FMT, int TM>
-__device__ __forceinline__ void rein_mmq_chunk_math(const MmqLds<TM>& lds, const MmqChunk<FMT>& ck,
-                                                    rein_v16f (&acc)[TM / 32], unsigned j, unsigned h)
+// One wavefront's LDS ring for the 16-byte weight plane(s): two slots of half a
+// chunk (32 rows x 4 sub-blocks, 2 KiB) each.  Slot entry of (row n, sub-block
+// s4 of the half) is 4n + ((s4 + n/2) & 3), which spreads the 32 rows of a
+// ds_read_b128 over all banks.  Q8_0 has one plane per lane half.
+template <int FMT>
+struct MmqWLds {
+    static constexpr int kPlanes = FMT == REIN_Q8_0 ? 2 : 1;
+    uint4 q[kPlanes][2][128];
+};
+
+// One 16-byte-per-lane HBM -> LDS transfer: lane l's bytes land at lds_base + 16 l
+// (lds_base wave-uniform, passed in M0).  Written as inline assembly on purpose:
+// through the builtin the compiler treats every later LDS read as a possible reader
+// of the transfer and waits for it on the spot (s_waitcnt vmcnt(0)), which turns the
+// prefetch into a blocking load.  Here the waits are placed by hand with
+// REIN_WAIT_VMCNT.  The compiler's own vmcnt waits stay correct: requests complete in
+// order and it can only under-count the younger ones, i.e. wait for more.
+__device__ __forceinline__ void rein_lds_dma16(const void* gptr, unsigned lds_base)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+// HBM -> LDS, asynchronous (counted by vmcnt), sub-blocks sb_first .. sb_first+3 of
+// rows row_base .. row_base+31 into slot `half`.  Lane l of load k covers row
+// 16k + l/4 (four lanes walk the row's 64 contiguous bytes).  2 * kPlanes loads.
+template <int FMT>
+__device__ __forceinline__ void rein_mmq_wload(MmqWLds<FMT>& dst, unsigned half, const Fmt<FMT>& fmt,
+                                               unsigned row_base, unsigned out_dim, unsigned sb_first, unsigned n_sub,
+                                               unsigned lane)
+{
+    typedef __attribute__((address_space(3))) void* lptr_t;
+#pragma unroll
+    for (int pl = 0; pl < MmqWLds<FMT>::kPlanes; pl++) {
+        const uint4* plane = MmqChunk<FMT>::plane(fmt, (unsigned)pl);
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const unsigned n = 16u * k + (lane >> 2);
+            const unsigned s4 = ((lane & 3u) - (n >> 1)) & 3u;
+            const unsigned row = min(row_base + n, out_dim - 1u);
+            const unsigned sb = rein_clamp_sb(sb_first + s4, n_sub);
+            const unsigned lds_base =
+                __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)&dst.q[pl][half][64 * k]);
+            rein_lds_dma16(plane + (size_t)row * fmt.nsp + sb, lds_base);
+        }
+    }
+}
+
+// s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding)
+#define REIN_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
+
+// The chunk math of the tuned kernel: one rolled iteration per sub-block pair so
+// that only one pair's tiles (two int32 dot tiles, one 2-block scale tile) are
+// live at a time.  Pairs 0,1 read ring slot 0 and pairs 2,3 slot 1; as soon as a
+// slot has been read, the same half of the NEXT chunk is requested into it
+// (`more`), so a weight request is in flight for about three quarters of a chunk.
+// `refill(half)` is the caller's: it issues the loads (see rein_mmq_pipelined for the
+// order that keeps every wait off the freshest requests).
+// `ck` and `sm` are private copies; they are rotated so the loop indexes entries
+// 0 and 1.
+template <int FMT, int TM, class Refill>
+__device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds, MmqWLds<FMT>& wl, unsigned wsel,
+                                                           MmqChunk<FMT> ck, typename MmqChunk<FMT>::Small sm,
+                                                           rein_v16f (&acc)[TM / 32], unsigned j, unsigned h,
+                                                           bool more, const Refill& refill)
 {
     using C = MmqChunk<FMT>;
     constexpr int NT = TM / 32;
-    rein_v16i z;
+    constexpr int kDma = 2 * MmqWLds<FMT>::kPlanes;
+    rein_v16i cinit;
 #pragma unroll
-    for (int v = 0; v < 16; v++) z[v] = 0;
+    for (int v = 0; v < 16; v++) cinit[v] = REIN_MMQ_MAGIC_I;
     rein_v32f z32;
 #pragma unroll
     for (int v = 0; v < 32; v++) z32[v] = 0.0f;
+    const unsigned rot = j >> 1;
 
-    if constexpr (C::kTwoScales) {
+#pragma unroll 1
+    for (unsigned p = 0; p < 4; p++) {
+        if (p == 2) {
+            // slot 1 of this chunk: only the refill of slot 0 (if any) is younger
+            if (more) REIN_WAIT_VMCNT(kDma); else REIN_WAIT_VMCNT(0);
+        }
+        const uint4* slot = wl.q[wsel][p >> 1];
+        const unsigned s4 = 2u * (p & 1u);
+        const rein_v4i b0 = C::operand(slot[4u * j + ((s4 + rot) & 3u)], sm, 0, h);
+        const rein_v4i b1 = C::operand(slot[4u * j + ((s4 + 1u + rot) & 3u)], sm, 1, h);
+        if (more && (p & 1u)) {
+            // both pairs of the slot are in registers: refill it.  The LDS reads above
+            // must have returned before the DMA may overwrite the slot.
+            __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0)
+            refill(p >> 1);
+        }
+        if constexpr (C::kTwoScales) {
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            rein_v4i blo, bhi;
+            for (int s = 0; s < 2; s++) {
+                const rein_v4i bs = s ? b1 : b0;
+                rein_v4i blo, bhi;
 #pragma unroll
-            for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : ck.b[s][k]; bhi[k] = h ? ck.b[s][k] : 0; }
+                for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : bs[k]; bhi[k] = h ? bs[k] : 0; }
 #pragma unroll
-            for (int t = 0; t < NT; t++) {
-                const uint4 a4 = lds.qs[h][s][t * 32 + j];
-                rein_v4i a;
-                a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
-                const rein_v16i clo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, z, 0, 0, 0);
-                const rein_v16i chi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, z, 0, 0, 0);
-                const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
+                for (int t = 0; t < NT; t++) {
+                    const uint4 a4 = lds.qs[h][2 * p + s][t * 32 + j];
+                    rein_v4i a;
+                    a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
+                    const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
+                    const rein_v16i clo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, cinit, 0, 0, 0);
+                    const rein_v16f flo = rein_mmq_unbias(clo);
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    acc[t][v] = fmaf((float)clo[v], sx[v], acc[t][v]);
-                    acc[t][v] = fmaf((float)chi[v], sx[16 + v], acc[t][v]);
+                    for (int v = 0; v < 16; v++) acc[t][v] = fmaf(flo[v], sx[v], acc[t][v]);
+                    const rein_v16i chi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, cinit, 0, 0, 0);
+                    const rein_v16f fhi = rein_mmq_unbias(chi);
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[t][v] = fmaf(fhi[v], sx[16 + v], acc[t][v]);
                 }
             }
-        }
-    } else {
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
+        } else {
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const uint4 a40 = lds.qs[h][2 * p][t * 32 + j];
@@ -472,17 +710,33 @@ __device__ __forceinline__ void rein_mmq_chunk_math(const MmqLds<TM>& lds, const
                 rein_v4i a0, a1;
                 a0[0] = (int)a40.x; a0[1] = (int)a40.y; a0[2] = (int)a40.z; a0[3] = (int)a40.w;
                 a1[0] = (int)a41.x; a1[1] = (int)a41.y; a1[2] = (int)a41.z; a1[3] = (int)a41.w;
-                const rein_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, ck.b[2 * p], z, 0, 0, 0);
-                const rein_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, ck.b[2 * p + 1], z, 0, 0, 0);
-                const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[p], z32, 0, 0, 0);
-                if constexpr (C::kHasMin)
-                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(lds.xsum[2 * p + h][t * 32 + j], ck.mn[p], acc[t], 0, 0, 0);
+                const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[0], z32, 0, 0, 0);
+                const rein_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0, cinit, 0, 0, 0);
+                const rein_v16f f0 = rein_mmq_unbias(c0);
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    acc[t][v] = fmaf((float)c0[v], sx[v], acc[t][v]);
-                    acc[t][v] = fmaf((float)c1[v], sx[16 + v], acc[t][v]);
-                }
+                for (int v = 0; v < 16; v++) acc[t][v] = fmaf(f0[v], sx[v], acc[t][v]);
+                const rein_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1, cinit, 0, 0, 0);
+                const rein_v16f f1 = rein_mmq_unbias(c1);
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[t][v] = fmaf(f1[v], sx[16 + v], acc[t][v]);
             }
+        }
+        ck.rotate(sm);
+    }
+    if constexpr (C::kHasMin) {
+        const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
+        const rein_v8bf mb2 = h ? __builtin_bit_cast(rein_v8bf, z4) : ck.mb;
+        rein_v16f z16;
+#pragma unroll
+        for (int v = 0; v < 16; v++) z16[v] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const uint4 x01 = *reinterpret_cast<const uint4*>(lds.xsb[h][t * 32 + j]);
+            const uint4 x2  = *reinterpret_cast<const uint4*>(lds.xsb[2][t * 32 + j]);
+            rein_v16f m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x01), ck.mb, z16, 0, 0, 0);
+            m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x2), mb2, m, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[t][v] = fmaf(m[v], ck.ndmin, acc[t][v]);
         }
     }
 }
@@ -495,7 +749,9 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
     using F = Fmt<FMT>;
     using C = MmqChunk<FMT>;
     constexpr int NT = TM / 32;
+    constexpr int kDma = 2 * MmqWLds<FMT>::kPlanes;
     __shared__ MmqLds<TM> lds[2];
+    __shared__ MmqWLds<FMT> wlds[4];
 
     // workgroup -> (row block, token tile), XCD-aware
     const unsigned n_rb = (out_dim + 127u) / 128u;
@@ -508,10 +764,13 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
     const unsigned j = lane & 31u, h = lane >> 5;
     const unsigned n_sub = in_dim >> 5;
     const F fmt(w, n_sub, out_dim);
-    const unsigned row = rb * 128u + wave * 32u + j;
+    const unsigned row_base = rb * 128u + wave * 32u;
+    const unsigned row = row_base + j;
     const unsigned rowc = row < out_dim ? row : out_dim - 1;
     const unsigned tok_base = tt * TM;
     const unsigned tok_end = min(p_rows, tok_base + TM);
+    const unsigned wsel = FMT == REIN_Q8_0 ? h : 0u;
+    MmqWLds<FMT>& wl = wlds[wave];
 
     rein_v16f acc[NT];
 #pragma unroll
@@ -519,24 +778,46 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
 
-    typename C::Raw raw;
+    // Request order per chunk c.  Requests complete in order and vmcnt counts those in
+    // flight.  The ring DMA is invisible to the compiler's own bookkeeping, so its waits
+    // for the register loads can only be stronger than it thinks; the hand-placed waits
+    // only ever count ring requests, never the compiler's (whose number of instructions
+    // is its own business):
+    //   top of c        small words of c+1                                  (registers)
+    //   after pair 1    activation image of c+1 -> LDS (blocks fetched during c-1),
+    //                   activation blocks of c+2 (registers), then ring slot 0 <- c+1
+    //   before pair 2   wait until only the slot 0 refill is in flight (slot 1 of c is in)
+    //   after pair 3    ring slot 1 <- c+1
+    //   end of c        wait until only the slot 1 refill is in flight (slot 0 of c+1 is
+    //                   in), barrier
+    typename C::Small small;
     MmqXRegs<TM> xr;
-    C::fetch(raw, fmt, rowc, 0, n_sub, h);
+    C::fetch_small(small, fmt, rowc, 0, n_sub, h);
     rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 0);
     rein_mmq_xstore<TM>(lds[0], xr, n_sub, tok_base, tok_end, 0);
+    rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 8 < n_sub ? 8 : 0);
+    rein_mmq_wload<FMT>(wl, 0, fmt, row_base, out_dim, 0, n_sub, lane);
+    rein_mmq_wload<FMT>(wl, 1, fmt, row_base, out_dim, 4, n_sub, lane);
+    REIN_WAIT_VMCNT(kDma);                           // slot 0 of chunk 0 has landed
     __syncthreads();
 
     unsigned buf = 0;
     for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 8, buf ^= 1u) {
         C ck;
-        ck.expand(raw, sb0, n_sub, h);
-        const bool more = sb0 + 8 < n_sub;
-        if (more) {                                  // next chunk goes out before the math
-            C::fetch(raw, fmt, rowc, sb0 + 8, n_sub, h);
-            rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, sb0 + 8);
-        }
-        rein_mmq_chunk_math<FMT, TM>(lds[buf], ck, acc, j, h);
-        if (more) rein_mmq_xstore<TM>(lds[buf ^ 1u], xr, n_sub, tok_base, tok_end, sb0 + 8);
+        ck.prepare(small, sb0, n_sub, h);
+        const typename C::Small cur = small;
+        const bool more = sb0 + 8 < n_sub, more2 = sb0 + 16 < n_sub;
+        if (more) C::fetch_small(small, fmt, rowc, sb0 + 8, n_sub, h);
+        MmqLds<TM>& nxt = lds[buf ^ 1u];
+        rein_mmq_chunk_math_rolled<FMT, TM>(lds[buf], wl, wsel, ck, cur, acc, j, h, more, [&](unsigned half) {
+            if (half == 0) {
+                rein_mmq_xstore<TM>(nxt, xr, n_sub, tok_base, tok_end, sb0 + 8);
+                // past the last chunk the fetch repeats on clamped addresses and is never stored
+                rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, more2 ? sb0 + 16 : sb0 + 8);
+            }
+            rein_mmq_wload<FMT>(wl, half, fmt, row_base, out_dim, sb0 + 8 + 4 * half, n_sub, lane);
+        });
+        if (more) REIN_WAIT_VMCNT(kDma);             // slot 0 of the next chunk has landed
         __syncthreads();
     }
 
@@ -594,25 +875,29 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     }
 }
 
+// Two wavefronts per SIMD: a 256-register budget, which makes the compiler keep
+// MFMA results in ordinary VGPRs (no AGPR round trips) without spilling.
+#define REIN_MMQ_OCC __attribute__((amdgpu_waves_per_eu(2)))
+
 #define REIN_MMQ_ARGS                                                                            \
     const unsigned char* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y, \
         unsigned int in_dim, unsigned int out_dim, unsigned int p_rows
 
 #define REIN_DEFINE_MMQ(name, FMT, TM)                                                           \
-    extern "C" __global__ __launch_bounds__(256) void name(REIN_MMQ_ARGS)                        \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(REIN_MMQ_ARGS)                        \
     {                                                                                            \
         rein_mmq_dense<FMT, TM, 0>(w, xq, y, nullptr, in_dim, out_dim, p_rows);                  \
     }
 
 // tuned entry: fixed 256-thread workgroups, 1-D XCD-aware grid
 #define REIN_DEFINE_MMQ_PIPE(name, FMT, TM)                                                      \
-    extern "C" __global__ __launch_bounds__(256) void name(REIN_MMQ_ARGS)                        \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(REIN_MMQ_ARGS)                        \
     {                                                                                            \
         rein_mmq_pipelined<FMT, TM>(w, xq, y, in_dim, out_dim, p_rows);                          \
     }
 
 #define REIN_DEFINE_MMQ_DOTS(name, FMT)                                                          \
-    extern "C" __global__ __launch_bounds__(256) void name(                                      \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                         \
         const unsigned char* __restrict__ w, const BlockQ8* __restrict__ xq, int* __restrict__ out, \
         unsigned int in_dim, unsigned int out_dim, unsigned int p_rows)                          \
     {                                                                                            \
@@ -620,7 +905,7 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     }
 
 #define REIN_DEFINE_MMQ_GROUPED(name, FMT)                                                       \
-    extern "C" __global__ __launch_bounds__(256) void name(                                      \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                         \
         const unsigned char* __restrict__ slab, unsigned int bytes_per_expert,                   \
         const int* __restrict__ expert_off, const int* __restrict__ tile_off, unsigned int n_expert, \
         const BlockQ8* __restrict__ xq, float* __restrict__ y, unsigned int in_dim,              \

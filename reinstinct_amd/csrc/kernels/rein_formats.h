@@ -81,6 +81,23 @@ __device__ __forceinline__ int rein_iq4_lut4(uint32_t n4)
     return (int)((hi & m) | (lo & ~m));
 }
 
+// Streaming (nontemporal) loads for the matvec weight planes: every weight byte is
+// read exactly once per launch, so it should not displace the activations in L2.
+typedef uint32_t rein_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t rein_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 rein_ldw(const uint4* p)
+{
+    const rein_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const rein_u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 rein_ldw(const uint2* p)
+{
+    const rein_u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const rein_u32x2*>(p));
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t rein_ldw(const uint32_t* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ uint16_t rein_ldw(const uint16_t* p) { return __builtin_nontemporal_load(p); }
+
 template <int FMT> struct Fmt;
 
 // ------------------------------------------------------------------ Q4_K
@@ -104,9 +121,9 @@ template <> struct Fmt<REIN_Q4_K> {
     {
         const size_t i = (size_t)row * nsp + sb;
         Raw r;
-        r.q  = nib[i];
-        r.sm = smp[i];
-        r.dd = ddp[(size_t)row * n_super + (sb >> 3)];
+        r.q  = rein_ldw(&nib[i]);
+        r.sm = rein_ldw(&smp[i]);
+        r.dd = rein_ldw(&ddp[(size_t)row * n_super + (sb >> 3)]);
         return r;
     }
     static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)
@@ -152,10 +169,10 @@ template <> struct Fmt<REIN_Q5_K> {
     {
         const size_t i = (size_t)row * nsp + sb;
         Raw r;
-        r.q  = nib[i];
-        r.qh = qhp[i];
-        r.sm = smp[i];
-        r.dd = ddp[(size_t)row * n_super + (sb >> 3)];
+        r.q  = rein_ldw(&nib[i]);
+        r.qh = rein_ldw(&qhp[i]);
+        r.sm = rein_ldw(&smp[i]);
+        r.dd = rein_ldw(&ddp[(size_t)row * n_super + (sb >> 3)]);
         return r;
     }
     static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)
@@ -203,10 +220,10 @@ template <> struct Fmt<REIN_Q6_K> {
     {
         const size_t i = (size_t)row * nsp + sb;
         Raw r;
-        r.q  = nib[i];
-        r.h2 = h2p[i];
-        r.sm = smp[i];
-        r.d  = dp[(size_t)row * n_super + (sb >> 3)];
+        r.q  = rein_ldw(&nib[i]);
+        r.h2 = rein_ldw(&h2p[i]);
+        r.sm = rein_ldw(&smp[i]);
+        r.d  = rein_ldw(&dp[(size_t)row * n_super + (sb >> 3)]);
         return r;
     }
     static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)
@@ -259,9 +276,9 @@ template <> struct Fmt<REIN_Q8_0> {
     {
         const size_t i = (size_t)row * nsp + sb;
         Raw r;
-        r.lo = lop[i];
-        r.hi = hip_[i];
-        r.d  = dp[i];
+        r.lo = rein_ldw(&lop[i]);
+        r.hi = rein_ldw(&hip_[i]);
+        r.d  = rein_ldw(&dp[i]);
         return r;
     }
     static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)
@@ -298,8 +315,8 @@ template <> struct Fmt<REIN_Q4_0> {
     {
         const size_t i = (size_t)row * nsp + sb;
         Raw r;
-        r.q = nib[i];
-        r.d = dp[i];
+        r.q = rein_ldw(&nib[i]);
+        r.d = rein_ldw(&dp[i]);
         return r;
     }
     static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)
@@ -345,8 +362,8 @@ template <> struct Fmt<REIN_IQ4_XS> {
     {
         const size_t i = (size_t)row * nsp + sb;
         Raw r;
-        r.q = nib[i];
-        r.d = dp[i];
+        r.q = rein_ldw(&nib[i]);
+        r.d = rein_ldw(&dp[i]);
         return r;
     }
     static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)

@@ -74,14 +74,21 @@ def rel_l2(a, b):
 
 
 def assert_close_f32(got, want, rel=1e-3, abs_=1e-4, what=""):
-    """fp32 output bar: |got-want| <= abs + rel*|want| element-wise."""
+    """fp32 output bar: |got-want| <= abs*max(1, rms(want)) + rel*|want| element-wise.
+
+    The absolute part is stated for outputs of unit scale (weights ~N(0,0.02),
+    activations ~N(0,1) give rms(y) ~ 1).  The random-byte weights of the
+    reference's GPU tests (kernels.rs:3026-3061) give sums of terms of magnitude
+    ~40 and rms(y) in the hundreds; there the order of the fp32 additions alone
+    moves an element by 1e-4, so the absolute part scales with rms(want)."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
     err = np.abs(got - want)
-    tol = abs_ + rel * np.abs(want)
-    bad = err > tol
+    scale = max(1.0, float(np.sqrt(np.mean(want * want)))) if want.size else 1.0
+    tol = abs_ * scale + rel * np.abs(want)
+    bad = ~(err <= tol)
     if bad.any():
-        i = int(np.argmax(err - tol))
+        i = int(np.argmax(np.where(np.isnan(err), np.inf, err - tol)))
         raise AssertionError(
-            f"{what}: {int(bad.sum())}/{bad.size} outside {rel} rel / {abs_} abs; worst at flat {i}: "
+            f"{what}: {int(bad.sum())}/{bad.size} outside {rel} rel / {abs_}*{scale:.3g} abs; worst at flat {i}: "
             f"got {got.ravel()[i]!r} want {want.ravel()[i]!r}")

@@ -229,6 +229,48 @@ def test_mmq_parity(fmt, p_rows):
     assert np.array_equal(dd.to_host(np.int32).reshape(parts.shape), parts)
 
 
+# The skinny MMQ (batches of up to 16 rows on the matrix cores, the contraction split
+# over the wavefronts of a workgroup): every split factor, ragged last chunks of the
+# fp16-scale formats, weight-row and token tails, and a shape (odd number of
+# superblocks, odd rows) in which half of Q6_K's fp16 scales sit in the upper half
+# of their dword.
+@pytest.mark.parametrize("fmt", ALL)
+@pytest.mark.parametrize("p_rows,in_dim,out_dim,ks", [
+    (8, 2048, 77, 1), (8, 2048, 77, 3), (7, 2048, 77, 8), (16, 1280, 45, 2), (9, 1280, 45, 5),
+    (3, 768, 130, 0), (13, 5120, 64, 16)])
+def test_skinny_mmq_parity(fmt, p_rows, in_dim, out_dim, ks, monkeypatch):
+    monkeypatch.setenv("REIN_SKINNY_KS", str(ks))
+    monkeypatch.setenv("REIN_SKINNY_FROM", "1")
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=1000 + fmt + p_rows)
+    x = np.random.default_rng(p_rows + ks).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    runtime.mmq_xq8(fmt, dev(packed), dq, dy, in_dim, out_dim, p_rows)
+    hip.synchronize()
+    y = dy.to_host(np.float32).reshape(p_rows, out_dim)
+    check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim, y, p_rows, x)
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])       # the formats with 32-element blocks on disk
+@pytest.mark.parametrize("n_sub,p_rows", [(11, 8), (9, 5), (15, 16), (8, 2), (7, 8)])
+def test_skinny_mmq_ragged_chunks(fmt, n_sub, p_rows, monkeypatch):
+    # in_dim only a multiple of 32: the last chunk has 1..7 sub-blocks; 7 sub-blocks in
+    # all (in_dim < 256) is below what the skinny kernel takes and falls back
+    monkeypatch.setenv("REIN_SKINNY_FROM", "1")
+    in_dim, out_dim = 32 * n_sub, 50
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=5 + n_sub)
+    x = np.random.default_rng(8).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    for entry in (runtime.mmq_xq8, runtime.matvec_batched_xq8):
+        if entry is runtime.matvec_batched_xq8 and p_rows > 8:
+            continue
+        dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+        entry(fmt, dev(packed), dq, dy, in_dim, out_dim, p_rows)
+        hip.synchronize()
+        y = dy.to_host(np.float32).reshape(p_rows, out_dim)
+        check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim, y, p_rows, x)
+
+
 @pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])
 def test_mmq_odd_sub_block_count(fmt):
     in_dim, out_dim, p_rows = 32 * 11, 50, 40          # 11 sub-blocks: ragged last chunk and pair
