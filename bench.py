@@ -169,12 +169,135 @@ def cpu_baseline(fmt, in_dim, out_dim, seed, budget_s=12.0):
                       f"algorithmic (repacked) bytes / time; {round(in_dim * out_dim * 4 / best / 1e9, 2)} GB/s of f32 traffic"}
 
 
+def tiled_weights(fmt, in_dim, out_dim, seed, base_rows=512):
+    """Repacked weights for timing only: quantize base_rows rows and tile them (the
+    kernels' speed does not depend on the values)."""
+    base_rows = min(base_rows, out_dim)
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((base_rows, in_dim), dtype=np.float32) * np.float32(0.02))
+    raw = quant.quantize_weights(fmt, w)
+    reps = -(-out_dim // base_rows)
+    raw = np.tile(raw, reps)[: out_dim * in_dim // quant.block_size(fmt) * quant.bytes_per_block(fmt)]
+    return quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+
+
+def time_graph(stream, launch_all, n_launches, steps=5):
+    """seconds per launch of a captured train of launches"""
+    stream.begin_capture()
+    launch_all()
+    g = stream.end_capture()
+    ex = g.instantiate()
+    ex.launch(stream)
+    stream.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record(stream)
+    for _ in range(steps):
+        ex.launch(stream)
+    e1.record(stream)
+    e1.synchronize()
+    return e0.elapsed_ms(e1) * 1e-3 / (steps * n_launches)
+
+
+def extras_mmq(stream):
+    """BASELINE configs[2]: B in {Q4_K, Q6_K, Q8_0} x M in {128, 512, 2048}, 5120 x 17408"""
+    out = []
+    k, n = 5120, 17408
+    for f in (rein.Q4_K, rein.Q6_K, rein.Q8_0):
+        packed = tiled_weights(f, k, n, seed=3)
+        ws = [hip.DeviceBuf.from_host(packed) for _ in range(4)]          # 4 x (52..95) MB > Infinity Cache
+        for m in (128, 512, 2048):
+            x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+            dx, dq, dy = hip.DeviceBuf.from_host(x), hip.DeviceBuf(m * (k // 32) * 40), hip.DeviceBuf(m * n * 4)
+            runtime.quantize_q8(dx, dq, k, m, stream)
+            sec = time_graph(stream, lambda: [runtime.mmq_xq8(f, w_, dq, dy, k, n, m, stream) for w_ in ws], len(ws))
+            tops = 2.0 * m * k * n / sec / 1e12
+            out.append({"fmt": FMT_NAME[f], "M": m, "us": round(sec * 1e6, 1), "TOPS": round(tops, 1),
+                        "frac_int8_peak": round(tops / INT8_PEAK_TOPS, 4)})
+            log("mmq", out[-1])
+            del dx, dq, dy
+        del ws
+    return out
+
+
+def extras_moe(stream):
+    """BASELINE configs[3]: 512 tokens, hidden 2048, 128 experts, top-8, expert ff 768; gate/up Q4_K,
+    down Q6_K; top-k -> sort -> gather -> grouped GEMMs with SwiGLU -> scatter -> combine."""
+    n_tok, hidden, n_expert, n_used, ff = 512, 2048, 128, 8, 768
+    rng = np.random.default_rng(11)
+    gate1 = tiled_weights(rein.Q4_K, hidden, ff, seed=1, base_rows=ff)
+    up1 = tiled_weights(rein.Q4_K, hidden, ff, seed=2, base_rows=ff)
+    down1 = tiled_weights(rein.Q6_K, ff, hidden, seed=3, base_rows=hidden)
+    gate = hip.DeviceBuf.from_host(np.tile(gate1, n_expert))
+    up = hip.DeviceBuf.from_host(np.tile(up1, n_expert))
+    down = hip.DeviceBuf.from_host(np.tile(down1, n_expert))
+    weight_bytes = (gate1.nbytes + up1.nbytes + down1.nbytes) * n_expert
+    x = rng.standard_normal((n_tok, hidden)).astype(np.float32)
+    logits = rng.standard_normal((n_tok, n_expert)).astype(np.float32)
+    dx, dl = hip.DeviceBuf.from_host(x), hip.DeviceBuf.from_host(logits)
+    ds = hip.DeviceBuf.from_host(np.ones(n_expert, np.float32))
+    shape = runtime.moe_shape(n_tok, hidden, n_expert, n_used, ff, rein.Q4_K, rein.Q6_K)
+    wsb = hip.DeviceBuf(runtime.moe_workspace_bytes(shape))
+    dout = hip.DeviceBuf(n_tok * hidden * 4)
+    reps = 4
+    sec = time_graph(stream, lambda: [runtime.moe_ffn(shape, dx, dl, gate, up, down, ds, wsb, dout, stream)
+                                      for _ in range(reps)], reps)
+    ops = 2.0 * n_tok * n_used * (2 * hidden * ff + ff * hidden)
+    res = {"workload": "MoE expert FFN, 512 tok x 128 experts top-8, hidden 2048, ff 768 (Q4_K gate/up, Q6_K down)",
+           "us": round(sec * 1e6, 1), "weight_GBs": round(weight_bytes / sec / 1e9, 0),
+           "frac_hbm_peak": round(weight_bytes / sec / 1e9 / HBM_PEAK_GBS, 4), "TOPS": round(ops / sec / 1e12, 1),
+           "weight_bytes": weight_bytes,
+           "note": "the 401 MB of expert weights are re-read from the 256 MB Infinity Cache + HBM on every repetition"}
+    log("moe", res)
+    return res
+
+
+def extras_decode_stream(stream):
+    """BASELINE configs[4]: 64 layers x {QKV 5120->7168, O 5120->5120, gate+up 5120->34816, down 17408->5120},
+    Q4_K with every fourth layer's down and the 5120->151936 LM head in Q6_K, batch 1, one hipGraph."""
+    n_layers, hidden, ffn = 64, 5120, 17408
+    shapes = [("qkv", hidden, 7168), ("o", hidden, hidden), ("gate_up", hidden, 2 * ffn), ("down", ffn, hidden)]
+    uniq = {}
+    for name, k, n in shapes:
+        for f in ((rein.Q4_K, rein.Q6_K) if name == "down" else (rein.Q4_K,)):
+            uniq[(name, f)] = tiled_weights(f, k, n, seed=len(uniq))
+    head = tiled_weights(rein.Q6_K, hidden, 151936, seed=99)
+    layers, total = [], 0
+    for layer in range(n_layers):
+        for name, k, n in shapes:
+            f = rein.Q6_K if (name == "down" and layer % 4 == 3) else rein.Q4_K
+            buf = hip.DeviceBuf.from_host(uniq[(name, f)])                  # every layer its own copy in HBM
+            layers.append((f, buf, k, n))
+            total += uniq[(name, f)].nbytes
+    dhead = hip.DeviceBuf.from_host(head)
+    total += head.nbytes
+    xs = {k: np.random.default_rng(k).standard_normal((1, k)).astype(np.float32) for k in (hidden, ffn)}
+    dq = {}
+    for k, x in xs.items():
+        dx = hip.DeviceBuf.from_host(x)
+        dq[k] = hip.DeviceBuf((k // 32) * 40)
+        runtime.quantize_q8(dx, dq[k], k, 1, stream)
+    dy = hip.DeviceBuf(151936 * 4)
+
+    def step():
+        for f, buf, k, n in layers:
+            runtime.matvec_xq8(f, buf, dq[k], dy, k, n, stream)
+        runtime.matvec_xq8(rein.Q6_K, dhead, dq[hidden], dy, hidden, 151936, stream)
+
+    sec = time_graph(stream, step, 1, steps=5)
+    res = {"workload": "decode weight stream, 64 layers (QKV, O, gate+up, down) + LM head, batch 1, one hipGraph of "
+                       f"{len(layers) + 1} matvecs (Q4_K; every 4th down and the head Q6_K)",
+           "ms_per_token": round(sec * 1e3, 3), "tokens_per_s": round(1.0 / sec, 1), "weight_GB": round(total / 1e9, 2),
+           "GBs": round(total / sec / 1e9, 0), "frac_hbm_peak": round(total / sec / 1e9 / HBM_PEAK_GBS, 4)}
+    log("decode stream", res)
+    return res
+
+
 HEADLINE_SHAPES = ((5120, 5120), (5120, 34816), (17408, 5120))      # (K, N) of configs[1]
 # HBM bytes per launch of the dominant kernel (Q4_K 5120 -> 34816, batch 1) from rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by the same counter's reading for the
-# set-up device-to-device copies of known size (fetch x1.99905, write x1.0); it cannot be read
+# set-up device-to-device copies of known size (fetch x1.9992, write x1.0); it cannot be read
 # live, so it is the recorded figure and only reported for the configuration it was taken on
-DOMINANT_TRAFFIC_BYTES = 104054700
+DOMINANT_TRAFFIC_BYTES = 109573400
 
 
 def main():
@@ -185,6 +308,8 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="also time the format x shape x batch sweep of configs[1]")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mmq", action="store_true")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time BASELINE configs[2..4]: MMQ formats x M, the MoE expert FFN, the decode weight stream")
     ap.add_argument("--fmt", default="q4_k")
     ap.add_argument("--batch", type=int, default=1)
     args = ap.parse_args()
@@ -271,6 +396,10 @@ def main():
                     log(sweep[-1])
                     del c
         out["sweep"] = sweep
+
+    if args.extras:
+        out["extras"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
+                         "decode_stream_configs4": extras_decode_stream(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)

@@ -741,10 +741,13 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
     }
 }
 
+// One workgroup tile of the tuned kernel: 256 threads, rows 128*rb .., tokens
+// tok_base .. tok_end (at most TM) of xq / y.  Ends on a barrier, so a workgroup may
+// run several tiles in a row.
 template <int FMT, int TM>
-__device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
-                                                   float* __restrict__ y, unsigned in_dim, unsigned out_dim,
-                                                   unsigned p_rows)
+__device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                        float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                        unsigned rb, unsigned tok_base, unsigned tok_end)
 {
     using F = Fmt<FMT>;
     using C = MmqChunk<FMT>;
@@ -753,13 +756,6 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
     __shared__ MmqLds<TM> lds[2];
     __shared__ MmqWLds<FMT> wlds[4];
 
-    // workgroup -> (row block, token tile), XCD-aware
-    const unsigned n_rb = (out_dim + 127u) / 128u;
-    const unsigned n_tt = (p_rows + TM - 1) / TM;
-    const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
-    const unsigned rb = (k / n_tt) * 8u + xcd, tt = k % n_tt;
-    if (rb >= n_rb) return;
-
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned j = lane & 31u, h = lane >> 5;
     const unsigned n_sub = in_dim >> 5;
@@ -767,8 +763,6 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
     const unsigned row_base = rb * 128u + wave * 32u;
     const unsigned row = row_base + j;
     const unsigned rowc = row < out_dim ? row : out_dim - 1;
-    const unsigned tok_base = tt * TM;
-    const unsigned tok_end = min(p_rows, tok_base + TM);
     const unsigned wsel = FMT == REIN_Q8_0 ? h : 0u;
     MmqWLds<FMT>& wl = wlds[wave];
 
@@ -830,6 +824,20 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
         }
 }
 
+template <int FMT, int TM>
+__device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                   float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                   unsigned p_rows)
+{
+    // workgroup -> (row block, token tile), XCD-aware
+    const unsigned n_rb = (out_dim + 127u) / 128u;
+    const unsigned n_tt = (p_rows + TM - 1) / TM;
+    const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
+    const unsigned rb = (k / n_tt) * 8u + xcd, tt = k % n_tt;
+    if (rb >= n_rb) return;
+    rein_mmq_pipelined_tile<FMT, TM>(w, xq, y, in_dim, out_dim, rb, tt * TM, min(p_rows, tt * TM + TM));
+}
+
 // Dense GEMM: grid-stride over (row block, token tile).
 template <int FMT, int TM, int DOTS>
 __device__ __forceinline__ void rein_mmq_dense(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
@@ -849,15 +857,17 @@ __device__ __forceinline__ void rein_mmq_dense(const uint8_t* __restrict__ w, co
 
 // Grouped-expert GEMM (kernels/mmq_gemm_q4k_grouped.cpp:38-165): tile index
 // blockIdx.y -> expert by binary search over tile_off; the tile's tokens are
-// rows expert_off[e] + 32*local .. of the expert-sorted xq / y.
+// rows expert_off[e] + 32*local .. of the expert-sorted xq / y.  Each tile runs
+// the tuned 32-token workgroup tile; any grid is correct, the block must be 256
+// threads (src/runtime/qwen35.rs:3062).
 template <int FMT>
 __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ slab, unsigned bytes_per_expert,
                                                  const int* __restrict__ expert_off, const int* __restrict__ tile_off,
                                                  unsigned n_expert, const BlockQ8* __restrict__ xq,
                                                  float* __restrict__ y, unsigned in_dim, unsigned out_dim)
 {
-    const unsigned rpb = 32u * (blockDim.x >> 6);
-    const unsigned n_rb = (out_dim + rpb - 1u) / rpb;
+    if (blockDim.x != 256u) return;                // the tuned tile is built for 4 wavefronts (the reference's launch)
+    const unsigned n_rb = (out_dim + 127u) / 128u;
     const unsigned n_tiles = (unsigned)tile_off[n_expert];
     for (unsigned tile = blockIdx.y; tile < n_tiles; tile += gridDim.y) {
         unsigned lo = 0, hi = n_expert;            // largest e with tile_off[e] <= tile
@@ -870,8 +880,8 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
         const unsigned tok_end = (unsigned)expert_off[e + 1];
         if (tok_base >= tok_end) continue;         // host counted tiles with a smaller bn
         for (unsigned rb = blockIdx.x; rb < n_rb; rb += gridDim.x)
-            rein_mmq_tile<FMT, 32, 0>(slab + (size_t)e * bytes_per_expert, xq, y, nullptr, in_dim, out_dim, rb,
-                                      tok_base, min(tok_end, tok_base + 32u));
+            rein_mmq_pipelined_tile<FMT, 32>(slab + (size_t)e * bytes_per_expert, xq, y, in_dim, out_dim, rb,
+                                             tok_base, min(tok_end, tok_base + 32u));
     }
 }
 
