@@ -144,14 +144,15 @@ unsigned pick_rows_per_wave(unsigned out_dim, unsigned batch)
 
 unsigned batch_slot(unsigned n_rows) { return n_rows <= 1 ? 1 : n_rows <= 2 ? 2 : n_rows <= 4 ? 4 : 8; }
 
-// Skinny MMQ (rein_mmqs_<fmt>_v<NV>): up to 16 activation rows per token group on
-// the matrix cores; KS wavefronts of a workgroup (the block size) split the
-// contraction over the same 32 weight rows.  The kernel hides latency with resident
-// wavefronts, so KS is the smallest split that fills the machine: waves_per_cu is
-// what LDS and the 128-register budget allow (at most 16), a CU holds
-// floor(waves_per_cu / KS) workgroups, and a choice costs
-// rounds x (chunks per wavefront + about two chunks of pipeline fill), with a
-// penalty when fewer than about 12 wavefronts per CU are resident.
+// Skinny MMQ launch: grid.x = 32-row tiles, grid.y = token groups, block = KS
+// wavefronts that split the contraction of one tile.  The kernels keep several
+// chunks of weights in flight in registers, which leaves room for two or three
+// wavefronts per SIMD (the table below mirrors the kernels' register budgets).
+// Measured on MI355X (Q4_K): a wavefront alone on its SIMD takes 1.5 us per chunk;
+// m >= 2 wavefronts sharing a SIMD take 1.14 us x m each (the SIMD is then busy).
+// KS is chosen by that model: when every wavefront is resident at once the fullest
+// SIMD sets the time; otherwise the work streams through the slots and the last
+// workgroups run underoccupied.
 int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
                   unsigned n_rows, rein_stream_t s)
 {
@@ -159,18 +160,25 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
     const unsigned tiles = ((out_dim + 31) / 32) * ((n_rows + tok - 1) / tok);
     const unsigned n_chunks = (in_dim / 32 + 7) / 8;
     const unsigned planes = fmt == REIN_TYPE_Q8_0 ? 2 : 1;
-    const unsigned small_lds = fmt == REIN_TYPE_Q4_K ? 640 : fmt == REIN_TYPE_Q5_K ? 1664 : fmt == REIN_TYPE_Q6_K ? 2688 : 512;
-    const unsigned lds_per_wave = planes * 4096 + 2 * (320 * tok + small_lds);    // sizeof(SkinnyWaveLds<FMT, TOK>)
-    const unsigned waves_per_cu = std::min(16u, 160u * 1024u / lds_per_wave);
-    const unsigned ks_max = std::min(std::min(16u, waves_per_cu), n_chunks);
+    const unsigned lds_per_wave = planes * 4096 + 320 * tok;                       // sizeof(SkinnyWaveLds<FMT, TOK>)
+    const bool three = nv == 4 && (fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q8_0 ||
+                                   fmt == REIN_TYPE_IQ4_XS);
+    const unsigned occ = three ? 3 : 2;                                            // wavefronts per SIMD (registers)
+    const unsigned waves_per_cu = std::min(4 * occ, 160u * 1024u / lds_per_wave);
+    const unsigned ks_max = std::min(std::min(8u, waves_per_cu), n_chunks);        // the kernels' launch bound is 512 threads
     unsigned ks = 1;
     double best = 1e30;
     for (unsigned k = 1; k <= ks_max; k++) {
         const unsigned wg_per_cu = waves_per_cu / k;
-        const unsigned rounds = (tiles + kCUs * wg_per_cu - 1) / (kCUs * wg_per_cu);
-        // wavefronts resident per CU in a typical round
-        const double resident = std::min((double)wg_per_cu * k, (double)tiles * k / (kCUs * rounds));
-        const double cost = rounds * ((n_chunks + k - 1) / k + 2.0) * std::max(1.0, 12.0 / resident);
+        const double waves = (double)tiles * k, slots = (double)kCUs * wg_per_cu * k;
+        const double per_wave = (n_chunks + k - 1) / k + 2.0;                      // chunks, plus pipeline fill and the reduction
+        double cost;
+        if (waves <= slots) {
+            const double m = std::ceil(waves / (kCUs * 4.0));
+            cost = per_wave * std::max(1.5, 1.14 * m);
+        } else {
+            cost = waves * per_wave / (kCUs * 4.0) * 1.14 + 0.5 * per_wave * 1.5;
+        }
         if (cost < best) { best = cost; ks = k; }
     }
     const unsigned forced = env_u("REIN_SKINNY_KS", 0);
@@ -181,10 +189,14 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
 }
 
 // Activation rows from which the batched decode leaves the dot4 kernels for the
-// skinny MMQ (v_dot4 issues at a quarter of the fp32 rate on this part, so eight
-// dot4 chains per weight row cost more than one MFMA tile).  Measured on MI355X,
-// Q4_K: at 4 rows the two are level, at 8 rows the skinny MMQ is 1.7-2.3x faster.
-unsigned skinny_from_rows() { return env_u("REIN_SKINNY_FROM", 5); }
+// skinny MMQ.  Measured on MI355X, 5120 -> 34816: Q4_K dot4 takes 21 / 28 / 39 / 39 us
+// at 1 / 2 / 3 / 4 rows (three rows run in the four-row kernel), the skinny MMQ 33 us
+// for anything up to 8 rows; Q4_0, Q8_0 and IQ4_XS behave alike.  Q5_K and Q6_K carry
+// more aux words per sub-block: there the skinny MMQ only wins from 5 rows.
+unsigned skinny_from_rows(int fmt)
+{
+    return env_u("REIN_SKINNY_FROM", fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q6_K ? 5 : 3);
+}
 
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
                   unsigned out_dim, unsigned n_rows, rein_stream_t s)
@@ -195,7 +207,7 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
-    if (n_rows >= skinny_from_rows() && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(out_dim, b);
     const unsigned wpb = 4;
@@ -326,7 +338,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows() <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // Token tile.  The 64-token tile does about 6 % more work per cycle when the
     // machine is evenly loaded (the weight unpack is shared by two MFMA tiles), but two
     // of its workgroups fit a CU against three of the 32-token tile (registers), so the
