@@ -292,6 +292,46 @@ def extras_decode_stream(stream):
     return res
 
 
+def extras_fused(stream):
+    """The producers in front of the matvecs: fused (one launch writes the BlockQ8 blocks) against the
+    two-launch chain they replace, at the decode shapes (hidden 5120, FFN 17408) and the MoE
+    intermediate (4096 expert rows x 768).  Launch-bound: microseconds per launch from a hipGraph."""
+    out = []
+    rng = np.random.default_rng(0)
+    n, ffn, rows, ff = 5120, 17408, 4096, 768
+    dev = hip.DeviceBuf.from_host
+    h, a, w = (dev(rng.standard_normal(n).astype(np.float32)) for _ in range(3))
+    y, q = hip.DeviceBuf(n * 4), hip.DeviceBuf(n // 32 * 40)
+    reps = 32
+
+    def t(fn):
+        return time_graph(stream, lambda: [fn() for _ in range(reps)], reps) * 1e6
+
+    out.append({"op": "add_rmsnorm_q8 n=5120 (hidden += add, norm, fp32 + BlockQ8)",
+                "us": round(t(lambda: runtime.add_rmsnorm_q8(h, a, w, y, q, n, 1, 1e-6, stream)), 2)})
+    out.append({"op": "rmsnorm_q8 n=5120", "us": round(t(lambda: runtime.rmsnorm_q8(h, w, q, n, 1, 1e-6, stream)), 2)})
+    out.append({"op": "quantize_q8 n=5120 alone", "us": round(t(lambda: runtime.quantize_q8(h, q, n, 1, stream)), 2)})
+    g, u = (dev(rng.standard_normal(ffn).astype(np.float32)) for _ in range(2))
+    o, q2 = hip.DeviceBuf(ffn * 4), hip.DeviceBuf(ffn // 32 * 40)
+    out.append({"op": "swiglu_q8 n=17408 fused", "us": round(t(lambda: runtime.swiglu_q8(g, u, o, q2, ffn, stream)), 2)})
+    out.append({"op": "swiglu_mul + quantize_q8 n=17408 (two launches)",
+                "us": round(t(lambda: (runtime.swiglu_mul(g, u, o, ffn, stream), runtime.quantize_q8(o, q2, ffn, 1, stream))), 2)})
+    big = rows * ff
+    g, u = (dev(rng.standard_normal(big).astype(np.float32)) for _ in range(2))
+    o, q3 = hip.DeviceBuf(big * 4), hip.DeviceBuf(big // 32 * 40)
+    fused = t(lambda: runtime.swiglu_q8(g, u, None, q3, big, stream))
+    chain = t(lambda: (runtime.swiglu_mul(g, u, o, big, stream), runtime.quantize_q8(o, q3, ff, rows, stream)))
+    out.append({"op": "swiglu_q8 4096 x 768 fused (MoE intermediate)", "us": round(fused, 2),
+                "GBs": round((2 * big * 4 + big // 32 * 40) / fused / 1e3, 0)})
+    out.append({"op": "swiglu_mul + quantize_q8 4096 x 768 (two launches)", "us": round(chain, 2),
+                "GBs": round((4 * big * 4 + big // 32 * 40) / chain / 1e3, 0)})
+    gu = dev(rng.standard_normal((rows, 2 * ff)).astype(np.float32))
+    out.append({"op": "moe_geglu_q8 4096 x 768", "us": round(t(lambda: runtime.moe_geglu_q8(gu, q3, ff, rows, stream)), 2)})
+    for r in out:
+        log("fused", r)
+    return out
+
+
 HEADLINE_SHAPES = ((5120, 5120), (5120, 34816), (17408, 5120))      # (K, N) of configs[1]
 # HBM bytes per launch of the dominant kernel (Q4_K 5120 -> 34816, batch 1) from rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by the same counter's reading for the
@@ -399,7 +439,7 @@ def main():
 
     if args.extras:
         out["extras"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
-                         "decode_stream_configs4": extras_decode_stream(stream)}
+                         "decode_stream_configs4": extras_decode_stream(stream), "fused_producers": extras_fused(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)

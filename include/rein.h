@@ -137,6 +137,37 @@ int rein_quantize_weights(int fmt, const float *src, size_t n, uint8_t *dst);
  * x [n_vec][in_dim] fp32 -> xq [n_vec][in_dim/32] 40-byte BlockQ8. */
 int rein_quantize_q8(const float *x, void *xq, unsigned in_dim, unsigned n_vec, rein_stream_t s);
 
+/* ---- fused BlockQ8 producers: the step in front of a quantized matvec writes
+ * the matvec's input blocks itself.  All dimensions are multiples of 32; every
+ * BlockQ8 output is byte-identical to rein_quantize_q8 of the fp32 result.
+ *
+ * rmsnorm_q8_f32 (kernels/rmsnorm_q8.cpp:38-103; launcher gemma4.rs:1303-1316):
+ * xq[v] = q8(x[v] * rsqrt(mean(x[v]^2) + eps) * w) for n_vec vectors of n values,
+ * n <= 32768.  w [n] is shared by the vectors. */
+int rein_rmsnorm_q8(const float *x, const float *w, void *xq, unsigned n, unsigned n_vec, float eps,
+                    rein_stream_t s);
+/* add_rmsnorm_q8_f32 (kernels/qwen35_fused.cpp:66-121; launcher qwen35.rs:2036-2054):
+ * hidden += add (add may be NULL), y = rmsnorm(hidden) * w as fp32 (y may be NULL)
+ * and as BlockQ8.  The reference handles one vector of n % 1024 == 0, n <= 8192;
+ * here n_vec vectors of any n % 32 == 0, n <= 32768. */
+int rein_add_rmsnorm_q8(float *hidden, const float *add, const float *w, float *y, void *xq,
+                        unsigned n, unsigned n_vec, float eps, rein_stream_t s);
+/* swiglu_q8_f32 (kernels/qwen35_fused.cpp:132-146; launcher qwen35.rs:2056-2069):
+ * out = silu(gate) * up as fp32 (out may be NULL or alias gate) and as BlockQ8. */
+int rein_swiglu_q8(const float *gate, const float *up, float *out, void *xq, unsigned n,
+                   rein_stream_t s);
+/* sigmoid_mul_q8_f32 (kernels/qwen35_fused.cpp:149-162; launcher qwen35.rs:2071-2079):
+ * x *= sigmoid(gate) in place, plus BlockQ8. */
+int rein_sigmoid_mul_q8(float *x, const float *gate, void *xq, unsigned n, rein_stream_t s);
+/* rmsnorm_gated_q8_f32 (kernels/qwen35_fused.cpp:195-217): per head of head_dim values,
+ * y = rmsnorm(x) * w * silu(z) as fp32 (y may be NULL) and as BlockQ8; w [head_dim]. */
+int rein_rmsnorm_gated_q8(const float *x, const float *z, const float *w, float *y, void *xq,
+                          unsigned n_heads, unsigned head_dim, float eps, rein_stream_t s);
+/* moe_geglu_q8_f32 (kernels/moe_geglu_q8.cpp:31-66; launcher gemma4.rs:1781-1796):
+ * gu [n_slot][2*ff_exp] (gate half, up half) -> xq [n_slot][ff_exp/32] =
+ * q8(gelu_tanh(gate) * up). */
+int rein_moe_geglu_q8(const float *gu, void *xq, unsigned ff_exp, unsigned n_slot, rein_stream_t s);
+
 /* launch_matvec_repacked_xq8 (src/runtime/qwen35.rs:2232-2280): y[out_dim] =
  * W . xq for one pre-quantized activation row. */
 int rein_matvec_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,

@@ -877,6 +877,133 @@ void orc_moe_combine(const float *experts, const int32_t *ids, const float *weig
     }
 }
 
+/* ---- fused BlockQ8 producers ---------------------------------------------- */
+
+float orc_exp_det(float x)
+{
+    x = fminf(fmaxf(x, -87.0f), 88.0f);
+    const float n = rintf(x * 1.44269504088896341f);
+    float r = fmaf(n, -0.693145751953125f, x);
+    r = fmaf(n, -1.42860682030941723e-6f, r);
+    float p = 1.0f / 720.0f;
+    p = fmaf(p, r, 1.0f / 120.0f);
+    p = fmaf(p, r, 1.0f / 24.0f);
+    p = fmaf(p, r, 1.0f / 6.0f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    const int ni = (int)n;
+    const int n1 = ni / 2, n2 = ni - n1;
+    const uint32_t b1 = (uint32_t)(n1 + 127) << 23, b2 = (uint32_t)(n2 + 127) << 23;
+    float s1, s2;
+    memcpy(&s1, &b1, 4);
+    memcpy(&s2, &b2, 4);
+    return p * s1 * s2;
+}
+
+float orc_silu_det(float x) { return x / (1.0f + orc_exp_det(-x)); }
+float orc_sigmoid_det(float x) { return 1.0f / (1.0f + orc_exp_det(-x)); }
+float orc_gelu_det(float x)
+{
+    const float c = x + 0.044715f * x * x * x;
+    return x / (1.0f + orc_exp_det(-2.0f * (0.7978845608028654f * c)));
+}
+
+void orc_map_det(int which, const float *x, float *out, size_t n)
+{
+    for (size_t i = 0; i < n; i++)
+        out[i] = which == 0 ? orc_exp_det(x[i]) : which == 1 ? orc_silu_det(x[i]) : which == 2 ? orc_sigmoid_det(x[i])
+               : orc_gelu_det(x[i]);
+}
+
+/* src/cpu/ops.rs:14-16, 20-22, 33-36 with libm */
+void orc_map_ref(int which, const float *x, float *out, size_t n)
+{
+    for (size_t i = 0; i < n; i++) {
+        const float v = x[i];
+        if (which == 1) out[i] = v / (1.0f + expf(-v));
+        else if (which == 2) out[i] = 1.0f / (1.0f + expf(-v));
+        else out[i] = 0.5f * v * (1.0f + tanhf(0.79788456f * (v + 0.044715f * v * v * v)));
+    }
+}
+
+float orc_sumsq_det(const float *x, size_t n)
+{
+    const size_t n_sub = n >> 5;
+    float lane[64];
+    for (int l = 0; l < 64; l++) lane[l] = 0.0f;
+    for (size_t sb = 0; sb < n_sub; sb++) {           /* ascending sb visits each lane's addends in its order */
+        float s[32], t[32];
+        for (int l = 0; l < 32; l++) s[l] = x[sb * 32 + l] * x[sb * 32 + l];
+        for (int o = 16; o > 0; o >>= 1) {
+            for (int l = 0; l < 32; l++) t[l] = s[l] + s[l ^ o];
+            memcpy(s, t, sizeof s);
+        }
+        lane[sb & 63] = lane[sb & 63] + s[0];
+    }
+    float t[64];
+    for (int o = 32; o > 0; o >>= 1) {
+        for (int l = 0; l < 64; l++) t[l] = lane[l] + lane[l ^ o];
+        memcpy(lane, t, sizeof lane);
+    }
+    return lane[0];
+}
+
+void orc_add_rmsnorm(float *hidden, const float *add, const float *w, float *y, size_t n, size_t n_vec, float eps)
+{
+    for (size_t v = 0; v < n_vec; v++) {
+        float *h = hidden + v * n;
+        if (add)
+            for (size_t i = 0; i < n; i++) h[i] = h[i] + add[v * n + i];
+        const float rrms = 1.0f / sqrtf(orc_sumsq_det(h, n) / (float)n + eps);
+        for (size_t i = 0; i < n; i++) y[v * n + i] = (h[i] * rrms) * w[i];
+    }
+}
+
+void orc_rmsnorm_gated(const float *x, const float *z, const float *w, float *y, size_t n_heads, size_t head_dim, float eps)
+{
+    for (size_t h = 0; h < n_heads; h++) {
+        const float *xh = x + h * head_dim, *zh = z + h * head_dim;
+        const float rrms = 1.0f / sqrtf(orc_sumsq_det(xh, head_dim) / (float)head_dim + eps);
+        for (size_t i = 0; i < head_dim; i++) y[h * head_dim + i] = ((xh[i] * rrms) * w[i]) * orc_silu_det(zh[i]);
+    }
+}
+
+void orc_swiglu_det(const float *gate, const float *up, float *out, size_t n)
+{
+    for (size_t i = 0; i < n; i++) out[i] = orc_silu_det(gate[i]) * up[i];
+}
+
+void orc_sigmoid_mul_det(const float *x, const float *gate, float *out, size_t n)
+{
+    for (size_t i = 0; i < n; i++) out[i] = x[i] * orc_sigmoid_det(gate[i]);
+}
+
+void orc_geglu_det(const float *gu, float *out, size_t ff_exp, size_t n_slot)
+{
+    for (size_t s = 0; s < n_slot; s++)
+        for (size_t i = 0; i < ff_exp; i++)
+            out[s * ff_exp + i] = orc_gelu_det(gu[s * 2 * ff_exp + i]) * gu[s * 2 * ff_exp + ff_exp + i];
+}
+
+/* src/cpu/ops.rs:47-57 */
+void orc_rmsnorm_ref(const float *x, const float *w, float eps, float *out, size_t n)
+{
+    float sum_sq = 0.0f;
+    for (size_t i = 0; i < n; i++) sum_sq += x[i] * x[i];
+    const float rrms = 1.0f / sqrtf(sum_sq / (float)n + eps);
+    for (size_t i = 0; i < n; i++) out[i] = x[i] * rrms * w[i];
+}
+
+/* src/cpu/ops.rs:63-76 */
+void orc_rmsnorm_gated_ref(const float *x, const float *gate, const float *w, float eps, float *out, size_t n)
+{
+    float sum_sq = 0.0f;
+    for (size_t i = 0; i < n; i++) sum_sq += x[i] * x[i];
+    const float rrms = 1.0f / sqrtf(sum_sq / (float)n + eps);
+    for (size_t i = 0; i < n; i++) out[i] = x[i] * rrms * w[i] * (gate[i] / (1.0f + expf(-gate[i])));
+}
+
 /* kernels/swiglu.cpp:10-21 */
 void orc_swiglu_mul(const float *gate, const float *up, float *out, size_t n)
 {

@@ -31,6 +31,11 @@
  *                                    dequant -> f32 matvec; brute force
  *   orc_moe_*                        textbook softmax/top-k, sort invariants,
  *                                    closed forms
+ *   orc_exp_det and the functions    libm expf / tanhf to a few ulp over the whole
+ *   built on it; orc_*_q8            range, the known values of ops.rs:176-188, the
+ *                                    reference CPU forms (orc_rmsnorm_ref etc.,
+ *                                    ops.rs:14-76) to rounding, and the identity
+ *                                    fused == quantize_q8(unfused)
  */
 #ifndef REIN_ORACLE_H
 #define REIN_ORACLE_H
@@ -122,6 +127,35 @@ void orc_moe_scatter_rows(const float *src, const int32_t *perm, float *dst, int
 /* kernels/moe_combine.cpp:15-38 */
 void orc_moe_combine(const float *experts, const int32_t *ids, const float *weights,
                      const float *down_exps_s, float *out, int n_tok, int hidden, int n_used);
+/* ---- fused BlockQ8 producers -------------------------------------------------
+ * Deterministic elementwise functions: IEEE add/mul/fma/div/sqrt only, in the
+ * order the device code spells out, so that device and checker agree bit for bit.
+ * exp: n = rint(x*log2 e), two-step fma reduction by ln 2, degree-6 Horner, scaled
+ * by 2^n in two exact steps; x clamped to [-87, 88]. */
+float orc_exp_det(float x);
+float orc_silu_det(float x);      /* x / (1 + exp(-x))           src/cpu/ops.rs:14-16 */
+float orc_sigmoid_det(float x);   /* 1 / (1 + exp(-x))           src/cpu/ops.rs:20-22 */
+float orc_gelu_det(float x);      /* tanh form as x / (1 + exp(-2z))   src/cpu/ops.rs:33-36 */
+void orc_map_det(int which, const float *x, float *out, size_t n);   /* 0 exp 1 silu 2 sigmoid 4 gelu */
+/* sum of squares in the order of the fused norm kernels: per 32-value sub-block
+ * the xor butterfly 16..1, then 64 strided running sums, then the butterfly 32..1 */
+float orc_sumsq_det(const float *x, size_t n);
+/* kernels/qwen35_fused.cpp:66-121 (add may be NULL; hidden is updated when it is
+ * not): y[v] = ((hidden[v] * rrms) * w), rrms = 1 / sqrt(sumsq/n + eps) */
+void orc_add_rmsnorm(float *hidden, const float *add, const float *w, float *y, size_t n, size_t n_vec, float eps);
+/* kernels/qwen35_fused.cpp:195-217: y = ((x * rrms) * w) * silu(z) per head */
+void orc_rmsnorm_gated(const float *x, const float *z, const float *w, float *y, size_t n_heads, size_t head_dim, float eps);
+/* kernels/qwen35_fused.cpp:132-146 / 149-162 / kernels/moe_geglu_q8.cpp:31-66 (fp32 results;
+ * the BlockQ8 form is orc_quantize_q8 of them) */
+void orc_swiglu_det(const float *gate, const float *up, float *out, size_t n);
+void orc_sigmoid_mul_det(const float *x, const float *gate, float *out, size_t n);
+void orc_geglu_det(const float *gu, float *out, size_t ff_exp, size_t n_slot);
+/* The reference's CPU forms, libm and sequential sums: src/cpu/ops.rs:47-57, 63-76,
+ * 14-16, 20-22, 33-36.  which: 1 silu 2 sigmoid 4 gelu */
+void orc_rmsnorm_ref(const float *x, const float *w, float eps, float *out, size_t n);
+void orc_rmsnorm_gated_ref(const float *x, const float *gate, const float *w, float eps, float *out, size_t n);
+void orc_map_ref(int which, const float *x, float *out, size_t n);
+
 /* kernels/swiglu.cpp:10-21 (expf in place of __expf) */
 void orc_swiglu_mul(const float *gate, const float *up, float *out, size_t n);
 /* kernels/mmq_gemm_q4k_grouped.cpp:38-165 — per expert e, rows

@@ -50,6 +50,16 @@ def _load():
         "orc_moe_scatter_rows": (None, [f32p, i32p, f32p, C.c_int, C.c_int]),
         "orc_moe_combine": (None, [f32p, i32p, f32p, f32p, f32p, C.c_int, C.c_int, C.c_int]),
         "orc_swiglu_mul": (None, [f32p, f32p, f32p, sz]),
+        "orc_map_det": (None, [C.c_int, f32p, f32p, sz]),
+        "orc_map_ref": (None, [C.c_int, f32p, f32p, sz]),
+        "orc_sumsq_det": (C.c_float, [f32p, sz]),
+        "orc_add_rmsnorm": (None, [f32p, f32p, f32p, f32p, sz, sz, C.c_float]),
+        "orc_rmsnorm_gated": (None, [f32p, f32p, f32p, f32p, sz, sz, C.c_float]),
+        "orc_swiglu_det": (None, [f32p, f32p, f32p, sz]),
+        "orc_sigmoid_mul_det": (None, [f32p, f32p, f32p, sz]),
+        "orc_geglu_det": (None, [f32p, f32p, sz, sz]),
+        "orc_rmsnorm_ref": (None, [f32p, f32p, C.c_float, f32p, sz]),
+        "orc_rmsnorm_gated_ref": (None, [f32p, f32p, f32p, C.c_float, f32p, sz]),
         "orc_grouped_gemm": (C.c_int, [C.c_int, u8p, sz, i32p, C.c_int, u8p, f32p, sz, sz, C.c_int]),
     }
     for name, (res, args) in sig.items():
@@ -235,6 +245,87 @@ def swiglu_mul(gate, up):
     gate, up = _f32(gate), _f32(up)
     out = np.empty_like(gate)
     lib.orc_swiglu_mul(_p(gate), _p(up), _p(out), gate.size)
+    return out
+
+
+# ---- fused BlockQ8 producers: fp32 results (BlockQ8 form = quantize_q8 of them)
+_DET = {"exp": 0, "silu": 1, "sigmoid": 2, "gelu": 4}
+
+
+def map_det(which, x):
+    """the deterministic elementwise functions the fused producers use"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib.orc_map_det(_DET[which], _p(x), _p(out), x.size)
+    return out
+
+
+def map_ref(which, x):
+    """the reference CPU forms with libm (src/cpu/ops.rs:14-36)"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib.orc_map_ref(_DET[which], _p(x), _p(out), x.size)
+    return out
+
+
+def sumsq_det(x):
+    x = _f32(x)
+    return float(lib.orc_sumsq_det(_p(x), x.size))
+
+
+def add_rmsnorm(hidden, add, w, eps):
+    """-> (hidden after the add, y); hidden/add [n_vec, n], w [n]"""
+    hidden = np.array(_f32(hidden), copy=True)
+    n_vec, n = hidden.shape
+    w = _f32(w)
+    y = np.empty_like(hidden)
+    a = _f32(add) if add is not None else None
+    lib.orc_add_rmsnorm(_p(hidden), _p(a) if a is not None else None, _p(w), _p(y), n, n_vec, eps)
+    return hidden, y
+
+
+def rmsnorm_gated(x, z, w, eps):
+    x, z, w = _f32(x), _f32(z), _f32(w)
+    n_heads, head_dim = x.shape
+    y = np.empty_like(x)
+    lib.orc_rmsnorm_gated(_p(x), _p(z), _p(w), _p(y), n_heads, head_dim, eps)
+    return y
+
+
+def swiglu_det(gate, up):
+    gate, up = _f32(gate), _f32(up)
+    out = np.empty_like(gate)
+    lib.orc_swiglu_det(_p(gate), _p(up), _p(out), gate.size)
+    return out
+
+
+def sigmoid_mul_det(x, gate):
+    x, gate = _f32(x), _f32(gate)
+    out = np.empty_like(x)
+    lib.orc_sigmoid_mul_det(_p(x), _p(gate), _p(out), x.size)
+    return out
+
+
+def geglu_det(gu):
+    """gu [n_slot, 2*ff] -> [n_slot, ff]"""
+    gu = _f32(gu)
+    n_slot, two_ff = gu.shape
+    out = np.empty((n_slot, two_ff // 2), np.float32)
+    lib.orc_geglu_det(_p(gu), _p(out), two_ff // 2, n_slot)
+    return out
+
+
+def rmsnorm_ref(x, w, eps):
+    x, w = _f32(x), _f32(w)
+    out = np.empty_like(x)
+    lib.orc_rmsnorm_ref(_p(x), _p(w), eps, _p(out), x.size)
+    return out
+
+
+def rmsnorm_gated_ref(x, gate, w, eps):
+    x, gate, w = _f32(x), _f32(gate), _f32(w)
+    out = np.empty_like(x)
+    lib.orc_rmsnorm_gated_ref(_p(x), _p(gate), _p(w), eps, _p(out), x.size)
     return out
 
 

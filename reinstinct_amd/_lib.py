@@ -81,6 +81,12 @@ SIGNATURES = {
     "rein_moe_scatter_rows": (_i, [_vp, _vp, _vp, _u, _u, _vp]),
     "rein_moe_grouped_gemm": (_i, [_i, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
     "rein_swiglu_mul": (_i, [_vp, _vp, _vp, _u, _vp]),
+    "rein_rmsnorm_q8": (_i, [_vp, _vp, _vp, _u, _u, C.c_float, _vp]),
+    "rein_add_rmsnorm_q8": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _u, C.c_float, _vp]),
+    "rein_swiglu_q8": (_i, [_vp, _vp, _vp, _vp, _u, _vp]),
+    "rein_sigmoid_mul_q8": (_i, [_vp, _vp, _vp, _u, _vp]),
+    "rein_rmsnorm_gated_q8": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _u, C.c_float, _vp]),
+    "rein_moe_geglu_q8": (_i, [_vp, _vp, _u, _u, _vp]),
     "rein_moe_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_moe_gemm_bn": (_u, []),
     "rein_moe_workspace_bytes": (_sz, [_P(MoeShape)]),

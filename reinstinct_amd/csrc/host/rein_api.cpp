@@ -312,10 +312,112 @@ int rein_quantize_q8(const float* x, void* xq, unsigned in_dim, unsigned n_vec, 
     if (n_vec > 65535) return fail(REIN_E_TOO_LARGE, "rein_quantize_q8: at most 65535 vectors per call");
     if (int rc = check_ptr("rein_quantize_q8", x, 4, "x")) return rc;
     if (int rc = check_ptr("rein_quantize_q8", xq, 8, "xq")) return rc;
-    // 8 sub-blocks per 256-thread workgroup, as the reference launch (qwen35.rs:3202-3211)
-    const unsigned gx = (in_dim + 255) / 256;
+    // 16 sub-blocks per 256-thread workgroup (a 16-lane row each); the reference launches
+    // 8 per workgroup (qwen35.rs:3202-3211), which the kernel accepts as well
+    const unsigned gx = (in_dim + 511) / 512;
     void* args[] = {(void*)&x, (void*)&xq, (void*)&in_dim};
     return launch("quantize_q8_f32", gx, n_vec, 1, 256, 0, s, args);
+}
+
+// ---- fused BlockQ8 producers (kernels/fused_q8.hip)
+
+namespace {
+int check_fused_n(const char* who, unsigned n, unsigned n_vec, unsigned n_max)
+{
+    if (n == 0 || n % 32 != 0 || n_vec == 0)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": the vector length must be a non-zero multiple of 32 and the count non-zero");
+    if (n_max && n > n_max) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most " + std::to_string(n_max) + " values per vector");
+    if (n_vec > 65535) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most 65535 vectors per call");
+    return 0;
+}
+// one workgroup per vector, a 16-lane row per sub-block: as many rows as the vector has
+// sub-blocks (the serial part of the kernel is per row), whole wavefronts, at most 1024
+// threads (the kernel keeps up to four sub-blocks per row in registers and re-reads
+// beyond that)
+unsigned fused_norm_block(unsigned n)
+{
+    const unsigned rows = n / 32;
+    return std::min(1024u, (rows * 16 + 63) / 64 * 64);
+}
+unsigned elementwise_grid(unsigned n)
+{
+    unsigned g = (n + 511) / 512;              // 16 rows of a 256-thread block, 32 values each
+    return std::min(g, kCUs * 32);
+}
+}  // namespace
+
+int rein_rmsnorm_q8(const float* x, const float* w, void* xq, unsigned n, unsigned n_vec, float eps, rein_stream_t s)
+{
+    const char* who = "rein_rmsnorm_q8";
+    if (int rc = check_fused_n(who, n, n_vec, 32768)) return rc;
+    if (int rc = check_ptr(who, x, 4, "x")) return rc;
+    if (int rc = check_ptr(who, w, 4, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    void* a[] = {(void*)&x, (void*)&w, (void*)&xq, (void*)&n, (void*)&eps};
+    return launch("rmsnorm_q8_f32", 1, n_vec, 1, fused_norm_block(n), 0, s, a);
+}
+
+int rein_add_rmsnorm_q8(float* hidden, const float* add, const float* w, float* y, void* xq, unsigned n,
+                        unsigned n_vec, float eps, rein_stream_t s)
+{
+    const char* who = "rein_add_rmsnorm_q8";
+    if (int rc = check_fused_n(who, n, n_vec, 32768)) return rc;
+    if (int rc = check_ptr(who, hidden, 4, "hidden")) return rc;
+    if (int rc = check_ptr(who, w, 4, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (add) if (int rc = check_ptr(who, add, 4, "add")) return rc;
+    if (y) if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    void* a[] = {(void*)&hidden, (void*)&add, (void*)&w, (void*)&y, (void*)&xq, (void*)&n, (void*)&eps};
+    return launch("add_rmsnorm_q8_f32", 1, n_vec, 1, fused_norm_block(n), 0, s, a);
+}
+
+int rein_swiglu_q8(const float* gate, const float* up, float* out, void* xq, unsigned n, rein_stream_t s)
+{
+    const char* who = "rein_swiglu_q8";
+    if (int rc = check_fused_n(who, n, 1, 0)) return rc;
+    if (int rc = check_ptr(who, gate, 4, "gate")) return rc;
+    if (int rc = check_ptr(who, up, 4, "up")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (out) if (int rc = check_ptr(who, out, 4, "out")) return rc;
+    void* a[] = {(void*)&gate, (void*)&up, (void*)&out, (void*)&xq, (void*)&n};
+    return launch("swiglu_q8_f32", elementwise_grid(n), 1, 1, 256, 0, s, a);
+}
+
+int rein_sigmoid_mul_q8(float* x, const float* gate, void* xq, unsigned n, rein_stream_t s)
+{
+    const char* who = "rein_sigmoid_mul_q8";
+    if (int rc = check_fused_n(who, n, 1, 0)) return rc;
+    if (int rc = check_ptr(who, x, 4, "x")) return rc;
+    if (int rc = check_ptr(who, gate, 4, "gate")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    void* a[] = {(void*)&x, (void*)&gate, (void*)&xq, (void*)&n};
+    return launch("sigmoid_mul_q8_f32", elementwise_grid(n), 1, 1, 256, 0, s, a);
+}
+
+int rein_rmsnorm_gated_q8(const float* x, const float* z, const float* w, float* y, void* xq, unsigned n_heads,
+                          unsigned head_dim, float eps, rein_stream_t s)
+{
+    const char* who = "rein_rmsnorm_gated_q8";
+    if (int rc = check_fused_n(who, head_dim, 1, 32768)) return rc;
+    if (n_heads == 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_heads is zero");
+    if (int rc = check_ptr(who, x, 4, "x")) return rc;
+    if (int rc = check_ptr(who, z, 4, "z")) return rc;
+    if (int rc = check_ptr(who, w, 4, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (y) if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    const unsigned block = std::max(64u, std::min(1024u, head_dim));
+    void* a[] = {(void*)&x, (void*)&z, (void*)&w, (void*)&y, (void*)&xq, (void*)&n_heads, (void*)&head_dim, (void*)&eps};
+    return launch("rmsnorm_gated_q8_f32", std::min(n_heads, kCUs * 16), 1, 1, block, 0, s, a);
+}
+
+int rein_moe_geglu_q8(const float* gu, void* xq, unsigned ff_exp, unsigned n_slot, rein_stream_t s)
+{
+    const char* who = "rein_moe_geglu_q8";
+    if (int rc = check_fused_n(who, ff_exp, n_slot, 0)) return rc;
+    if (int rc = check_ptr(who, gu, 4, "gu")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    void* a[] = {(void*)&gu, (void*)&xq, (void*)&ff_exp};
+    return launch("moe_geglu_q8_f32", (ff_exp + 511) / 512, n_slot, 1, 256, 0, s, a);
 }
 
 int rein_matvec_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
@@ -598,13 +700,13 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
                                        base + w.g_in, (float*)(base + w.e_gate), sh.hidden, sh.expert_ff, ne, s)) return rc;
     if (int rc = rein_moe_grouped_gemm(sh.gate_up_fmt, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
                                        base + w.g_in, (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;
-    if (int rc = rein_swiglu_mul((float*)(base + w.e_gate), (float*)(base + w.e_up), (float*)(base + w.e_gate),
-                                 ne * sh.expert_ff, s)) return rc;
-    // the quantizer's grid.y carries the row count: split long batches
-    for (unsigned r0 = 0; r0 < ne; r0 += 32768) {
-        const unsigned nr = ne - r0 < 32768 ? ne - r0 : 32768;
-        if (int rc = rein_quantize_q8((float*)(base + w.e_gate) + (size_t)r0 * sh.expert_ff,
-                                      base + w.xq_exp + (size_t)r0 * (sh.expert_ff / 32) * 40, sh.expert_ff, nr, s)) return rc;
+    // SwiGLU straight into the down projection's BlockQ8 rows (rows are expert_ff long,
+    // a multiple of 32, so the flat array quantizes as one vector)
+    for (size_t e0 = 0; e0 < (size_t)ne * sh.expert_ff; e0 += (size_t)1 << 30) {
+        const size_t left = (size_t)ne * sh.expert_ff - e0;
+        const unsigned cnt = (unsigned)std::min(left, (size_t)1 << 30);
+        if (int rc = rein_swiglu_q8((float*)(base + w.e_gate) + e0, (float*)(base + w.e_up) + e0, nullptr,
+                                    base + w.xq_exp + e0 / 32 * 40, cnt, s)) return rc;
     }
     if (int rc = rein_moe_grouped_gemm(sh.down_fmt, down_exps, (unsigned)bpe_dn, eoff, toff, sh.n_expert,
                                        base + w.xq_exp, (float*)(base + w.g_out), sh.expert_ff, sh.hidden, ne, s)) return rc;

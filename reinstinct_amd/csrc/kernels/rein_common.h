@@ -38,12 +38,15 @@ __device__ __forceinline__ int rein_dot4(int a, int b, int c)
 // ---- wave64 reductions over DPP (gfx9 row ops + row broadcasts) -------------
 // dpp_ctrl encodings: quad_perm = low 8 bits; row_half_mirror 0x141;
 // row_mirror 0x140; row_bcast15 0x142; row_bcast31 0x143.
-template <int CTRL, int ROW_MASK = 0xF>
+// row_shl:n 0x100+n (lane <- lane+n), row_shr:n 0x110+n (lane <- lane-n),
+// row_ror:n 0x120+n.  Lanes masked out by ROW_MASK / BANK_MASK (bank = 4 lanes of a
+// row) keep `old`.
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
 __device__ __forceinline__ float rein_dpp_f32(float old, float v)
 {
     return __builtin_bit_cast(
         float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v),
-                                           CTRL, ROW_MASK, 0xF, false));
+                                           CTRL, ROW_MASK, BANK_MASK, false));
 }
 
 // Sum over the 16 lanes of each DPP row; every lane of the row ends with it.

@@ -21,6 +21,36 @@ def quantize_q8(x, xq, in_dim, n_vec=1, stream=None):
     check(lib.rein_quantize_q8(_p(x), _p(xq), in_dim, n_vec, _s(stream)))
 
 
+def rmsnorm_q8(x, w, xq, n, n_vec=1, eps=1e-6, stream=None):
+    """rmsnorm_q8_f32 (kernels/rmsnorm_q8.cpp:38-103): xq = q8(rmsnorm(x) * w)"""
+    check(lib.rein_rmsnorm_q8(_p(x), _p(w), _p(xq), n, n_vec, eps, _s(stream)))
+
+
+def add_rmsnorm_q8(hidden, add, w, y, xq, n, n_vec=1, eps=1e-6, stream=None):
+    """add_rmsnorm_q8_f32 (kernels/qwen35_fused.cpp:66-121): hidden += add; y, xq = rmsnorm(hidden) * w"""
+    check(lib.rein_add_rmsnorm_q8(_p(hidden), _p(add), _p(w), _p(y), _p(xq), n, n_vec, eps, _s(stream)))
+
+
+def swiglu_q8(gate, up, out, xq, n, stream=None):
+    """swiglu_q8_f32 (kernels/qwen35_fused.cpp:132-146): out, xq = silu(gate) * up"""
+    check(lib.rein_swiglu_q8(_p(gate), _p(up), _p(out), _p(xq), n, _s(stream)))
+
+
+def sigmoid_mul_q8(x, gate, xq, n, stream=None):
+    """sigmoid_mul_q8_f32 (kernels/qwen35_fused.cpp:149-162): x *= sigmoid(gate); xq = q8(x)"""
+    check(lib.rein_sigmoid_mul_q8(_p(x), _p(gate), _p(xq), n, _s(stream)))
+
+
+def rmsnorm_gated_q8(x, z, w, y, xq, n_heads, head_dim, eps=1e-6, stream=None):
+    """rmsnorm_gated_q8_f32 (kernels/qwen35_fused.cpp:195-217)"""
+    check(lib.rein_rmsnorm_gated_q8(_p(x), _p(z), _p(w), _p(y), _p(xq), n_heads, head_dim, eps, _s(stream)))
+
+
+def moe_geglu_q8(gu, xq, ff_exp, n_slot, stream=None):
+    """moe_geglu_q8_f32 (kernels/moe_geglu_q8.cpp:31-66): xq = q8(gelu(gate) * up)"""
+    check(lib.rein_moe_geglu_q8(_p(gu), _p(xq), ff_exp, n_slot, _s(stream)))
+
+
 def matvec_xq8(fmt, w, xq, y, in_dim, out_dim, stream=None):
     """launch_matvec_repacked_xq8 (src/runtime/qwen35.rs:2232-2280)"""
     check(lib.rein_matvec_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, _s(stream)))
