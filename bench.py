@@ -251,6 +251,46 @@ def extras_moe(stream):
     return res
 
 
+def extras_moe_decode(stream):
+    """One decode token through the MoE expert FFN of configs[3] (128 experts, top-8, hidden 2048,
+    ff 768): fused gate+up+SwiGLU matvec (Q4_K) -> quantize -> down matvec (Q6_K) -> combine, expert
+    ids read on the device.  16 tokens with disjoint expert sets per graph, so every launch streams
+    experts that are not in cache."""
+    hidden, n_expert, n_used, ff = 2048, 128, 8, 768
+    gate1 = tiled_weights(rein.Q4_K, hidden, ff, seed=1, base_rows=ff)
+    up1 = tiled_weights(rein.Q4_K, hidden, ff, seed=2, base_rows=ff)
+    down1 = tiled_weights(rein.Q6_K, ff, hidden, seed=3, base_rows=hidden)
+    gate = hip.DeviceBuf.from_host(np.tile(gate1, n_expert))
+    up = hip.DeviceBuf.from_host(np.tile(up1, n_expert))
+    down = hip.DeviceBuf.from_host(np.tile(down1, n_expert))
+    per_token = (gate1.nbytes + up1.nbytes + down1.nbytes) * n_used
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((1, hidden)).astype(np.float32)
+    dxq = hip.DeviceBuf(hidden // 32 * 40)
+    runtime.quantize_q8(hip.DeviceBuf.from_host(x), dxq, hidden, 1, stream)
+    toks = n_expert // n_used
+    ids = [hip.DeviceBuf.from_host(np.arange(t * n_used, (t + 1) * n_used, dtype=np.int32)) for t in range(toks)]
+    wts = hip.DeviceBuf.from_host(np.full(n_used, 1.0 / n_used, np.float32))
+    ones = hip.DeviceBuf.from_host(np.ones(n_expert, np.float32))
+    act, aq = hip.DeviceBuf(n_used * ff * 4), hip.DeviceBuf(n_used * ff // 32 * 40)
+    eo, out = hip.DeviceBuf(n_used * hidden * 4), hip.DeviceBuf(hidden * 4)
+    ns_h, ns_f = hidden // 32, ff // 32
+
+    def token(t):
+        runtime.moe_gate_up_swiglu(rein.Q4_K, gate, up, ids[t], dxq, act, hidden, ff, gate1.nbytes, ns_h, 0, n_used, 1, stream)
+        runtime.quantize_q8(act, aq, ff, n_used, stream)
+        runtime.moe_down(rein.Q6_K, down, ids[t], aq, eo, ff, hidden, down1.nbytes, n_used * ns_f, ns_f, n_used, 1, stream)
+        runtime.moe_combine(eo, ids[t], wts, ones, out, 1, hidden, n_used, stream)
+
+    sec = time_graph(stream, lambda: [token(t) for t in range(toks)], toks)
+    res = {"workload": "MoE decode expert FFN, 1 token, 128 experts top-8, hidden 2048, ff 768: gate+up+SwiGLU (Q4_K) -> "
+                       "quantize -> down (Q6_K) -> combine, 4 launches",
+           "us_per_token": round(sec * 1e6, 2), "expert_bytes_per_token": per_token,
+           "GBs": round(per_token / sec / 1e9, 0), "frac_hbm_peak": round(per_token / sec / 1e9 / HBM_PEAK_GBS, 4)}
+    log("moe decode", res)
+    return res
+
+
 def extras_decode_stream(stream):
     """BASELINE configs[4]: 64 layers x {QKV 5120->7168, O 5120->5120, gate+up 5120->34816, down 17408->5120},
     Q4_K with every fourth layer's down and the 5120->151936 LM head in Q6_K, batch 1, one hipGraph."""
@@ -439,7 +479,8 @@ def main():
 
     if args.extras:
         out["extras"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
-                         "decode_stream_configs4": extras_decode_stream(stream), "fused_producers": extras_fused(stream)}
+                         "decode_stream_configs4": extras_decode_stream(stream), "fused_producers": extras_fused(stream),
+                         "moe_decode": extras_moe_decode(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)

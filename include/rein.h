@@ -222,6 +222,28 @@ int rein_moe_grouped_gemm(int fmt, const void *slab, unsigned bytes_per_expert,
                           const int32_t *expert_off, const int32_t *tile_off, unsigned n_expert,
                           const void *xq, float *y, unsigned in_dim, unsigned out_dim,
                           unsigned n_entries, rein_stream_t s);
+/* ---- MoE decode: expert matvecs, the expert id is read on the device.
+ * launch_moe_expert_matvec (qwen35.rs:3071-3100; kernels/moe_matvec_*_repacked.cpp):
+ * y[tok][slot][out_dim] = W[ids[tok*n_used+slot]] . xq row at
+ * xq + tok*xq_tok_stride + slot*xq_slot_stride (strides in BlockQ8 blocks; slot
+ * stride 0 = every slot reads the token's row).  Formats Q4_K, Q5_K, Q6_K, Q8_0. */
+int rein_moe_expert_matvec(int fmt, const void *slab, const int32_t *ids, const void *xq, float *y,
+                           unsigned in_dim, unsigned out_dim, unsigned bytes_per_expert,
+                           unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used,
+                           unsigned n_tok, rein_stream_t s);
+/* launch_moe_down (qwen35.rs:3102-3139; kernels/moe_matvec_{q5k,q6k}_down.cpp): the same
+ * product for the down projection, whose short contraction (expert_ff) is walked by
+ * half-wavefronts. */
+int rein_moe_down(int fmt, const void *slab, const int32_t *ids, const void *xq, float *y,
+                  unsigned in_dim, unsigned out_dim, unsigned bytes_per_expert,
+                  unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used, unsigned n_tok,
+                  rein_stream_t s);
+/* launch_moe_gate_up_swiglu (qwen35.rs:3141-3167; kernels/moe_gate_up_swiglu_q4k_repacked.cpp):
+ * y = silu(Wgate . xq) * (Wup . xq) in one pass over both slabs.  fmt must be Q4_K. */
+int rein_moe_gate_up_swiglu(int fmt, const void *gate_slab, const void *up_slab, const int32_t *ids,
+                            const void *xq, float *y, unsigned in_dim, unsigned out_dim,
+                            unsigned bytes_per_expert, unsigned xq_tok_stride,
+                            unsigned xq_slot_stride, unsigned n_used, unsigned n_tok, rein_stream_t s);
 /* swiglu_mul_f32 (kernels/swiglu.cpp:10-21) */
 int rein_swiglu_mul(const float *gate, const float *up, float *out, unsigned n, rein_stream_t s);
 /* moe_combine_f32 (kernels/moe_combine.cpp:15-38) */

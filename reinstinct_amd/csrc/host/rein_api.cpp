@@ -604,6 +604,76 @@ int rein_moe_grouped_gemm(int fmt, const void* slab, unsigned bytes_per_expert, 
     return launch(name, (out_dim + 127) / 128, tile_ub, 1, 256, 0, s, a);
 }
 
+namespace {
+int moe_mv_launch(const char* who, const std::string& kernel, unsigned rows_per_block, int fmt, const void* slab0,
+                  const void* slab1, const int32_t* ids, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                  unsigned bytes_per_expert, unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used,
+                  unsigned n_tok, rein_stream_t s)
+{
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_tok)) return rc;
+    if (n_used == 0 || n_used > 65535 || n_tok > 65535)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_used and n_tok must be in 1..65535");
+    if (bytes_per_expert < rein_repacked_len(fmt, in_dim, out_dim))
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert is smaller than one repacked expert");
+    if (int rc = check_ptr(who, slab0, 16, "slab")) return rc;
+    if (slab1) if (int rc = check_ptr(who, slab1, 16, "up_slab")) return rc;
+    if (bytes_per_expert % 16 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert must be a multiple of 16");
+    if (int rc = check_ptr(who, ids, 4, "ids")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    const unsigned gx = (out_dim + rows_per_block - 1) / rows_per_block;
+    if (slab1) {
+        void* a[] = {(void*)&slab0, (void*)&slab1, (void*)&ids, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim,
+                     (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
+        return launch(kernel, gx, n_used, n_tok, 256, 0, s, a);
+    }
+    void* a[] = {(void*)&slab0, (void*)&ids, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim,
+                 (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
+    return launch(kernel, gx, n_used, n_tok, 256, 0, s, a);
+}
+bool moe_mv_fmt(int fmt) { return fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q8_0; }
+}  // namespace
+
+int rein_moe_expert_matvec(int fmt, const void* slab, const int32_t* ids, const void* xq, float* y, unsigned in_dim,
+                           unsigned out_dim, unsigned bytes_per_expert, unsigned xq_tok_stride,
+                           unsigned xq_slot_stride, unsigned n_used, unsigned n_tok, rein_stream_t s)
+{
+    const char* who = "rein_moe_expert_matvec";
+    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    // 4 wavefronts x 2 rows per 256-thread workgroup (the reference's grid, qwen35.rs:3086)
+    return moe_mv_launch(who, std::string("moe_matvec_") + fmt_tag(fmt) + "_repacked_f32", 8, fmt, slab, nullptr, ids, xq,
+                         y, in_dim, out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, s);
+}
+
+int rein_moe_down(int fmt, const void* slab, const int32_t* ids, const void* xq, float* y, unsigned in_dim,
+                  unsigned out_dim, unsigned bytes_per_expert, unsigned xq_tok_stride, unsigned xq_slot_stride,
+                  unsigned n_used, unsigned n_tok, rein_stream_t s)
+{
+    const char* who = "rein_moe_down";
+    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (in_dim / 32 > 32)       // long contraction: the full-wavefront mapping wastes nothing
+        return rein_moe_expert_matvec(fmt, slab, ids, xq, y, in_dim, out_dim, bytes_per_expert, xq_tok_stride,
+                                      xq_slot_stride, n_used, n_tok, s);
+    const std::string kernel = fmt == REIN_TYPE_Q4_K   ? "rein_moe_matvec_q4k_down_f32"
+                               : fmt == REIN_TYPE_Q8_0 ? "moe_matvec_q8_0_repacked_down_f32"
+                                                       : std::string("moe_matvec_") + fmt_tag(fmt) + "_down_f32";
+    // 8 half-wavefronts x 2 rows per workgroup
+    return moe_mv_launch(who, kernel, 16, fmt, slab, nullptr, ids, xq, y, in_dim, out_dim, bytes_per_expert,
+                         xq_tok_stride, xq_slot_stride, n_used, n_tok, s);
+}
+
+int rein_moe_gate_up_swiglu(int fmt, const void* gate_slab, const void* up_slab, const int32_t* ids, const void* xq,
+                            float* y, unsigned in_dim, unsigned out_dim, unsigned bytes_per_expert,
+                            unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used, unsigned n_tok,
+                            rein_stream_t s)
+{
+    const char* who = "rein_moe_gate_up_swiglu";
+    if (fmt != REIN_TYPE_Q4_K) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": the fused form exists for Q4_K experts");
+    if (!up_slab) return fail(REIN_E_BAD_POINTER, std::string(who) + ": up_slab is NULL");
+    return moe_mv_launch(who, "moe_gate_up_swiglu_q4k_repacked_f32", 8, fmt, gate_slab, up_slab, ids, xq, y, in_dim,
+                         out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, s);
+}
+
 int rein_swiglu_mul(const float* gate, const float* up, float* out, unsigned n, rein_stream_t s)
 {
     if (n == 0) return fail(REIN_E_BAD_SHAPE, "rein_swiglu_mul: n is zero");

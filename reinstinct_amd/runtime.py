@@ -105,6 +105,27 @@ def moe_grouped_gemm(fmt, slab, bytes_per_expert, expert_off, tile_off, n_expert
                                     _p(xq), _p(y), in_dim, out_dim, n_entries, _s(stream)))
 
 
+def moe_expert_matvec(fmt, slab, ids, xq, y, in_dim, out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride,
+                      n_used, n_tok=1, stream=None):
+    """launch_moe_expert_matvec (src/runtime/qwen35.rs:3071-3100)"""
+    check(lib.rein_moe_expert_matvec(fmt, _p(slab), _p(ids), _p(xq), _p(y), in_dim, out_dim, bytes_per_expert,
+                                     xq_tok_stride, xq_slot_stride, n_used, n_tok, _s(stream)))
+
+
+def moe_down(fmt, slab, ids, xq, y, in_dim, out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used,
+             n_tok=1, stream=None):
+    """launch_moe_down (src/runtime/qwen35.rs:3102-3139)"""
+    check(lib.rein_moe_down(fmt, _p(slab), _p(ids), _p(xq), _p(y), in_dim, out_dim, bytes_per_expert,
+                            xq_tok_stride, xq_slot_stride, n_used, n_tok, _s(stream)))
+
+
+def moe_gate_up_swiglu(fmt, gate_slab, up_slab, ids, xq, y, in_dim, out_dim, bytes_per_expert, xq_tok_stride,
+                       xq_slot_stride, n_used, n_tok=1, stream=None):
+    """launch_moe_gate_up_swiglu (src/runtime/qwen35.rs:3141-3167)"""
+    check(lib.rein_moe_gate_up_swiglu(fmt, _p(gate_slab), _p(up_slab), _p(ids), _p(xq), _p(y), in_dim, out_dim,
+                                      bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, _s(stream)))
+
+
 def swiglu_mul(gate, up, out, n, stream=None):
     check(lib.rein_swiglu_mul(_p(gate), _p(up), _p(out), n, _s(stream)))
 
