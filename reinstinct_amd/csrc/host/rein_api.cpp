@@ -701,7 +701,7 @@ int rein_moe_combine(const float* experts, const int32_t* ids, const float* weig
 // Workspace carve-up for rein_moe_ffn (all offsets 256-byte aligned).
 namespace {
 struct MoeWs {
-    size_t ids, weights, count, cursor, perm, eoff, toff, xq_in, g_in, e_gate, e_up, xq_exp, g_out, e_out, total;
+    size_t ids, weights, count, cursor, perm, inv, eoff, toff, xq_in, g_in, e_gate, e_up, xq_exp, g_out, total;
 };
 size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 MoeWs moe_ws(const rein_moe_shape& sh)
@@ -715,6 +715,7 @@ MoeWs moe_ws(const rein_moe_shape& sh)
     w.count   = take((size_t)sh.n_expert * 4);
     w.cursor  = take((size_t)sh.n_expert * 4);
     w.perm    = take(ne * 4);
+    w.inv     = take(ne * 4);
     w.eoff    = take(((size_t)sh.n_expert + 1) * 4);
     w.toff    = take(((size_t)sh.n_expert + 1) * 4);
     w.xq_in   = take((size_t)sh.n_tok * (sh.hidden / 32) * 40);
@@ -723,7 +724,6 @@ MoeWs moe_ws(const rein_moe_shape& sh)
     w.e_up    = take(ne * sh.expert_ff * 4);
     w.xq_exp  = take(ne * (sh.expert_ff / 32) * 40);
     w.g_out   = take(ne * sh.hidden * 4);
-    w.e_out   = take(ne * sh.hidden * 4);
     w.total   = o;
     return w;
 }
@@ -747,10 +747,22 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     if (int rc = check_shape(who, sh.gate_up_fmt, sh.hidden, sh.expert_ff, sh.n_tok)) return rc;
     if (int rc = check_shape(who, sh.down_fmt, sh.expert_ff, sh.hidden, sh.n_tok)) return rc;
     if (int rc = check_ptr(who, workspace, 256, "workspace")) return rc;
+    if (!moe_mv_fmt(sh.gate_up_fmt) || !moe_mv_fmt(sh.down_fmt))
+        return fail(REIN_E_BAD_FORMAT, std::string(who) + ": expert formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (sh.n_tok > 65535) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most 65535 tokens per call");
+    if (int rc = check_ptr(who, x, 4, "x")) return rc;
+    if (int rc = check_ptr(who, logits, 4, "logits")) return rc;
+    if (int rc = check_ptr(who, gate_exps, 16, "gate_exps")) return rc;
+    if (int rc = check_ptr(who, up_exps, 16, "up_exps")) return rc;
+    if (int rc = check_ptr(who, down_exps, 16, "down_exps")) return rc;
+    if (int rc = check_ptr(who, down_exps_s, 4, "down_exps_s")) return rc;
+    if (int rc = check_ptr(who, out, 4, "out")) return rc;
     const size_t bpe_gu = rein_repacked_len(sh.gate_up_fmt, sh.hidden, sh.expert_ff);
     const size_t bpe_dn = rein_repacked_len(sh.down_fmt, sh.expert_ff, sh.hidden);
     if (bpe_gu > 0xFFFFFFFFull || bpe_dn > 0xFFFFFFFFull)
         return fail(REIN_E_TOO_LARGE, std::string(who) + ": an expert slab must stay below 4 GiB");   // u32, qwen35.rs:3052
+    if (bpe_gu % 16 != 0 || bpe_dn % 16 != 0)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": expert slabs must be multiples of 16 bytes (hidden and expert_ff multiples of 8 rows)");
 
     const MoeWs w = moe_ws(sh);
     char* base = static_cast<char*>(workspace);
@@ -763,13 +775,39 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
 
     if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
     if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
-    if (int rc = rein_moe_sort(ids, ne, sh.n_expert, rein_moe_gemm_bn(), (int32_t*)(base + w.count),
-                               (int32_t*)(base + w.cursor), perm, eoff, toff, s)) return rc;
+    // counting sort by expert (moe_expert_sort.hip), with the inverse permutation kept so
+    // that the combine can read the sorted expert outputs in place
+    {
+        int32_t* count = (int32_t*)(base + w.count);
+        int32_t* cursor = (int32_t*)(base + w.cursor);
+        int32_t* inv = (int32_t*)(base + w.inv);
+        const unsigned bn = rein_moe_gemm_bn();
+        const unsigned zn = (unsigned)((w.cursor - w.count) / 4) + sh.n_expert;     // count .. cursor are adjacent
+        const unsigned gn = (ne + 255) / 256;
+        void* a0[] = {(void*)&count, (void*)&zn};
+        if (int rc = launch("moe_sort_zero", (zn + 255) / 256, 1, 1, 256, 0, s, a0)) return rc;
+        void* a1[] = {(void*)&ids, (void*)&count, (void*)&ne, (void*)&sh.n_expert};
+        if (int rc = launch("moe_sort_histogram", gn, 1, 1, 256, 0, s, a1)) return rc;
+        void* a2[] = {(void*)&count, (void*)&eoff, (void*)&toff, (void*)&sh.n_expert, (void*)&bn};
+        if (int rc = launch("moe_sort_scan", 1, 1, 1, 64, 0, s, a2)) return rc;
+        void* a3[] = {(void*)&ids, (void*)&eoff, (void*)&cursor, (void*)&perm, (void*)&inv, (void*)&ne, (void*)&sh.n_expert};
+        if (int rc = launch("rein_moe_sort_scatter_inv", gn, 1, 1, 256, 0, s, a3)) return rc;
+    }
     if (int rc = rein_moe_gather_xq(base + w.xq_in, perm, base + w.g_in, sh.hidden / 32, sh.n_used, ne, s)) return rc;
-    if (int rc = rein_moe_grouped_gemm(sh.gate_up_fmt, gate_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
-                                       base + w.g_in, (float*)(base + w.e_gate), sh.hidden, sh.expert_ff, ne, s)) return rc;
-    if (int rc = rein_moe_grouped_gemm(sh.gate_up_fmt, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
-                                       base + w.g_in, (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;
+    // gate and up projections in one launch (grid.z = 2)
+    {
+        const unsigned bn = rein_moe_gemm_bn();
+        unsigned tile_ub = (ne + bn - 1) / bn + sh.n_expert;
+        if (tile_ub > 65535) tile_ub = 65535;
+        const unsigned bpe = (unsigned)bpe_gu;
+        const void* xq_in = base + w.g_in;
+        float* y0 = (float*)(base + w.e_gate);
+        float* y1 = (float*)(base + w.e_up);
+        const std::string name = std::string("rein_mmq_") + fmt_tag(sh.gate_up_fmt) + "_grouped_pair";
+        void* a[] = {(void*)&gate_exps, (void*)&up_exps, (void*)&bpe, (void*)&eoff, (void*)&toff, (void*)&sh.n_expert,
+                     (void*)&xq_in, (void*)&y0, (void*)&y1, (void*)&sh.hidden, (void*)&sh.expert_ff};
+        if (int rc = launch(name, (sh.expert_ff + 127) / 128, tile_ub, 2, 256, 0, s, a)) return rc;
+    }
     // SwiGLU straight into the down projection's BlockQ8 rows (rows are expert_ff long,
     // a multiple of 32, so the flat array quantizes as one vector)
     for (size_t e0 = 0; e0 < (size_t)ne * sh.expert_ff; e0 += (size_t)1 << 30) {
@@ -780,8 +818,14 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     }
     if (int rc = rein_moe_grouped_gemm(sh.down_fmt, down_exps, (unsigned)bpe_dn, eoff, toff, sh.n_expert,
                                        base + w.xq_exp, (float*)(base + w.g_out), sh.expert_ff, sh.hidden, ne, s)) return rc;
-    if (int rc = rein_moe_scatter_rows((float*)(base + w.g_out), perm, (float*)(base + w.e_out), sh.hidden, ne, s)) return rc;
-    return rein_moe_combine((float*)(base + w.e_out), ids, weights, down_exps_s, out, sh.n_tok, sh.hidden, sh.n_used, s);
+    // scatter + weighted combine in one pass over the sorted rows
+    {
+        const float* sorted = (const float*)(base + w.g_out);
+        const int32_t* inv = (const int32_t*)(base + w.inv);
+        void* a[] = {(void*)&sorted, (void*)&inv, (void*)&ids, (void*)&weights, (void*)&down_exps_s, (void*)&out,
+                     (void*)&sh.hidden, (void*)&sh.n_used};
+        return launch("rein_moe_combine_sorted_f32", (sh.hidden + 255) / 256, sh.n_tok, 1, 256, 0, s, a);
+    }
 }
 
 }  // extern "C"

@@ -885,6 +885,22 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     }
 }
 
+// Two grouped GEMMs over the same sorted activations in one launch (the gate and up
+// projections of an expert FFN): blockIdx.z selects the slab and its output.  Twice
+// the workgroups per launch fill the machine better than two launches of half the
+// size, and the second launch's fill / drain disappears.
+template <int FMT>
+__device__ __forceinline__ void rein_mmq_grouped_pair(const uint8_t* __restrict__ slab0, const uint8_t* __restrict__ slab1,
+                                                      unsigned bytes_per_expert, const int* __restrict__ expert_off,
+                                                      const int* __restrict__ tile_off, unsigned n_expert,
+                                                      const BlockQ8* __restrict__ xq, float* __restrict__ y0,
+                                                      float* __restrict__ y1, unsigned in_dim, unsigned out_dim)
+{
+    for (unsigned z = blockIdx.z; z < 2u; z += gridDim.z)
+        rein_mmq_grouped<FMT>(z ? slab1 : slab0, bytes_per_expert, expert_off, tile_off, n_expert, xq, z ? y1 : y0,
+                              in_dim, out_dim);
+}
+
 // Two wavefronts per SIMD: a 256-register budget, which makes the compiler keep
 // MFMA results in ordinary VGPRs (no AGPR round trips) without spilling.
 #define REIN_MMQ_OCC __attribute__((amdgpu_waves_per_eu(2)))
@@ -923,4 +939,15 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     {                                                                                            \
         rein_mmq_grouped<FMT>(slab, bytes_per_expert, expert_off, tile_off, n_expert, xq, y,     \
                               in_dim, out_dim);                                                  \
+    }
+
+#define REIN_DEFINE_MMQ_GROUPED_PAIR(name, FMT)                                                  \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                         \
+        const unsigned char* __restrict__ slab0, const unsigned char* __restrict__ slab1,        \
+        unsigned int bytes_per_expert, const int* __restrict__ expert_off,                       \
+        const int* __restrict__ tile_off, unsigned int n_expert, const BlockQ8* __restrict__ xq, \
+        float* __restrict__ y0, float* __restrict__ y1, unsigned int in_dim, unsigned int out_dim) \
+    {                                                                                            \
+        rein_mmq_grouped_pair<FMT>(slab0, slab1, bytes_per_expert, expert_off, tile_off,         \
+                                   n_expert, xq, y0, y1, in_dim, out_dim);                       \
     }

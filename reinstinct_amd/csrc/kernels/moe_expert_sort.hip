@@ -100,3 +100,20 @@ extern "C" __global__ void moe_scatter_rows(const float* __restrict__ src, const
         for (unsigned c = blockIdx.x * blockDim.x + threadIdx.x; c < dim; c += gridDim.x * blockDim.x) d[c] = s[c];
     }
 }
+
+// moe_sort_scatter that also records where each routing entry went: inv[i] = position
+// of entry i in the sorted order (perm[inv[i]] == i).  Lets the combine read the
+// sorted expert outputs directly instead of through a scatter pass.
+extern "C" __global__ void rein_moe_sort_scatter_inv(const int* __restrict__ ids, const int* __restrict__ expert_off,
+                                                     int* __restrict__ cursor, int* __restrict__ perm,
+                                                     int* __restrict__ inv, unsigned int n_entries,
+                                                     unsigned int n_expert)
+{
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n_entries; i += gridDim.x * blockDim.x) {
+        const int e = ids[i];
+        if (e < 0 || (unsigned)e >= n_expert) { inv[i] = -1; continue; }
+        const int pos = expert_off[e] + atomicAdd(&cursor[e], 1);
+        perm[pos] = (int)i;
+        inv[i] = pos;
+    }
+}

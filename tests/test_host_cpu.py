@@ -128,7 +128,9 @@ def test_moe_workspace_layout():
     sh = runtime.moe_shape(512, 2048, 128, 8, 768, rein.Q4_K, rein.Q6_K)
     n = runtime.moe_workspace_bytes(sh)
     ne = 512 * 8
-    need = ne * 4 * 3 + 128 * 4 * 2 + 129 * 4 * 2 + 512 * 64 * 40 + ne * 64 * 40 + ne * 768 * 4 * 2 + ne * 24 * 40 \
-        + ne * 2048 * 4 * 2
+    # ids, weights, perm, inverse perm; count, cursor; two offset arrays; quantized x; gathered x;
+    # gate and up outputs; quantized intermediate; sorted down outputs (combined in place)
+    need = ne * 4 * 4 + 128 * 4 * 2 + 129 * 4 * 2 + 512 * 64 * 40 + ne * 64 * 40 + ne * 768 * 4 * 2 + ne * 24 * 40 \
+        + ne * 2048 * 4
     assert need <= n <= need + 14 * 256
     assert runtime.moe_gemm_bn() == 32
