@@ -291,6 +291,50 @@ def extras_moe_decode(stream):
     return res
 
 
+def extras_ondisk(stream):
+    """The matvec call sites outside the repacked path: the tied LM head in on-disk Q6_K blocks
+    (5120 -> 151936, 638 MB) and the split-K Q8_0 matvec for a tiny projection (5120 -> 96)."""
+    out = []
+    k, n = 5120, 151936
+    w = (np.random.default_rng(0).standard_normal((1024, k)) * 0.02).astype(np.float32)
+    raw = np.tile(quant.quantize_weights(rein.Q6_K, w), n // 1024 + 1)[: n * (k // 256) * 210]
+    dw = [hip.DeviceBuf.from_host(raw) for _ in range(2)]
+    x = np.random.default_rng(1).standard_normal((1, k)).astype(np.float32)
+    dq = hip.DeviceBuf(k // 32 * 40)
+    runtime.quantize_q8(hip.DeviceBuf.from_host(x), dq, k, 1, stream)
+    dy = hip.DeviceBuf(n * 4)
+    sec = time_graph(stream, lambda: [runtime.matvec_ondisk_xq8(rein.Q6_K, b, dq, dy, k, n, stream) for b in dw], 2)
+    out.append({"op": "on-disk Q6_K matvec 5120 -> 151936 (tied LM head)", "us": round(sec * 1e6, 1),
+                "GBs": round(raw.nbytes / sec / 1e9, 0), "frac_hbm_peak": round(raw.nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)})
+    packed = quant.repack_for_matvec(rein.Q6_K, raw, k, n)
+    dp = [hip.DeviceBuf.from_host(packed) for _ in range(2)]
+    sec = time_graph(stream, lambda: [runtime.matvec_xq8(rein.Q6_K, b, dq, dy, k, n, stream) for b in dp], 2)
+    out.append({"op": "repacked Q6_K matvec, same matrix", "us": round(sec * 1e6, 1),
+                "GBs": round(packed.nbytes / sec / 1e9, 0), "frac_hbm_peak": round(packed.nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)})
+    del dw, dp
+    # the decode kernel away from the launch ramp: the same K = 5120 contraction, Q4_K, at the
+    # vocabulary-sized N (450 MB per launch)
+    p4 = tiled_weights(rein.Q4_K, k, n, seed=4)
+    d4 = [hip.DeviceBuf.from_host(p4) for _ in range(2)]
+    sec = time_graph(stream, lambda: [runtime.matvec_xq8(rein.Q4_K, b, dq, dy, k, n, stream) for b in d4], 2)
+    out.append({"op": "repacked Q4_K matvec 5120 -> 151936 (450 MB per launch)", "us": round(sec * 1e6, 1),
+                "GBs": round(p4.nbytes / sec / 1e9, 0), "frac_hbm_peak": round(p4.nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)})
+    del d4
+    n2 = 96
+    w8 = quant.repack_for_matvec(rein.Q8_0, quant.quantize_weights(rein.Q8_0, w[:n2]), k, n2)
+    d8 = hip.DeviceBuf.from_host(w8)
+    yp = hip.DeviceBuf(16 * n2 * 4)
+    reps = 32
+    for ns in (1, 4, 8, 16):
+        sec = time_graph(stream, lambda: [runtime.matvec_q8_0_splitk(d8, dq, yp, k, n2, ns, stream) for _ in range(reps)], reps)
+        out.append({"op": f"Q8_0 split-K matvec 5120 -> 96, n_split {ns}", "us": round(sec * 1e6, 2)})
+    sec = time_graph(stream, lambda: [runtime.matvec_xq8(rein.Q8_0, d8, dq, yp, k, n2, stream) for _ in range(reps)], reps)
+    out.append({"op": "Q8_0 matvec 5120 -> 96 without the split", "us": round(sec * 1e6, 2)})
+    for r in out:
+        log("ondisk", r)
+    return out
+
+
 def extras_decode_stream(stream):
     """BASELINE configs[4]: 64 layers x {QKV 5120->7168, O 5120->5120, gate+up 5120->34816, down 17408->5120},
     Q4_K with every fourth layer's down and the 5120->151936 LM head in Q6_K, batch 1, one hipGraph."""
@@ -451,6 +495,24 @@ def main():
                      "algorithmic_bytes_per_launch": dom["bytes_per_launch"]},
     }
 
+    if is_headline:
+        # the same kernel and contraction (Q4_K, K = 5120) where one launch is long enough for the
+        # launch / ramp time not to matter: the vocabulary-sized N = 151936, 450 MB per launch
+        k, n = 5120, 151936
+        p4 = tiled_weights(rein.Q4_K, k, n, seed=4)
+        d4 = [hip.DeviceBuf.from_host(p4) for _ in range(2)]
+        xq = hip.DeviceBuf(k // 32 * 40)
+        runtime.quantize_q8(hip.DeviceBuf.from_host(np.random.default_rng(1).standard_normal((1, k)).astype(np.float32)),
+                            xq, k, 1, stream)
+        dy = hip.DeviceBuf(n * 4)
+        sec = time_graph(stream, lambda: [runtime.matvec_xq8(rein.Q4_K, b, xq, dy, k, n, stream) for b in d4], 2)
+        nbytes = p4.nbytes + k // 32 * 40 + n * 4
+        out["large_n"] = {"workload": "Q4_K decode matvec K=5120 -> N=151936, batch 1 (same kernel, 450 MB per launch)",
+                          "us_per_launch": round(sec * 1e6, 1), "GBs": round(nbytes / sec / 1e9, 0),
+                          "frac_of_hbm_peak": round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)}
+        log("large N:", out["large_n"])
+        del d4, p4
+
     if not args.no_mmq:
         mm = MmqCase(rein.Q4_K, 512, 5120, 17408, stream, seed=77)
         sec = mm.time(max(4, min(args.steps, 20)), 2)
@@ -480,7 +542,7 @@ def main():
     if args.extras:
         out["extras"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
                          "decode_stream_configs4": extras_decode_stream(stream), "fused_producers": extras_fused(stream),
-                         "moe_decode": extras_moe_decode(stream)}
+                         "moe_decode": extras_moe_decode(stream), "other_matvec_sites": extras_ondisk(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)

@@ -176,6 +176,18 @@ int rein_matvec_xq8(int fmt, const void *w, const void *xq, float *y, unsigned i
  * 448-508): y[n_rows][out_dim], 1 <= n_rows <= 8; the weights are streamed once. */
 int rein_matvec_batched_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                             unsigned out_dim, unsigned n_rows, rein_stream_t s);
+/* The on-disk-layout matvec (src/runtime/qwen35.rs:2209-2229; kernels/matvec_q4_k_dp4a.cpp
+ * and its Q5_K / Q6_K / Q8_0 siblings): `w_blocks` holds out_dim rows of GGUF blocks as
+ * they are on disk (not repacked) -- the path a tied token_embd / output matrix takes.
+ * Formats Q4_K, Q5_K, Q6_K, Q8_0; w_blocks 16-byte aligned. */
+int rein_matvec_ondisk_xq8(int fmt, const void *w_blocks, const void *xq, float *y, unsigned in_dim,
+                           unsigned out_dim, rein_stream_t s);
+/* matvec_q8_0_repacked_splitk_f32 (kernels/matvec_q8_0_repacked.cpp:117-176): repacked
+ * Q8_0, the contraction split into n_split ranges of ceil(n_sub/n_split) sub-blocks;
+ * y_partials [n_split][out_dim] receives one partial sum per range, the caller adds
+ * them.  For projections whose out_dim is too small to fill the machine. */
+int rein_matvec_q8_0_splitk(const void *w, const void *xq, float *y_partials, unsigned in_dim,
+                            unsigned out_dim, unsigned n_split, rein_stream_t s);
 /* matmul_mmq_into without its quantize step (src/runtime/prefill.rs:512-567):
  * Y[p_rows][out_dim] = Xq . W^T on the int8 MFMA path. */
 int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,

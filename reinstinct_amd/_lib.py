@@ -81,6 +81,8 @@ SIGNATURES = {
     "rein_moe_scatter_rows": (_i, [_vp, _vp, _vp, _u, _u, _vp]),
     "rein_moe_grouped_gemm": (_i, [_i, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
     "rein_swiglu_mul": (_i, [_vp, _vp, _vp, _u, _vp]),
+    "rein_matvec_ondisk_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _vp]),
+    "rein_matvec_q8_0_splitk": (_i, [_vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_moe_expert_matvec": (_i, [_i, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
     "rein_moe_down": (_i, [_i, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
     "rein_moe_gate_up_swiglu": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),

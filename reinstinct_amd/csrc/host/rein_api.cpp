@@ -432,6 +432,37 @@ int rein_matvec_batched_xq8(int fmt, const void* w, const void* xq, float* y, un
     return launch_matvec("rein_matvec_batched_xq8", fmt, w, xq, y, in_dim, out_dim, n_rows, s);
 }
 
+int rein_matvec_ondisk_xq8(int fmt, const void* w_blocks, const void* xq, float* y, unsigned in_dim,
+                           unsigned out_dim, rein_stream_t s)
+{
+    const char* who = "rein_matvec_ondisk_xq8";
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, 1)) return rc;
+    const char* name = fmt == REIN_TYPE_Q4_K ? "matvec_q4_k_dp4a_f32" : fmt == REIN_TYPE_Q5_K ? "matvec_q5_k_dp4a_f32"
+                     : fmt == REIN_TYPE_Q6_K ? "matvec_q6_k_dp4a_f32" : fmt == REIN_TYPE_Q8_0 ? "matvec_q8_0_dp4a_f32" : nullptr;
+    if (!name) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (int rc = check_ptr(who, w_blocks, 16, "w_blocks")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    // 4 wavefronts x 2 rows per workgroup; the kernel strides, so cap the grid at a few waves per SIMD
+    const unsigned gx = std::min((out_dim + 7) / 8, kCUs * 16);
+    void* a[] = {(void*)&w_blocks, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim};
+    return launch(name, gx, 1, 1, 256, 0, s, a);
+}
+
+int rein_matvec_q8_0_splitk(const void* w, const void* xq, float* y_partials, unsigned in_dim, unsigned out_dim,
+                            unsigned n_split, rein_stream_t s)
+{
+    const char* who = "rein_matvec_q8_0_splitk";
+    if (int rc = check_shape(who, REIN_TYPE_Q8_0, in_dim, out_dim, 1)) return rc;
+    if (n_split == 0 || n_split > 65535) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_split must be in 1..65535");
+    if (int rc = check_ptr(who, w, 16, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y_partials, 4, "y_partials")) return rc;
+    void* a[] = {(void*)&w, (void*)&xq, (void*)&y_partials, (void*)&in_dim, (void*)&out_dim, (void*)&n_split};
+    // one wavefront per row pair, as the reference (block 64, grid (ceil(out/2), n_split))
+    return launch("matvec_q8_0_repacked_splitk_f32", (out_dim + 1) / 2, n_split, 1, 64, 0, s, a);
+}
+
 int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
                  unsigned p_rows, rein_stream_t s)
 {

@@ -61,6 +61,16 @@ def matvec_batched_xq8(fmt, w, xq, y, in_dim, out_dim, n_rows, stream=None):
     check(lib.rein_matvec_batched_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, n_rows, _s(stream)))
 
 
+def matvec_ondisk_xq8(fmt, w_blocks, xq, y, in_dim, out_dim, stream=None):
+    """the on-disk-layout dp4a matvec (src/runtime/qwen35.rs:2209-2229)"""
+    check(lib.rein_matvec_ondisk_xq8(fmt, _p(w_blocks), _p(xq), _p(y), in_dim, out_dim, _s(stream)))
+
+
+def matvec_q8_0_splitk(w, xq, y_partials, in_dim, out_dim, n_split, stream=None):
+    """matvec_q8_0_repacked_splitk_f32 (kernels/matvec_q8_0_repacked.cpp:117-176)"""
+    check(lib.rein_matvec_q8_0_splitk(_p(w), _p(xq), _p(y_partials), in_dim, out_dim, n_split, _s(stream)))
+
+
 def mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, stream=None):
     """matmul_mmq_into minus its quantize (src/runtime/prefill.rs:512-567)"""
     check(lib.rein_mmq_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _s(stream)))
