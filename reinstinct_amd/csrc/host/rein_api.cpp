@@ -156,12 +156,12 @@ unsigned batch_slot(unsigned n_rows) { return n_rows <= 1 ? 1 : n_rows <= 2 ? 2 
 int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
                   unsigned n_rows, rein_stream_t s)
 {
-    const unsigned nv = n_rows <= 8 ? 4 : 8, tok = 2 * nv;
+    const unsigned nv = n_rows <= 2 ? 1 : n_rows <= 4 ? 2 : n_rows <= 8 ? 4 : 8, tok = 2 * nv;
     const unsigned tiles = ((out_dim + 31) / 32) * ((n_rows + tok - 1) / tok);
     const unsigned n_chunks = (in_dim / 32 + 7) / 8;
     const unsigned planes = fmt == REIN_TYPE_Q8_0 ? 2 : 1;
     const unsigned lds_per_wave = planes * 4096 + 320 * tok;                       // sizeof(SkinnyWaveLds<FMT, TOK>)
-    const bool three = nv == 4 && (fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q8_0 ||
+    const bool three = nv <= 4 && (fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q8_0 ||
                                    fmt == REIN_TYPE_IQ4_XS);
     const unsigned occ = three ? 3 : 2;                                            // wavefronts per SIMD (registers)
     const unsigned waves_per_cu = std::min(4 * occ, 160u * 1024u / lds_per_wave);
@@ -189,13 +189,17 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
 }
 
 // Activation rows from which the batched decode leaves the dot4 kernels for the
-// skinny MMQ.  Measured on MI355X, 5120 -> 34816: Q4_K dot4 takes 21 / 28 / 39 / 39 us
-// at 1 / 2 / 3 / 4 rows (three rows run in the four-row kernel), the skinny MMQ 33 us
-// for anything up to 8 rows; Q4_0, Q8_0 and IQ4_XS behave alike.  Q5_K and Q6_K carry
-// more aux words per sub-block: there the skinny MMQ only wins from 5 rows.
-unsigned skinny_from_rows(int fmt)
+// skinny MMQ.  v_dot4 is a quarter-rate instruction on this part, so every extra row
+// costs the dot4 kernels ~7 us at 5120 -> 34816 (Q4_K: 21 / 28 / 39 us at 1 / 2 / 3-4
+// rows) while the skinny MMQ takes 27 / 30 / 33 us for up to 2 / 4 / 8 rows.  Two rows
+// stay on dot4 (level at large N, faster at small N) except for Q8_0 at large N;
+// Q6_K (two MFMAs and the most aux words per sub-block) switches at 5.
+unsigned skinny_from_rows(int fmt, unsigned out_dim)
 {
-    return env_u("REIN_SKINNY_FROM", fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q6_K ? 5 : 3);
+    unsigned dflt = 3;
+    if (fmt == REIN_TYPE_Q6_K) dflt = 5;
+    if (fmt == REIN_TYPE_Q8_0 && out_dim >= 16384) dflt = 2;
+    return env_u("REIN_SKINNY_FROM", dflt);
 }
 
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
@@ -207,7 +211,7 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
-    if (n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (n_rows >= skinny_from_rows(fmt, out_dim) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(out_dim, b);
     const unsigned wpb = 4;
@@ -471,7 +475,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt, out_dim) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // Token tile.  The 64-token tile does about 6 % more work per cycle when the
     // machine is evenly loaded (the weight unpack is shared by two MFMA tiles), but two
     // of its workgroups fit a CU against three of the 32-token tile (registers), so the

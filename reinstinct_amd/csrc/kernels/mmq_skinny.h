@@ -214,7 +214,7 @@ __device__ __forceinline__ void rein_skinny_wstash(SkinnyWImage<FMT>& l, const S
 // branch makes its destination a merge of two values, which costs copies and a wait
 // right behind the load.  `live == false` points every lane at the first bytes of the
 // plane instead (one cache line, always valid) and the result is never used.
-template <int TOK> struct SkinnyARegs { BlockQ8 b[TOK * 8 / 64]; };
+template <int TOK> struct SkinnyARegs { BlockQ8 b[(TOK * 8 + 63) / 64]; };      // TOK < 8: lanes past TOK*8 idle
 template <int TOK>
 struct SkinnyAct {
     uint4 qs[2][8][TOK];                                 // [half][sub-block][row]
@@ -228,8 +228,8 @@ __device__ __forceinline__ void rein_skinny_afetch(SkinnyARegs<TOK>& r, const Bl
                                                    bool live)
 {
 #pragma unroll
-    for (int k = 0; k < TOK * 8 / 64; k++) {
-        const unsigned e = 64u * k + lane;
+    for (int k = 0; k < (TOK * 8 + 63) / 64; k++) {
+        const unsigned e = min(64u * k + lane, TOK * 8u - 1u);
         const unsigned tok = min(tok_base + e % TOK, tok_end - 1u), sb = rein_clamp_sb(sb0 + e / TOK, n_sub);
         r.b[k] = *(live ? xq + (size_t)tok * n_sub + sb : xq);
     }
@@ -239,8 +239,9 @@ template <int TOK, bool XS>
 __device__ __forceinline__ void rein_skinny_astash(SkinnyAct<TOK>& a, const SkinnyARegs<TOK>& r, unsigned lane)
 {
 #pragma unroll
-    for (int k = 0; k < TOK * 8 / 64; k++) {
+    for (int k = 0; k < (TOK * 8 + 63) / 64; k++) {
         const unsigned e = 64u * k + lane;
+        if (TOK * 8 < 64 && e >= TOK * 8u) continue;
         const BlockQ8& b = r.b[k];
         a.qs[0][e / TOK][e % TOK] = make_uint4((unsigned)b.qs[0], (unsigned)b.qs[1], (unsigned)b.qs[2], (unsigned)b.qs[3]);
         a.qs[1][e / TOK][e % TOK] = make_uint4((unsigned)b.qs[4], (unsigned)b.qs[5], (unsigned)b.qs[6], (unsigned)b.qs[7]);
@@ -291,7 +292,10 @@ __device__ __forceinline__ void rein_mmq_skinny(const uint8_t* __restrict__ w, c
     const unsigned tok_base = blockIdx.y * TOK;
     const unsigned tok_end = min(p_rows, tok_base + TOK);
     const unsigned wsel = FMT == REIN_Q8_0 ? h : 0u;
-    const unsigned ja = j & (TOK - 1);                 // tile rows >= TOK repeat real tokens (never read back)
+    // tile row of lane half h, register v is 8(v/4) + 4h + v%4: with NV <= 4 the tokens a lane
+    // converts are NV*h + v, i.e. token t sits in tile row (t % NV) + 4(t / NV); the other
+    // rows repeat real tokens and are never read back
+    const unsigned ja = NV >= 4 ? (j & (TOK - 1)) : ((j & (NV - 1)) | (((j >> 2) & 1u) * NV));
     const unsigned rot = j >> 1;
     WaveLds& my = reinterpret_cast<WaveLds*>(rein_skinny_lds)[wave];
 
@@ -342,13 +346,21 @@ __device__ __forceinline__ void rein_mmq_skinny(const uint8_t* __restrict__ w, c
                 rein_v4i av;
                 av[0] = (int)a4.x; av[1] = (int)a4.y; av[2] = (int)a4.z; av[3] = (int)a4.w;
                 float dxv[NV], xsv[NV];
+                if constexpr (NV >= 4) {
 #pragma unroll
-                for (int q = 0; q < NV / 4; q++) {
-                    const float4 d4 = *reinterpret_cast<const float4*>(&a.dx[sb][8 * q + 4 * h]);
-                    dxv[4 * q] = d4.x; dxv[4 * q + 1] = d4.y; dxv[4 * q + 2] = d4.z; dxv[4 * q + 3] = d4.w;
-                    if constexpr (XS) {
-                        const float4 x4 = *reinterpret_cast<const float4*>(&a.xs[sb][8 * q + 4 * h]);
-                        xsv[4 * q] = x4.x; xsv[4 * q + 1] = x4.y; xsv[4 * q + 2] = x4.z; xsv[4 * q + 3] = x4.w;
+                    for (int q = 0; q < NV / 4; q++) {
+                        const float4 d4 = *reinterpret_cast<const float4*>(&a.dx[sb][8 * q + 4 * h]);
+                        dxv[4 * q] = d4.x; dxv[4 * q + 1] = d4.y; dxv[4 * q + 2] = d4.z; dxv[4 * q + 3] = d4.w;
+                        if constexpr (XS) {
+                            const float4 x4 = *reinterpret_cast<const float4*>(&a.xs[sb][8 * q + 4 * h]);
+                            xsv[4 * q] = x4.x; xsv[4 * q + 1] = x4.y; xsv[4 * q + 2] = x4.z; xsv[4 * q + 3] = x4.w;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < NV; v++) {
+                        dxv[v] = a.dx[sb][NV * h + v];
+                        if constexpr (XS) xsv[v] = a.xs[sb][NV * h + v];
                     }
                 }
                 if constexpr (SK::kTwoScales) {
@@ -406,7 +418,7 @@ __device__ __forceinline__ void rein_mmq_skinny(const uint8_t* __restrict__ w, c
 #pragma unroll 1
         for (unsigned k = 1; k < KS; k++) s += red[k * kStride + e];
         const unsigned v = e >> 6, l = e & 63u;
-        const unsigned tok = tok_base + 8u * (v >> 2) + 4u * (l >> 5) + (v & 3u);
+        const unsigned tok = tok_base + (NV >= 4 ? 8u * (v >> 2) + 4u * (l >> 5) + (v & 3u) : NV * (l >> 5) + v);
         const unsigned r = row_base + (l & 31u);
         if (tok < tok_end && r < out_dim) y[(size_t)tok * out_dim + r] = s;
     }

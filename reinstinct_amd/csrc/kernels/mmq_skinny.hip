@@ -15,3 +15,16 @@ REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q8_0_v4, REIN_Q8_0, 4, 3)
 REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q8_0_v8, REIN_Q8_0, 8, 2)
 REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq4xs_v4, REIN_IQ4_XS, 4, 3)
 REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq4xs_v8, REIN_IQ4_XS, 8, 2)
+// two and four activation rows: fewer accumulator registers are converted and scaled per sub-block
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q4_0_v1, REIN_Q4_0, 1, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q4_0_v2, REIN_Q4_0, 2, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q4k_v1, REIN_Q4_K, 1, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q4k_v2, REIN_Q4_K, 2, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q5k_v1, REIN_Q5_K, 1, 2)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q5k_v2, REIN_Q5_K, 2, 2)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q6k_v1, REIN_Q6_K, 1, 2)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q6k_v2, REIN_Q6_K, 2, 2)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q8_0_v1, REIN_Q8_0, 1, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q8_0_v2, REIN_Q8_0, 2, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq4xs_v1, REIN_IQ4_XS, 1, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq4xs_v2, REIN_IQ4_XS, 2, 3)
