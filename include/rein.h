@@ -34,6 +34,13 @@ enum {
     REIN_TYPE_Q6_K   = 14,
     REIN_TYPE_IQ4_XS = 23
 };
+/* ggml types that have no kernels of their own but load onto one of the layouts above
+ * (rein_ingest_for_matvec) */
+enum {
+    REIN_GGML_Q3_K   = 11,   /* -> Q6_K, exact */
+    REIN_GGML_IQ4_NL = 20,   /* -> IQ4_XS, exact */
+    REIN_GGML_BF16   = 30    /* -> Q8_0, one quantization step */
+};
 
 enum {
     REIN_OK            = 0,
@@ -126,6 +133,19 @@ int rein_bytes_per_block(int fmt);
  * bytes.  The reference asserts on a bad in_dim; this returns REIN_E_BAD_SHAPE. */
 int rein_repack_for_matvec(int fmt, const uint8_t *src, size_t in_dim, size_t out_dim,
                            uint8_t *dst);
+/* GpuMatvecTensor::from_bytes_matvec (src/runtime/qwen35.rs:251-331): GGUF tensor bytes of
+ * `ggml_type` -> repacked slab in `dst`, *out_fmt = the format id whose kernels read it.
+ * The six kernel formats repack as they are; IQ4_NL -> IQ4_XS and Q3_K -> Q6_K relabel
+ * without rounding (src/quant/iq4_nl.rs:52-75, q3_k.rs:85-122); BF16 -> Q8_0.  `dst` holds
+ * rein_repacked_len(rein_ingest_format(ggml_type), in_dim, out_dim) bytes, `src`
+ * rein_ingest_src_len(...).  Other types: REIN_E_BAD_FORMAT. */
+int rein_ingest_format(int ggml_type);                 /* 0 when the type has no layout here */
+size_t rein_ingest_src_len(int ggml_type, size_t in_dim, size_t out_dim);
+int rein_ingest_for_matvec(int ggml_type, const uint8_t *src, size_t in_dim, size_t out_dim,
+                           uint8_t *dst, int *out_fmt);
+/* q3_k::transcode_to_q6_k (src/quant/q3_k.rs:85-122): n_weights/256 blocks of 110 bytes ->
+ * blocks of 210 bytes that dequantize to the same values bit for bit. */
+int rein_transcode_q3_k_to_q6_k(const uint8_t *src, size_t n_weights, uint8_t *dst);
 /* fp32 -> on-disk blocks, host to host, for building synthetic weights.  Q8_0
  * follows q8_0::quantize_from_f32 (q8_0.rs:45-61); the reference has no
  * quantizer for the other five formats, these follow ggml's reference

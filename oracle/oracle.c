@@ -877,6 +877,83 @@ void orc_moe_combine(const float *experts, const int32_t *ids, const float *weig
     }
 }
 
+/* ---- relabelled GGUF types -------------------------------------------------- */
+
+/* src/quant/q3_k.rs:124-165, the walk of ggml's dequantize_row_q3_K: two halves of 128
+ * weights, four 2-bit shift levels each, two 16-weight sub-blocks per level; the third
+ * quant bit comes from hmask with one mask bit per (half, level); bit CLEAR subtracts 4 */
+static void q3k_scales(const uint8_t *sc, int out[16])
+{
+    /* src/quant/q3_k.rs:41-61: low nibbles of scales 0..7 in bytes 0..7, of 8..15 in their
+     * high nibbles, the two top bits four per byte in bytes 8..11 */
+    uint32_t a0, a1, tmp;
+    memcpy(&a0, sc, 4);
+    memcpy(&a1, sc + 4, 4);
+    memcpy(&tmp, sc + 8, 4);
+    const uint32_t k1 = 0x03030303u, k2 = 0x0f0f0f0fu;
+    uint32_t aux[4];
+    aux[0] = (a0 & k2) | (((tmp >> 0) & k1) << 4);
+    aux[1] = (a1 & k2) | (((tmp >> 2) & k1) << 4);
+    aux[2] = ((a0 >> 4) & k2) | (((tmp >> 4) & k1) << 4);
+    aux[3] = ((a1 >> 4) & k2) | (((tmp >> 6) & k1) << 4);
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++) out[4 * i + j] = (int)(int8_t)((aux[i] >> (8 * j)) & 0xFF);
+}
+
+void orc_q3_k_dequantize(const uint8_t *src, float *out, size_t n)
+{
+    for (size_t b = 0; b < n / 256; b++) {
+        const uint8_t *blk = src + b * 110;
+        const uint8_t *hmask = blk, *qs = blk + 32;
+        uint16_t dbits;
+        memcpy(&dbits, blk + 108, 2);
+        const float d_all = orc_f16_to_f32(dbits);
+        int scales[16];
+        q3k_scales(blk + 96, scales);
+        float *ob = out + b * 256;
+        size_t y = 0;
+        int is = 0;
+        unsigned m = 1;
+        for (int half = 0; half < 2; half++) {
+            const uint8_t *q = qs + 32 * half;
+            for (int shift = 0; shift < 8; shift += 2) {
+                for (int part = 0; part < 2; part++) {
+                    const float dl = d_all * (float)(scales[is++] - 32);
+                    for (int l = 0; l < 16; l++) {
+                        const int lo = (q[l + 16 * part] >> shift) & 3;
+                        const int hi = (hmask[l + 16 * part] & m) ? 0 : 4;
+                        ob[y++] = dl * (float)(lo - hi);
+                    }
+                }
+                m <<= 1;
+            }
+        }
+    }
+}
+
+/* src/quant/iq4_nl.rs:34-50: w[k] = d * kvalues[qs[k] & 15], w[k+16] = d * kvalues[qs[k] >> 4] */
+void orc_iq4_nl_dequantize(const uint8_t *src, float *out, size_t n)
+{
+    for (size_t b = 0; b < n / 32; b++) {
+        const uint8_t *blk = src + b * 18;
+        uint16_t dbits;
+        memcpy(&dbits, blk, 2);
+        const float d = orc_f16_to_f32(dbits);
+        for (int k = 0; k < 16; k++) {
+            out[b * 32 + k] = d * (float)KVALUES_IQ4NL[blk[2 + k] & 15];
+            out[b * 32 + k + 16] = d * (float)KVALUES_IQ4NL[blk[2 + k] >> 4];
+        }
+    }
+}
+
+void orc_bf16_to_f32(const uint16_t *src, float *out, size_t n)
+{
+    for (size_t i = 0; i < n; i++) {
+        const uint32_t bits = (uint32_t)src[i] << 16;
+        memcpy(&out[i], &bits, 4);
+    }
+}
+
 /* ---- fused BlockQ8 producers ---------------------------------------------- */
 
 float orc_exp_det(float x)

@@ -156,6 +156,13 @@ void orc_rmsnorm_ref(const float *x, const float *w, float eps, float *out, size
 void orc_rmsnorm_gated_ref(const float *x, const float *gate, const float *w, float eps, float *out, size_t n);
 void orc_map_ref(int which, const float *x, float *out, size_t n);
 
+/* ---- relabelled GGUF types: CPU dequantizers of the source formats -----------------
+ * src/quant/q3_k.rs:124-165 (110-byte blocks), src/quant/iq4_nl.rs:34-50 (18-byte blocks),
+ * src/quant/half.rs:42-46 (bf16 = high half of an f32) */
+void orc_q3_k_dequantize(const uint8_t *src, float *out, size_t n);
+void orc_iq4_nl_dequantize(const uint8_t *src, float *out, size_t n);
+void orc_bf16_to_f32(const uint16_t *src, float *out, size_t n);
+
 /* kernels/swiglu.cpp:10-21 (expf in place of __expf) */
 void orc_swiglu_mul(const float *gate, const float *up, float *out, size_t n);
 /* kernels/mmq_gemm_q4k_grouped.cpp:38-165 — per expert e, rows

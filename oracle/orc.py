@@ -50,6 +50,9 @@ def _load():
         "orc_moe_scatter_rows": (None, [f32p, i32p, f32p, C.c_int, C.c_int]),
         "orc_moe_combine": (None, [f32p, i32p, f32p, f32p, f32p, C.c_int, C.c_int, C.c_int]),
         "orc_swiglu_mul": (None, [f32p, f32p, f32p, sz]),
+        "orc_q3_k_dequantize": (None, [u8p, f32p, sz]),
+        "orc_iq4_nl_dequantize": (None, [u8p, f32p, sz]),
+        "orc_bf16_to_f32": (None, [u8p, f32p, sz]),
         "orc_map_det": (None, [C.c_int, f32p, f32p, sz]),
         "orc_map_ref": (None, [C.c_int, f32p, f32p, sz]),
         "orc_sumsq_det": (C.c_float, [f32p, sz]),
@@ -245,6 +248,31 @@ def swiglu_mul(gate, up):
     gate, up = _f32(gate), _f32(up)
     out = np.empty_like(gate)
     lib.orc_swiglu_mul(_p(gate), _p(up), _p(out), gate.size)
+    return out
+
+
+# ---- relabelled GGUF types
+def q3_k_dequantize(raw, n):
+    """src/quant/q3_k.rs:124-165"""
+    raw = _u8(raw)
+    out = np.empty(n, np.float32)
+    lib.orc_q3_k_dequantize(_p(raw), _p(out), n)
+    return out
+
+
+def iq4_nl_dequantize(raw, n):
+    """src/quant/iq4_nl.rs:34-50"""
+    raw = _u8(raw)
+    out = np.empty(n, np.float32)
+    lib.orc_iq4_nl_dequantize(_p(raw), _p(out), n)
+    return out
+
+
+def bf16_to_f32(bits):
+    """src/quant/half.rs:42-46"""
+    bits = np.ascontiguousarray(bits, np.uint16)
+    out = np.empty(bits.size, np.float32)
+    lib.orc_bf16_to_f32(_p(bits), _p(out), bits.size)
     return out
 
 

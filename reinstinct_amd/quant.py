@@ -51,3 +51,29 @@ def quantize_weights(fmt, w):
     out = np.empty(max(w.size // max(bs, 1) * bb, 1), np.uint8)
     check(lib.rein_quantize_weights(fmt, _ptr(w), w.size, _ptr(out)))
     return out[: w.size // bs * bb]
+
+
+GGML_Q3_K, GGML_IQ4_NL, GGML_BF16 = 11, 20, 30
+
+
+def ingest_for_matvec(ggml_type, raw, in_dim, out_dim):
+    """GpuMatvecTensor::from_bytes_matvec (src/runtime/qwen35.rs:251-331): GGUF tensor bytes ->
+    (repacked slab, format id of the kernels that read it)."""
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    label = lib.rein_ingest_format(ggml_type)
+    if label == 0:
+        check(lib.rein_ingest_for_matvec(ggml_type, _ptr(raw), in_dim, out_dim, None, None))
+    if raw.size < lib.rein_ingest_src_len(ggml_type, in_dim, out_dim):
+        raise ValueError("tensor bytes too short for the shape")
+    out = np.empty(max(repacked_len(label, in_dim, out_dim), 1), np.uint8)
+    fmt = C.c_int(0)
+    check(lib.rein_ingest_for_matvec(ggml_type, _ptr(raw), in_dim, out_dim, _ptr(out), C.byref(fmt)))
+    return out[: repacked_len(label, in_dim, out_dim)], fmt.value
+
+
+def transcode_q3_k_to_q6_k(raw, n_weights):
+    """q3_k::transcode_to_q6_k (src/quant/q3_k.rs:85-122)"""
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    out = np.empty(n_weights // 256 * 210, np.uint8)
+    check(lib.rein_transcode_q3_k_to_q6_k(_ptr(raw), n_weights, _ptr(out)))
+    return out

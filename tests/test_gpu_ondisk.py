@@ -118,3 +118,43 @@ def test_q8_0_splitk(in_dim, out_dim, n_split):
     hip.Module.builtin().function("matvec_q8_0_repacked_splitk_f32").launch(((out_dim + 1) // 2, n_split, 1), (64, 1, 1), 0, None, args)
     hip.synchronize()
     assert np.array_equal(dy2.to_host(np.uint32), dy.to_host(np.uint32))
+
+
+@pytest.mark.parametrize("ggml_type", ["q3_k", "iq4_nl", "bf16"])
+def test_ingested_types_run_on_the_relabelled_kernels(ggml_type):
+    # GGUF bytes of a type without kernels of its own -> rein_ingest_for_matvec -> decode matvec;
+    # compared with the CPU path of the SOURCE format (dequantize -> f32 matvec, the reference's
+    # rel_l2 < 1.5e-2 bar) and with the int8 oracle on the relabelled planes
+    from helpers import Lcg
+    in_dim, out_dim = 2048, 384
+    n = in_dim * out_dim
+    rng = np.random.default_rng(5)
+    if ggml_type == "q3_k":
+        raw = Lcg(0xD3A40001).bytes(n // 256 * 110).reshape(-1, 110)
+        d = (((np.arange(raw.shape[0]) % 23) - 11) * 0.004).astype(np.float32).astype(np.float16).view(np.uint16)
+        raw[:, 108], raw[:, 109] = d & 0xFF, d >> 8
+        raw = raw.reshape(-1)
+        wf = orc.q3_k_dequantize(raw, n)
+        gg = quant.GGML_Q3_K
+    elif ggml_type == "iq4_nl":
+        raw = rng.integers(0, 256, (n // 32, 18), dtype=np.uint8)
+        d = (((np.arange(raw.shape[0]) % 29) - 14) * 0.0003).astype(np.float32).astype(np.float16).view(np.uint16)
+        raw[:, 0], raw[:, 1] = d & 0xFF, d >> 8
+        raw = raw.reshape(-1)
+        wf = orc.iq4_nl_dequantize(raw, n)
+        gg = quant.GGML_IQ4_NL
+    else:
+        w = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        bits = (w.view(np.uint32) >> 16).astype(np.uint16)
+        raw = bits.view(np.uint8)
+        wf = orc.bf16_to_f32(bits)
+        gg = quant.GGML_BF16
+    slab, fmt = quant.ingest_for_matvec(gg, raw, in_dim, out_dim)
+    x = (Lcg(0x13579BDF).acts(in_dim)).reshape(1, in_dim)
+    dq = gpu_quantize(x)
+    dy = dev(np.full(out_dim, np.nan, np.float32))
+    runtime.matvec_xq8(fmt, dev(slab), dq, dy, in_dim, out_dim)
+    hip.synchronize()
+    got = dy.to_host(np.float32)
+    assert_close_f32(got, orc.matvec_q8(fmt, slab, in_dim, out_dim, dq.to_host(np.uint8), 1)[0], what=ggml_type)
+    assert rel_l2(got, orc.matvec_f32(x[0], wf.reshape(out_dim, in_dim))) < 1.5e-2
