@@ -49,7 +49,9 @@ enum {
     REIN_E_BAD_SHAPE   = -3,   /* dimension not a block multiple, zero, or out of range */
     REIN_E_BAD_POINTER = -4,   /* NULL or misaligned pointer */
     REIN_E_NO_KERNEL   = -5,   /* symbol missing from the code object */
-    REIN_E_TOO_LARGE   = -6    /* exceeds a documented fixed limit */
+    REIN_E_TOO_LARGE   = -6,   /* exceeds a documented fixed limit */
+    REIN_E_BAD_FILE    = -7,   /* GGUF container: io error, bad magic / version, truncated, bad type or shape */
+    REIN_E_NOT_FOUND   = -8    /* no tensor / metadata key of that name, or index out of range */
 };
 
 typedef void *rein_stream_t;   /* hipStream_t   */
@@ -146,6 +148,60 @@ int rein_ingest_for_matvec(int ggml_type, const uint8_t *src, size_t in_dim, siz
 /* q3_k::transcode_to_q6_k (src/quant/q3_k.rs:85-122): n_weights/256 blocks of 110 bytes ->
  * blocks of 210 bytes that dequantize to the same values bit for bit. */
 int rein_transcode_q3_k_to_q6_k(const uint8_t *src, size_t n_weights, uint8_t *dst);
+/* ------------------------------------------------------- src/gguf mirror */
+/* GGUF v3 container (src/gguf/mod.rs:97-217).  The handle owns a read-only mapping of
+ * the file (or borrows the caller's bytes); every pointer handed out points into it and
+ * dies with rein_gguf_close.  Parse errors are REIN_E_BAD_FILE with the reference's
+ * error text (src/gguf/error.rs:4-47) in rein_last_error(). */
+typedef struct rein_gguf rein_gguf;
+typedef struct rein_gguf_tensor {        /* TensorInfo (src/gguf/tensor_info.rs:7-17) + its payload */
+    const char    *name;                 /* NUL-terminated, owned by the handle */
+    int            ggml_type;            /* types.rs:37-59 */
+    unsigned       n_dims;               /* 1..4 */
+    uint64_t       dims[4];              /* fastest first; unused trailing dims are 1 */
+    uint64_t       offset;               /* from the start of the data section */
+    uint64_t       byte_size;            /* TensorInfo::byte_size (tensor_info.rs:34-46) */
+    const uint8_t *data;                 /* GgufFile::tensor_data (mod.rs:196-201) */
+} rein_gguf_tensor;
+typedef struct rein_gguf_dims {
+    unsigned in_dim, out_dim, n_expert;  /* dims[0], dims[1], dims[2] (1 for a 2-D tensor) */
+    size_t   bytes_per_expert;           /* repacked bytes of one [in_dim, out_dim] slab */
+} rein_gguf_dims;
+/* GgufFile::open (mod.rs:97-102) / from_mmap (mod.rs:104-177) */
+int rein_gguf_open(const char *path, rein_gguf **out);
+int rein_gguf_from_bytes(const uint8_t *bytes, size_t len, rein_gguf **out);   /* caller keeps bytes alive */
+void rein_gguf_close(rein_gguf *g);
+/* Header, alignment, data_section_offset (mod.rs:45-49,64-68); any out pointer may be NULL */
+int rein_gguf_header(const rein_gguf *g, uint32_t *version, uint64_t *tensor_count,
+                     uint64_t *metadata_kv_count, uint64_t *alignment, uint64_t *data_section_offset);
+/* align_up (mod.rs:208-210): align <= 1 leaves v as it is */
+uint64_t rein_gguf_align_up(uint64_t v, uint64_t align);
+/* GgufFile::tensors[i] / tensor(name) (mod.rs:186-188); REIN_E_NOT_FOUND when absent */
+int rein_gguf_tensor_at(const rein_gguf *g, uint64_t index, rein_gguf_tensor *out);
+int rein_gguf_tensor_by_name(const rein_gguf *g, const char *name, rein_gguf_tensor *out);
+/* GgufFile::metadata[i] / metadata_get(key) (mod.rs:181-183) with MetaValue's coercions
+ * (src/gguf/value.rs:50-101): u64 from any non-negative integer variant, f32 from F32 / F64.
+ * value_type is gguf_metadata_value_type (types.rs:108-113).  A wrong variant is
+ * REIN_E_BAD_FORMAT, an absent key REIN_E_NOT_FOUND.  Strings are not NUL-terminated.
+ * rein_gguf_meta_raw points at the value's little-endian bytes in the mapping, whatever
+ * its type.  For an array `first` points at its packed payload: count fixed-width little-endian
+ * elements, or (u64 length, bytes) strings back to back. */
+int rein_gguf_meta_at(const rein_gguf *g, uint64_t index, const char **key, int *value_type);
+int rein_gguf_meta_type(const rein_gguf *g, const char *key, int *value_type);
+int rein_gguf_meta_raw(const rein_gguf *g, const char *key, int *value_type, const uint8_t **value);
+int rein_gguf_meta_u64(const rein_gguf *g, const char *key, uint64_t *out);
+int rein_gguf_meta_f32(const rein_gguf *g, const char *key, float *out);
+int rein_gguf_meta_bool(const rein_gguf *g, const char *key, int *out);
+int rein_gguf_meta_str(const rein_gguf *g, const char *key, const char **s, size_t *len);
+int rein_gguf_meta_array(const rein_gguf *g, const char *key, int *elem_type, uint64_t *count,
+                         const uint8_t **first);
+/* GpuMatvecTensor::from_gguf_matvec (src/runtime/qwen35.rs:235-245) for a 2-D tensor and
+ * GpuExpertTensor::from_gguf (qwen35.rs:397-431) for a 3-D one: repack tensor `name` into
+ * `dst` through rein_ingest_for_matvec, expert slabs back to back.  With dst == NULL only
+ * *out_fmt and *dims are filled (dims->bytes_per_expert * dims->n_expert bytes are needed). */
+int rein_gguf_load_for_matvec(const rein_gguf *g, const char *name, uint8_t *dst, size_t dst_len,
+                              int *out_fmt, rein_gguf_dims *dims);
+
 /* fp32 -> on-disk blocks, host to host, for building synthetic weights.  Q8_0
  * follows q8_0::quantize_from_f32 (q8_0.rs:45-61); the reference has no
  * quantizer for the other five formats, these follow ggml's reference

@@ -18,7 +18,17 @@ class MoeShape(C.Structure):
                 ("expert_ff", C.c_uint), ("gate_up_fmt", C.c_int), ("down_fmt", C.c_int)]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_int), ("n_dims", C.c_uint), ("dims", C.c_uint64 * 4),
+                ("offset", C.c_uint64), ("byte_size", C.c_uint64), ("data", C.c_void_p)]
+
+
+class GgufDims(C.Structure):
+    _fields_ = [("in_dim", C.c_uint), ("out_dim", C.c_uint), ("n_expert", C.c_uint), ("bytes_per_expert", C.c_size_t)]
+
+
 _vp, _u, _i, _sz = C.c_void_p, C.c_uint, C.c_int, C.c_size_t
+_u64 = C.c_uint64
 _P = C.POINTER
 
 # name -> (restype, argtypes); every symbol declared in include/rein.h
@@ -85,6 +95,22 @@ SIGNATURES = {
     "rein_ingest_src_len": (_sz, [_i, _sz, _sz]),
     "rein_ingest_for_matvec": (_i, [_i, _vp, _sz, _sz, _vp, _P(_i)]),
     "rein_transcode_q3_k_to_q6_k": (_i, [_vp, _sz, _vp]),
+    "rein_gguf_open": (_i, [C.c_char_p, _P(_vp)]),
+    "rein_gguf_from_bytes": (_i, [_vp, _sz, _P(_vp)]),
+    "rein_gguf_close": (None, [_vp]),
+    "rein_gguf_header": (_i, [_vp, _P(C.c_uint32), _P(_u64), _P(_u64), _P(_u64), _P(_u64)]),
+    "rein_gguf_align_up": (_u64, [_u64, _u64]),
+    "rein_gguf_tensor_at": (_i, [_vp, _u64, _P(GgufTensor)]),
+    "rein_gguf_tensor_by_name": (_i, [_vp, C.c_char_p, _P(GgufTensor)]),
+    "rein_gguf_meta_at": (_i, [_vp, _u64, _P(C.c_char_p), _P(_i)]),
+    "rein_gguf_meta_type": (_i, [_vp, C.c_char_p, _P(_i)]),
+    "rein_gguf_meta_raw": (_i, [_vp, C.c_char_p, _P(_i), _P(_vp)]),
+    "rein_gguf_meta_u64": (_i, [_vp, C.c_char_p, _P(_u64)]),
+    "rein_gguf_meta_f32": (_i, [_vp, C.c_char_p, _P(C.c_float)]),
+    "rein_gguf_meta_bool": (_i, [_vp, C.c_char_p, _P(_i)]),
+    "rein_gguf_meta_str": (_i, [_vp, C.c_char_p, _P(_vp), _P(_sz)]),
+    "rein_gguf_meta_array": (_i, [_vp, C.c_char_p, _P(_i), _P(_u64), _P(_vp)]),
+    "rein_gguf_load_for_matvec": (_i, [_vp, C.c_char_p, _vp, _sz, _P(_i), _P(GgufDims)]),
     "rein_matvec_ondisk_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _vp]),
     "rein_matvec_q8_0_splitk": (_i, [_vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_moe_expert_matvec": (_i, [_i, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),

@@ -92,3 +92,56 @@ def assert_close_f32(got, want, rel=1e-3, abs_=1e-4, what=""):
         raise AssertionError(
             f"{what}: {int(bad.sum())}/{bad.size} outside {rel} rel / {abs_}*{scale:.3g} abs; worst at flat {i}: "
             f"got {got.ravel()[i]!r} want {want.ravel()[i]!r}")
+
+
+# ---- a GGUF v3 writer for the container tests (layout: src/gguf/mod.rs:4-18 of the reference)
+GGUF_U8, GGUF_I8, GGUF_U16, GGUF_I16, GGUF_U32, GGUF_I32, GGUF_F32, GGUF_BOOL, GGUF_STRING, GGUF_ARRAY, \
+    GGUF_U64, GGUF_I64, GGUF_F64 = range(13)
+_GGUF_PACK = {GGUF_U8: "<B", GGUF_I8: "<b", GGUF_U16: "<H", GGUF_I16: "<h", GGUF_U32: "<I", GGUF_I32: "<i",
+              GGUF_F32: "<f", GGUF_BOOL: "<B", GGUF_U64: "<Q", GGUF_I64: "<q", GGUF_F64: "<d"}
+
+
+def gguf_string(s):
+    import struct
+    b = s if isinstance(s, bytes) else s.encode()
+    return struct.pack("<Q", len(b)) + b
+
+
+def gguf_value(vt, v):
+    """payload of one metadata value; arrays are (element type, [values])"""
+    import struct
+    if vt == GGUF_STRING:
+        return gguf_string(v)
+    if vt == GGUF_ARRAY:
+        et, items = v
+        return struct.pack("<IQ", et, len(items)) + b"".join(gguf_value(et, x) for x in items)
+    return struct.pack(_GGUF_PACK[vt], v)
+
+
+def write_gguf(meta, tensors, version=3, magic=b"GGUF", pad_data=0):
+    """meta: [(key, value type, value)]; tensors: [(name, dims, ggml type, payload bytes)].
+    Returns (file bytes, {name: offset in the data section}).  The alignment is what a
+    `general.alignment` entry of `meta` says, else 32."""
+    import struct
+    align = 32
+    for k, vt, v in meta:
+        if k == "general.alignment" and vt != GGUF_STRING:
+            align = int(v)
+    out = bytearray(magic + struct.pack("<IQQ", version, len(tensors), len(meta)))
+    for k, vt, v in meta:
+        out += gguf_string(k) + struct.pack("<I", vt) + gguf_value(vt, v)
+    offs, at = {}, 0
+    for name, dims, ty, payload in tensors:
+        offs[name] = at
+        out += gguf_string(name) + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
+        out += struct.pack("<IQ", ty, at)
+        at += len(payload)
+        if align > 1:
+            at = (at + align - 1) // align * align
+    if align > 1:
+        out += b"\0" * (-len(out) % align)
+    data_at = len(out)
+    for name, dims, ty, payload in tensors:
+        out += b"\0" * (data_at + offs[name] - len(out)) + bytes(payload)
+    out += b"\0" * pad_data
+    return bytes(out), offs
