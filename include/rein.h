@@ -32,7 +32,12 @@ enum {
     REIN_TYPE_Q4_K   = 12,
     REIN_TYPE_Q5_K   = 13,
     REIN_TYPE_Q6_K   = 14,
-    REIN_TYPE_IQ4_XS = 23
+    REIN_TYPE_IQ4_XS = 23,
+    /* relabelled: own repack, the kernels of another format compiled with another scale
+     * source / codebook (src/quant/q5_1.rs:12-20, src/quant/iq3_s.rs:13-19).  Q5_1 has MoE
+     * expert kernels only, IQ3_S dense kernels only, as in the reference. */
+    REIN_TYPE_Q5_1   = 7,
+    REIN_TYPE_IQ3_S  = 21
 };
 /* ggml types that have no kernels of their own but load onto one of the layouts above
  * (rein_ingest_for_matvec) */
@@ -138,10 +143,13 @@ int rein_repack_for_matvec(int fmt, const uint8_t *src, size_t in_dim, size_t ou
 /* GpuMatvecTensor::from_bytes_matvec (src/runtime/qwen35.rs:251-331): GGUF tensor bytes of
  * `ggml_type` -> repacked slab in `dst`, *out_fmt = the format id whose kernels read it.
  * The six kernel formats repack as they are; IQ4_NL -> IQ4_XS and Q3_K -> Q6_K relabel
- * without rounding (src/quant/iq4_nl.rs:52-75, q3_k.rs:85-122); BF16 -> Q8_0.  `dst` holds
+ * without rounding (src/quant/iq4_nl.rs:52-75, q3_k.rs:85-122); IQ3_S keeps its id on the
+ * IQ4_XS planes (src/quant/iq3_s.rs:186-207); BF16 -> Q8_0.  `dst` holds
  * rein_repacked_len(rein_ingest_format(ggml_type), in_dim, out_dim) bytes, `src`
  * rein_ingest_src_len(...).  Other types: REIN_E_BAD_FORMAT. */
 int rein_ingest_format(int ggml_type);                 /* 0 when the type has no layout here */
+/* the types GpuExpertTensor::from_gguf accepts (qwen35.rs:415-425): Q4_K, Q5_K, Q6_K, Q8_0, Q5_1 */
+int rein_ingest_expert_format(int ggml_type);
 size_t rein_ingest_src_len(int ggml_type, size_t in_dim, size_t out_dim);
 int rein_ingest_for_matvec(int ggml_type, const uint8_t *src, size_t in_dim, size_t out_dim,
                            uint8_t *dst, int *out_fmt);

@@ -80,10 +80,48 @@ static inline uint32_t rd32(const uint8_t *p)
 static const int8_t KVALUES_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10,
                                          1,    13,   25,  38,  53,  69,  89,  113};
 
+/* The IQ3_S grid (IQ3S_GRID of src/quant/iq3_s.rs:41-107, ggml's iq3s_grid): 512 groups
+ * of four magnitudes.  Every magnitude is odd, 2*l + 1 with l in 0..7, so a group is four
+ * octal digits; they are written here weight 0 first. */
+static const char IQ3S_GRID_OCTAL[2048 + 1] =
+    "000010002000500070000100110021004100610002001200520033000400240054007400150035000600260017004700"
+    "770000101010201040100110111051100210321072101310531044101610561027100020102050207020012031206120"
+    "122052200320432024205420742015203520072037203030113051300230223013303330633044300530253076301730"
+    "573000403140714012404240234004403440154007402050405002502250625033501450545074506650375060601160"
+    "316013602560176000702070407002702270627033700570457000011001200140010101110131015101710102012201"
+    "130143016301450165011601270100111011301160110111411112110311331114110511251107116711002121215121"
+    "712102214221232104213421552106212721103140317031013131311231723103314331143126310731304150412141"
+    "414113413341244164410541454110510151315112510351235115510261426172614461646110713071017121711271"
+    "537114712671077100021002300250027002010221024102610212023202720203022302140234025402050225027602"
+    "070237025702001220120112311271122212521213124312241215121022402270221222322203227322142235227522"
+    "172247220032203250321132223242321332333224320532663210427042024232422342534214422742574240521152"
+    "225273520452355207520062206270621262556216625072117262720372347205722003110331035103710322031303"
+    "330353032403440374031503360317031013301350134113121332130413061327136713002321230223232343230523"
+    "103301334133123332337233033314333433743355333733304311436143224313432543064346431053015321535253"
+    "235344536553375361631463107330730273227353730004400421040204420472042304140405040704201470141114"
+    "311422140314531434141514551410243024012451241224332404247524262407244034113431340234223413345334"
+    "004420444244734404441744505470541254265431644364066401745174037434741574200501054105220504054405"
+    "740525056605470510153015501521151215231527150025112532250325632535252035703501357235443515355635"
+    "373510454045024523456445215562551555355524652075407522751106310651061306330606060016021672164616"
+    "212643262426552626260726003641361236043652463446264600563056435606565066046611763176000740077007"
+    "020722076307040745072607201711174217341754171027402701276127122703271527203723375337353710475047"
+    "31470247054722572457206713670077";
+
+/* magnitude of weight j (0..3) of grid entry idx (0..511) */
+static inline int iq3s_grid_mag(int idx, int j) { return 2 * (IQ3S_GRID_OCTAL[4 * idx + j] - '0') + 1; }
+
+uint32_t orc_iq3s_grid_entry(int idx)
+{
+    uint32_t v = 0;
+    for (int j = 0; j < 4; j++) v |= (uint32_t)iq3s_grid_mag(idx, j) << (8 * j);
+    return v;
+}
+
 int orc_block_size(int fmt)
 {
     switch (fmt) {
-    case ORC_Q4_0: case ORC_Q8_0: return 32;                      /* q4_0.rs:22, q8_0.rs:8 */
+    case ORC_Q4_0: case ORC_Q8_0: case ORC_Q5_1: return 32;       /* q4_0.rs:22, q8_0.rs:8, q5_1.rs:25 */
+    case ORC_IQ3_S:                                               /* iq3_s.rs:24 */
     case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_IQ4_XS: return 256;
     default: return 0;
     }
@@ -98,6 +136,8 @@ int orc_bytes_per_block(int fmt)
     case ORC_Q5_K:   return 176;   /* q5_k.rs:22  */
     case ORC_Q6_K:   return 210;   /* q6_k.rs:19  */
     case ORC_IQ4_XS: return 136;   /* iq4_xs.rs:24 */
+    case ORC_Q5_1:   return 24;    /* q5_1.rs:26  */
+    case ORC_IQ3_S:  return 110;   /* iq3_s.rs:25 */
     default: return 0;
     }
 }
@@ -228,6 +268,50 @@ static void dequant_iq4_xs(const uint8_t *b, float *y)
     }
 }
 
+/* src/quant/q5_1.rs:38-56: w = d*q5 + m, the 5th bit of weight i is bit i of qh */
+static void dequant_q5_1(const uint8_t *b, float *y)
+{
+    float d = orc_f16_to_f32(rd16(b)), m = orc_f16_to_f32(rd16(b + 2));
+    uint32_t qh = rd32(b + 4);
+    const uint8_t *qs = b + 8;
+    for (int k = 0; k < 16; k++) {
+        int lo = (qs[k] & 0x0F) | (int)(((qh >> k) & 1u) << 4);
+        int hi = (qs[k] >> 4) | (int)(((qh >> (k + 16)) & 1u) << 4);
+        y[k] = d * (float)lo + m;
+        y[k + 16] = d * (float)hi + m;
+    }
+}
+
+/* The eight sub-blocks of an IQ3_S block as (db, 32 signed odd values), src/quant/iq3_s.rs:
+ * 113-147: sub-block s reads 8 index bytes qs[8s..], one qh byte (bit i = 9th bit of index
+ * i), 4 sign bytes (bit j of byte l flips weight 8l + j) and the nibble s of scales;
+ * db = d * (1 + 2*nibble). */
+static void iq3s_sub_block(const uint8_t *b, int s, float *db, int vals[32])
+{
+    const uint8_t *qs = b + 2 + 8 * s, *signs = b + 2 + 64 + 8 + 4 * s;
+    int qh = b[2 + 64 + s];
+    int sc = (b[2 + 64 + 8 + 32 + s / 2] >> (4 * (s & 1))) & 0x0F;
+    *db = orc_f16_to_f32(rd16(b)) * (1.0f + 2.0f * (float)sc);
+    for (int i = 0; i < 8; i++) {                /* index i covers weights 4i .. 4i+3 */
+        int idx = qs[i] | (((qh >> i) & 1) << 8);
+        for (int j = 0; j < 4; j++) {
+            int w = 4 * i + j;
+            int mag = iq3s_grid_mag(idx, j);
+            vals[w] = (signs[w >> 3] >> (w & 7)) & 1 ? -mag : mag;
+        }
+    }
+}
+
+static void dequant_iq3_s(const uint8_t *b, float *y)
+{
+    for (int s = 0; s < 8; s++) {
+        float db;
+        int v[32];
+        iq3s_sub_block(b, s, &db, v);
+        for (int i = 0; i < 32; i++) y[32 * s + i] = db * (float)v[i];
+    }
+}
+
 int orc_dequantize_to_f32(int fmt, const uint8_t *bytes, float *out, size_t n)
 {
     int bs = orc_block_size(fmt), bb = orc_bytes_per_block(fmt);
@@ -243,6 +327,8 @@ int orc_dequantize_to_f32(int fmt, const uint8_t *bytes, float *out, size_t n)
         case ORC_Q8_0:   dequant_q8_0(b, y); break;
         case ORC_Q4_0:   dequant_q4_0(b, y); break;
         case ORC_IQ4_XS: dequant_iq4_xs(b, y); break;
+        case ORC_Q5_1:   dequant_q5_1(b, y); break;
+        case ORC_IQ3_S:  dequant_iq3_s(b, y); break;
         }
     }
     return 0;
@@ -268,6 +354,8 @@ static void plane_bytes(int fmt, size_t *per_sub, size_t *per_super)
     case ORC_Q8_0:   *per_sub = 32 + 2;     *per_super = 0; break;  /* q8_0.rs:74-77   */
     case ORC_Q4_0:   *per_sub = 16 + 2;     *per_super = 0; break;  /* q4_0.rs:66-69   */
     case ORC_IQ4_XS: *per_sub = 16 + 2;     *per_super = 0; break;  /* iq4_xs.rs:85-88 */
+    case ORC_IQ3_S:  *per_sub = 16 + 2;     *per_super = 0; break;  /* iq3_s.rs:178-184 */
+    case ORC_Q5_1:   *per_sub = 16 + 4 + 4; *per_super = 0; break;  /* q5_1.rs:76-81   */
     default:         *per_sub = 0;          *per_super = 0; break;
     }
 }
@@ -432,6 +520,46 @@ static void repack_iq4_xs(const uint8_t *bytes, size_t in_dim, size_t out_dim, u
         }
 }
 
+/* src/quant/q5_1.rs:61-104: nibbles verbatim; qh re-ordered so that bit 8j+b is the 5th
+ * bit of weight 4j+b and bit 8j+4+b that of weight 16+4j+b; raw fp16 d | m << 16 */
+static void repack_q5_1(const uint8_t *bytes, size_t in_dim, size_t out_dim, uint8_t *out)
+{
+    size_t n_sub = in_dim / 32, nsp = orc_repacked_n_sub_padded(in_dim);
+    size_t nib_len = out_dim * nsp * 16, qh_len = out_dim * nsp * 4;
+    for (size_t row = 0; row < out_dim; row++)
+        for (size_t sb = 0; sb < n_sub; sb++) {
+            const uint8_t *b = bytes + (row * n_sub + sb) * 24;
+            size_t i = row * nsp + sb;
+            memcpy(out + i * 16, b + 8, 16);
+            uint32_t qh = rd32(b + 4), packed = 0;
+            for (int w = 0; w < 32; w++) {
+                int j = (w & 15) >> 2, bb = w & 3, upper = w >> 4;
+                packed |= ((qh >> w) & 1u) << (8 * j + 4 * upper + bb);
+            }
+            uint8_t *q = out + nib_len + i * 4;
+            q[0] = (uint8_t)packed; q[1] = (uint8_t)(packed >> 8); q[2] = (uint8_t)(packed >> 16); q[3] = (uint8_t)(packed >> 24);
+            memcpy(out + nib_len + qh_len + i * 4, b, 4);
+        }
+}
+
+/* src/quant/iq3_s.rs:186-207: nibble (v + 15) / 2 of weight k low / k+16 high, fp16(db) */
+static void repack_iq3_s(const uint8_t *bytes, size_t in_dim, size_t out_dim, uint8_t *out)
+{
+    size_t nb = in_dim / 256, nsp = orc_repacked_n_sub_padded(in_dim);
+    size_t nib_len = out_dim * nsp * 16;
+    for (size_t row = 0; row < out_dim; row++)
+        for (size_t blk = 0; blk < nb; blk++)
+            for (int s = 0; s < 8; s++) {
+                float db;
+                int v[32];
+                iq3s_sub_block(bytes + (row * nb + blk) * 110, s, &db, v);
+                size_t i = row * nsp + blk * 8 + (size_t)s;
+                for (int k = 0; k < 16; k++)
+                    out[i * 16 + (size_t)k] = (uint8_t)(((v[k] + 15) / 2) | (((v[k + 16] + 15) / 2) << 4));
+                wr16(out + nib_len + i * 2, orc_f32_to_f16(db));
+            }
+}
+
 int orc_repack_for_matvec(int fmt, const uint8_t *bytes, size_t in_dim, size_t out_dim,
                           uint8_t *out)
 {
@@ -445,6 +573,8 @@ int orc_repack_for_matvec(int fmt, const uint8_t *bytes, size_t in_dim, size_t o
     case ORC_Q8_0:   repack_q8_0(bytes, in_dim, out_dim, out); break;
     case ORC_Q4_0:   repack_q4_0(bytes, in_dim, out_dim, out); break;
     case ORC_IQ4_XS: repack_iq4_xs(bytes, in_dim, out_dim, out); break;
+    case ORC_Q5_1:   repack_q5_1(bytes, in_dim, out_dim, out); break;
+    case ORC_IQ3_S:  repack_iq3_s(bytes, in_dim, out_dim, out); break;
     }
     return 0;
 }
@@ -477,7 +607,9 @@ static planes_t planes_of(int fmt, const uint8_t *w, size_t in_dim, size_t out_d
     case ORC_Q5_K:   p.aux = w + n * 16; p.sm = p.aux + n * 4; p.sup = p.sm + n * 2; break;
     case ORC_Q6_K:   p.aux = w + n * 16; p.sm = p.aux + n * 8; p.sup = p.sm + n * 2; break;
     case ORC_Q8_0:   p.aux = w + n * 16; p.sm = w + n * 32; break;
+    case ORC_Q5_1:   p.aux = w + n * 16; p.sm = p.aux + n * 4; break;      /* sm: 4 B / sub-block here */
     case ORC_Q4_0:
+    case ORC_IQ3_S:
     case ORC_IQ4_XS: p.sm = w + n * 16; break;
     }
     return p;
@@ -497,7 +629,7 @@ static void sub_block_ints(int fmt, const planes_t *p, size_t row, size_t sb, in
         return;
     }
     for (int k = 0; k < 16; k++) { wq[k] = nb[k] & 0x0F; wq[16 + k] = nb[k] >> 4; }
-    if (fmt == ORC_Q5_K) {
+    if (fmt == ORC_Q5_K || fmt == ORC_Q5_1) {
         /* bit 4g+b of qh = 5th bit of weight b of dot group g; group 2j = weights
          * 4j.., group 2j+1 = weights 16+4j.. (matvec_q5k_repacked.cpp:90-91) */
         uint32_t qh = rd32(p->aux + idx * 4);
@@ -517,6 +649,8 @@ static void sub_block_ints(int fmt, const planes_t *p, size_t row, size_t sb, in
             }
     } else if (fmt == ORC_IQ4_XS) {
         for (int k = 0; k < 32; k++) wq[k] = KVALUES_IQ4NL[wq[k]];
+    } else if (fmt == ORC_IQ3_S) {
+        for (int k = 0; k < 32; k++) wq[k] = 2 * wq[k] - 15;      /* KVALUES_IQ3S, iq3_s.rs:161-162 */
     }
 }
 
@@ -548,6 +682,9 @@ int orc_decode_repacked_to_f32(int fmt, const uint8_t *packed, size_t in_dim, si
                 const uint8_t *dd = p.sup + (row * p.n_super + sb / 8) * 4;
                 float dsc  = orc_f16_to_f32(rd16(dd)) * (float)p.sm[idx * 2];
                 float deff = orc_f16_to_f32(rd16(dd + 2)) * (float)p.sm[idx * 2 + 1];
+                for (int k = 0; k < 32; k++) o[orig_pos(fmt, sb, k)] = dsc * (float)wq[k] - deff;
+            } else if (fmt == ORC_Q5_1) {
+                float dsc = orc_f16_to_f32(rd16(p.sm + idx * 4)), deff = -orc_f16_to_f32(rd16(p.sm + idx * 4 + 2));
                 for (int k = 0; k < 32; k++) o[orig_pos(fmt, sb, k)] = dsc * (float)wq[k] - deff;
             } else if (fmt == ORC_Q6_K) {
                 float d = orc_f16_to_f32(rd16(p.sup + (row * p.n_super + sb / 8) * 2));
@@ -685,6 +822,10 @@ static float block_term(int fmt, const planes_t *p, size_t row, size_t sb, const
         const uint8_t *dd = p->sup + (row * p->n_super + sb / 8) * 4;
         float dsc  = orc_f16_to_f32(rd16(dd)) * (float)p->sm[idx * 2];
         float deff = orc_f16_to_f32(rd16(dd + 2)) * (float)p->sm[idx * 2 + 1];
+        return dsc * dx * (float)parts[0] - deff * xsum;
+    }
+    if (fmt == ORC_Q5_1) {                           /* moe_matvec_q5k_repacked.cpp:86-91: dsc = d, deff = -m */
+        float dsc = orc_f16_to_f32(rd16(p->sm + idx * 4)), deff = -orc_f16_to_f32(rd16(p->sm + idx * 4 + 2));
         return dsc * dx * (float)parts[0] - deff * xsum;
     }
     if (fmt == ORC_Q6_K) {

@@ -54,7 +54,9 @@ enum {
     ORC_Q4_K   = 12,
     ORC_Q5_K   = 13,
     ORC_Q6_K   = 14,
-    ORC_IQ4_XS = 23
+    ORC_IQ4_XS = 23,
+    ORC_Q5_1   = 7,    /* runs on the Q5_K kernels with raw (d, m) scales, src/quant/q5_1.rs:12-20 */
+    ORC_IQ3_S  = 21    /* runs on the IQ4_XS kernels with the codebook 2n-15, src/quant/iq3_s.rs:13-19 */
 };
 
 /* src/quant/half.rs:9-40, 51-84 */
@@ -161,6 +163,9 @@ void orc_map_ref(int which, const float *x, float *out, size_t n);
  * src/quant/half.rs:42-46 (bf16 = high half of an f32) */
 void orc_q3_k_dequantize(const uint8_t *src, float *out, size_t n);
 void orc_iq4_nl_dequantize(const uint8_t *src, float *out, size_t n);
+/* entry idx (0..511) of the IQ3_S grid as the reference states it: four magnitude bytes,
+ * weight 0 in the low byte (IQ3S_GRID, src/quant/iq3_s.rs:41-107) */
+uint32_t orc_iq3s_grid_entry(int idx);
 void orc_bf16_to_f32(const uint16_t *src, float *out, size_t n);
 
 /* kernels/swiglu.cpp:10-21 (expf in place of __expf) */

@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboracle.so")
 
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 2, 8, 12, 13, 14, 23
+Q5_1, IQ3_S = 7, 21          # relabelled onto the Q5_K / IQ4_XS kernels (src/quant/q5_1.rs, iq3_s.rs)
 FORMATS = {"q4_0": Q4_0, "q8_0": Q8_0, "q4_k": Q4_K, "q5_k": Q5_K, "q6_k": Q6_K, "iq4_xs": IQ4_XS}
 
 
@@ -52,6 +53,7 @@ def _load():
         "orc_swiglu_mul": (None, [f32p, f32p, f32p, sz]),
         "orc_q3_k_dequantize": (None, [u8p, f32p, sz]),
         "orc_iq4_nl_dequantize": (None, [u8p, f32p, sz]),
+        "orc_iq3s_grid_entry": (C.c_uint32, [C.c_int]),
         "orc_bf16_to_f32": (None, [u8p, f32p, sz]),
         "orc_map_det": (None, [C.c_int, f32p, f32p, sz]),
         "orc_map_ref": (None, [C.c_int, f32p, f32p, sz]),
@@ -266,6 +268,10 @@ def iq4_nl_dequantize(raw, n):
     out = np.empty(n, np.float32)
     lib.orc_iq4_nl_dequantize(_p(raw), _p(out), n)
     return out
+
+
+def iq3s_grid_entry(idx):
+    return int(lib.orc_iq3s_grid_entry(idx))
 
 
 def bf16_to_f32(bits):

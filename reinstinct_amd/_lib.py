@@ -92,6 +92,7 @@ SIGNATURES = {
     "rein_moe_grouped_gemm": (_i, [_i, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
     "rein_swiglu_mul": (_i, [_vp, _vp, _vp, _u, _vp]),
     "rein_ingest_format": (_i, [_i]),
+    "rein_ingest_expert_format": (_i, [_i]),
     "rein_ingest_src_len": (_sz, [_i, _sz, _sz]),
     "rein_ingest_for_matvec": (_i, [_i, _vp, _sz, _sz, _vp, _P(_i)]),
     "rein_transcode_q3_k_to_q6_k": (_i, [_vp, _sz, _vp]),

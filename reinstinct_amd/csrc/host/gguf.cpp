@@ -485,8 +485,12 @@ int rein_gguf_load_for_matvec(const rein_gguf* g, const char* name, uint8_t* dst
     if (int rc = rein_gguf_tensor_by_name(g, name, &t)) return rc;
     if (t.n_dims != 2 && t.n_dims != 3)
         return fail(REIN_E_BAD_SHAPE, std::string("tensor ") + name + ": expected 2D or 3D, got " + std::to_string(t.n_dims) + "D");
-    const int label = rein_ingest_format(t.ggml_type);
-    if (!label) return fail(REIN_E_BAD_FORMAT, std::string("tensor ") + name + ": no kernels for ggml type " + std::to_string(t.ggml_type));
+    // a 3-D tensor is a stack of experts and takes the expert formats, a 2-D one the dense formats
+    const int label = t.n_dims == 3 ? rein_ingest_expert_format(t.ggml_type) : rein_ingest_format(t.ggml_type);
+    if (!label)
+        return fail(REIN_E_BAD_FORMAT, std::string("tensor ") + name + ": no " + (t.n_dims == 3 ? "MoE " : "") +
+                                           "kernels for ggml type " + std::to_string(t.ggml_type) +
+                                           (t.n_dims == 3 ? " (experts must be Q4_K, Q5_K, Q6_K, Q8_0 or Q5_1)" : ""));
     if (t.dims[0] > 0xFFFFFFFFull || t.dims[1] > 0xFFFFFFFFull || t.dims[2] > 0xFFFFFFFFull)
         return fail(REIN_E_BAD_SHAPE, std::string("tensor ") + name + ": dimension above 32 bits");
     const size_t in_dim = (size_t)t.dims[0], out_dim = (size_t)t.dims[1], n_expert = (size_t)t.dims[2];
@@ -508,8 +512,11 @@ int rein_gguf_load_for_matvec(const rein_gguf* g, const char* name, uint8_t* dst
     if (dst_len < per * n_expert)
         return fail(REIN_E_BAD_SHAPE, std::string("tensor ") + name + ": destination holds " + std::to_string(dst_len) + " bytes, " +
                                           std::to_string(per * n_expert) + " needed");
-    for (size_t e = 0; e < n_expert; e++)
-        if (int rc = rein_ingest_for_matvec(t.ggml_type, t.data + e * src_per, in_dim, out_dim, dst + e * per, nullptr)) return rc;
+    for (size_t e = 0; e < n_expert; e++) {
+        const int rc = t.n_dims == 3 ? rein_repack_for_matvec(label, t.data + e * src_per, in_dim, out_dim, dst + e * per)
+                                     : rein_ingest_for_matvec(t.ggml_type, t.data + e * src_per, in_dim, out_dim, dst + e * per, nullptr);
+        if (rc) return rc;
+    }
     return REIN_OK;
 }
 

@@ -11,8 +11,9 @@
 //            factor (src/quant/q3_k.rs:85-122), then the Q6_K repack.
 //   BF16   -> f32 (high half of the word) -> Q8_0 blocks (src/quant/q8_0.rs:45-61) -> Q8_0 repack.
 //
-// Q5_1 and IQ3_S (which the reference runs on re-compiled Q5_K / IQ4_XS kernels) are
-// not handled: REIN_E_BAD_FORMAT.
+// IQ3_S repacks onto the IQ4_XS planes under its own format id (the kernels differ in the
+// codebook).  Q5_1 is an expert-tensor format only (rein_ingest_expert_format), as in the
+// reference, where a dense Q5_1 tensor stays in its on-disk layout.
 #include <cstring>
 #include <string>
 #include <vector>
@@ -69,7 +70,7 @@ int label_of(int ggml_type)
 {
     switch (ggml_type) {
     case REIN_TYPE_Q4_0: case REIN_TYPE_Q8_0: case REIN_TYPE_Q4_K: case REIN_TYPE_Q5_K: case REIN_TYPE_Q6_K:
-    case REIN_TYPE_IQ4_XS: return ggml_type;
+    case REIN_TYPE_IQ4_XS: case REIN_TYPE_IQ3_S: return ggml_type;
     case REIN_GGML_IQ4_NL: return REIN_TYPE_IQ4_XS;
     case REIN_GGML_Q3_K:   return REIN_TYPE_Q6_K;
     case REIN_GGML_BF16:   return REIN_TYPE_Q8_0;
@@ -80,6 +81,15 @@ int label_of(int ggml_type)
 }  // namespace
 
 extern "C" int rein_ingest_format(int ggml_type) { return label_of(ggml_type); }
+
+// the types GpuExpertTensor::from_gguf repacks (src/runtime/qwen35.rs:415-425)
+extern "C" int rein_ingest_expert_format(int ggml_type)
+{
+    switch (ggml_type) {
+    case REIN_TYPE_Q4_K: case REIN_TYPE_Q5_K: case REIN_TYPE_Q6_K: case REIN_TYPE_Q8_0: case REIN_TYPE_Q5_1: return ggml_type;
+    default: return 0;
+    }
+}
 
 extern "C" size_t rein_ingest_src_len(int ggml_type, size_t in_dim, size_t out_dim)
 {
@@ -110,7 +120,7 @@ extern "C" int rein_ingest_for_matvec(int ggml_type, const uint8_t* src, size_t 
     const int label = label_of(ggml_type);
     if (!label)
         return rein::fail(REIN_E_BAD_FORMAT, std::string(who) + ": no repacked layout for ggml type " + std::to_string(ggml_type) +
-                                             " (handled: Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, BF16)");
+                                             " (handled: Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ3_S, IQ4_NL, IQ4_XS, BF16)");
     if (!src || !dst) return rein::fail(REIN_E_BAD_POINTER, std::string(who) + ": null pointer");
     if (out_fmt) *out_fmt = label;
     if (label == ggml_type) return rein_repack_for_matvec(ggml_type, src, in_dim, out_dim, dst);

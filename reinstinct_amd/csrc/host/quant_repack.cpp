@@ -10,6 +10,7 @@
 
 #include "../../../include/rein.h"
 #include "hip_api.h"
+#include "iq3s_grid.h"
 
 namespace {
 
@@ -29,6 +30,8 @@ bool geometry(int fmt, Geometry* g)
     case REIN_TYPE_Q5_K:   *g = {256, 176, 16 + 4 + 2, 4}; return true; // src/quant/q5_k.rs:21-22,100-104
     case REIN_TYPE_Q6_K:   *g = {256, 210, 16 + 8 + 2, 2}; return true; // src/quant/q6_k.rs:18-19,89-93
     case REIN_TYPE_IQ4_XS: *g = {256, 136, 16 + 2, 0}; return true;     // src/quant/iq4_xs.rs:23-24,85-88
+    case REIN_TYPE_Q5_1:   *g = {32, 24, 16 + 4 + 4, 0}; return true;   // src/quant/q5_1.rs:25-26,76-81
+    case REIN_TYPE_IQ3_S:  *g = {256, 110, 16 + 2, 0}; return true;     // src/quant/iq3_s.rs:24-25,178-184
     default: return false;
     }
 }
@@ -104,6 +107,18 @@ inline void emit_nibbles(const SubBlock& s, uint8_t* dst)
     for (int k = 0; k < 16; k++) dst[k] = (uint8_t)(s.lo4[k] | (s.lo4[16 + k] << 4));
 }
 
+// qh word of the Q5_K kernels: bit 4g+b = 5th bit of weight b of dot group g; group 2j is
+// weights 4j.., group 2j+1 weights 16+4j.. (q5_k.rs:122-141, q5_1.rs:70-73)
+inline uint32_t fifth_bits(const SubBlock& w)
+{
+    uint32_t qh = 0;
+    for (int k = 0; k < 16; k++) {
+        qh |= (uint32_t)(w.ext[k] & 1) << (8 * (k / 4) + (k % 4));
+        qh |= (uint32_t)(w.ext[16 + k] & 1) << (8 * (k / 4) + 4 + (k % 4));
+    }
+    return qh;
+}
+
 void repack_rows(int fmt, const Geometry& g, const uint8_t* src, size_t in_dim, size_t out_dim,
                  uint8_t* dst, size_t row_begin, size_t row_end)
 {
@@ -138,6 +153,35 @@ void repack_rows(int fmt, const Geometry& g, const uint8_t* src, size_t in_dim, 
                 store16(dst + n * 16 + i * 2, float_to_half(half_to_float(load16(b)) * (float)(ls - 32)));
                 break;
             }
+            case REIN_TYPE_Q5_1: {     // q5_1.rs:82-104: nibbles verbatim, qh in dot-group order, raw fp16 d | m
+                const uint8_t* b = src + (row * n_sub + sb) * 24;
+                std::memcpy(nib + i * 16, b + 8, 16);
+                const uint32_t bits = (uint32_t)b[4] | ((uint32_t)b[5] << 8) | ((uint32_t)b[6] << 16) | ((uint32_t)b[7] << 24);
+                SubBlock w;
+                for (int k = 0; k < 32; k++) w.ext[k] = (uint8_t)((bits >> k) & 1);   // on disk bit k is weight k
+                const uint32_t qh = fifth_bits(w);
+                std::memcpy(dst + n * 16 + i * 4, &qh, 4);
+                std::memcpy(dst + n * 20 + i * 4, b, 4);
+                break;
+            }
+            case REIN_TYPE_IQ3_S: {    // iq3_s.rs:186-207: signed odd values -> nibble (v + 15) / 2, fp16(d * (1 + 2*scale))
+                const uint8_t* b = src + (row * n_super + sb / 8) * 110;
+                const int s = (int)(sb % 8);
+                const uint8_t* index = b + 2 + 8 * s;                // eight grid indices, low 8 bits
+                const unsigned high = b[66 + s];                     // their 9th bits
+                const uint8_t* sign = b + 74 + 4 * s;                // one bit per weight
+                const int scale = (b[106 + s / 2] >> (4 * (s & 1))) & 15;
+                SubBlock w;
+                for (int k = 0; k < 32; k++) {
+                    const unsigned entry = index[k / 4] | (((high >> (k / 4)) & 1u) << 8);
+                    const int mag = rein::iq3s_magnitude(entry, (unsigned)k % 4);
+                    const int v = ((sign[k / 8] >> (k % 8)) & 1) ? -mag : mag;
+                    w.lo4[k] = (uint8_t)((v + 15) / 2);
+                }
+                emit_nibbles(w, nib + i * 16);
+                store16(dst + n * 16 + i * 2, float_to_half(half_to_float(load16(b)) * (1.0f + 2.0f * (float)scale)));
+                break;
+            }
             case REIN_TYPE_Q4_K:       // q4_k.rs:126-176
             case REIN_TYPE_Q5_K: {     // q5_k.rs:97-151
                 const bool q5 = fmt == REIN_TYPE_Q5_K;
@@ -153,13 +197,7 @@ void repack_rows(int fmt, const Geometry& g, const uint8_t* src, size_t in_dim, 
                 emit_nibbles(w, nib + i * 16);
                 size_t off = n * 16;
                 if (q5) {
-                    // bit 4g+b = 5th bit of weight b of dot group g; group 2j is
-                    // weights 4j.., group 2j+1 weights 16+4j.. (q5_k.rs:122-141)
-                    uint32_t qh = 0;
-                    for (int k = 0; k < 16; k++) {
-                        qh |= (uint32_t)w.ext[k] << (8 * (k / 4) + (k % 4));
-                        qh |= (uint32_t)w.ext[16 + k] << (8 * (k / 4) + 4 + (k % 4));
-                    }
+                    const uint32_t qh = fifth_bits(w);
                     std::memcpy(dst + off + i * 4, &qh, 4);
                     off += n * 4;
                 }

@@ -96,6 +96,8 @@ const char* fmt_tag(int fmt)
     case REIN_TYPE_Q5_K:   return "q5k";
     case REIN_TYPE_Q6_K:   return "q6k";
     case REIN_TYPE_IQ4_XS: return "iq4xs";
+    case REIN_TYPE_Q5_1:   return "q5_1";
+    case REIN_TYPE_IQ3_S:  return "iq3s";
     default: return nullptr;
     }
 }
@@ -107,6 +109,15 @@ int check_shape(const char* who, int fmt, unsigned in_dim, unsigned out_dim, uns
     if (in_dim == 0 || in_dim % (unsigned)bs != 0)
         return fail(REIN_E_BAD_SHAPE, std::string(who) + ": in_dim " + std::to_string(in_dim) + " is not a non-zero multiple of " + std::to_string(bs));
     if (out_dim == 0 || n_rows == 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": out_dim and the row count must be non-zero");
+    return 0;
+}
+
+// Q5_1 has expert kernels only and IQ3_S dense kernels only (src/runtime/qwen35.rs:2264,3045,
+// 3082,3116 are every site the reference dispatches them at).
+int check_dense_fmt(const char* who, int fmt)
+{
+    if (fmt == REIN_TYPE_Q5_1)
+        return fail(REIN_E_BAD_FORMAT, std::string(who) + ": Q5_1 has MoE expert kernels only (a dense Q5_1 tensor keeps its on-disk layout)");
     return 0;
 }
 
@@ -162,7 +173,7 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
     const unsigned planes = fmt == REIN_TYPE_Q8_0 ? 2 : 1;
     const unsigned lds_per_wave = planes * 4096 + 320 * tok;                       // sizeof(SkinnyWaveLds<FMT, TOK>)
     const bool three = nv <= 4 && (fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q8_0 ||
-                                   fmt == REIN_TYPE_IQ4_XS);
+                                   fmt == REIN_TYPE_IQ4_XS || fmt == REIN_TYPE_IQ3_S);
     const unsigned occ = three ? 3 : 2;                                            // wavefronts per SIMD (registers)
     const unsigned waves_per_cu = std::min(4 * occ, 160u * 1024u / lds_per_wave);
     const unsigned ks_max = std::min(std::min(8u, waves_per_cu), n_chunks);        // the kernels' launch bound is 512 threads
@@ -206,6 +217,7 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
                   unsigned out_dim, unsigned n_rows, rein_stream_t s)
 {
     if (int rc = check_shape(who, fmt, in_dim, out_dim, n_rows)) return rc;
+    if (int rc = check_dense_fmt(who, fmt)) return rc;
     if (n_rows > 8) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most 8 activation rows");
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
@@ -472,6 +484,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
 {
     const char* who = "rein_mmq_xq8";
     if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
+    if (int rc = check_dense_fmt(who, fmt)) return rc;
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
@@ -514,6 +527,7 @@ int rein_matmul(int fmt, const void* w, const float* x, float* y, unsigned in_di
                 unsigned n_rows, void* xq_scratch, rein_stream_t s)
 {
     if (int rc = check_shape("rein_matmul", fmt, in_dim, out_dim, n_rows)) return rc;
+    if (int rc = check_dense_fmt("rein_matmul", fmt)) return rc;
     if (int rc = rein_quantize_q8(x, xq_scratch, in_dim, n_rows, s)) return rc;
     switch (rein_matmul_path(fmt, n_rows)) {
     case 0:  return rein_matvec_xq8(fmt, w, xq_scratch, y, in_dim, out_dim, s);
@@ -534,6 +548,7 @@ int rein_block_dots(int fmt, const void* w, const void* xq, int32_t* out, unsign
     if (int rc = check_ptr(who, out, 4, "out")) return rc;
     if (n_rows > 65535) return fail(REIN_E_TOO_LARGE, "rein_block_dots: at most 65535 rows");
     if (via_mfma) {
+        if (int rc = check_dense_fmt(who, fmt)) return rc;
         const std::string name = std::string("rein_mmq_dots_") + fmt_tag(fmt);
         void* args[] = {(void*)&w, (void*)&xq, (void*)&out, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
         return launch(name, (out_dim + 127) / 128, (n_rows + 31) / 32, 1, 256, 0, s, args);
@@ -619,8 +634,8 @@ int rein_moe_grouped_gemm(int fmt, const void* slab, unsigned bytes_per_expert, 
                           unsigned out_dim, unsigned n_entries, rein_stream_t s)
 {
     const char* who = "rein_moe_grouped_gemm";
-    if (fmt != REIN_TYPE_Q4_K && fmt != REIN_TYPE_Q5_K && fmt != REIN_TYPE_Q6_K && fmt != REIN_TYPE_Q8_0)
-        return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (!rein_ingest_expert_format(fmt))
+        return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0, Q5_1");
     if (int rc = check_shape(who, fmt, in_dim, out_dim, n_entries)) return rc;
     if (n_expert == 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_expert is zero");
     if (bytes_per_expert % 16 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert must be a multiple of 16");
@@ -666,7 +681,7 @@ int moe_mv_launch(const char* who, const std::string& kernel, unsigned rows_per_
                  (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
     return launch(kernel, gx, n_used, n_tok, 256, 0, s, a);
 }
-bool moe_mv_fmt(int fmt) { return fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q8_0; }
+bool moe_mv_fmt(int fmt) { return rein_ingest_expert_format(fmt) != 0; }       // Q4_K, Q5_K, Q6_K, Q8_0, Q5_1
 }  // namespace
 
 int rein_moe_expert_matvec(int fmt, const void* slab, const int32_t* ids, const void* xq, float* y, unsigned in_dim,
@@ -674,7 +689,7 @@ int rein_moe_expert_matvec(int fmt, const void* slab, const int32_t* ids, const 
                            unsigned xq_slot_stride, unsigned n_used, unsigned n_tok, rein_stream_t s)
 {
     const char* who = "rein_moe_expert_matvec";
-    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0, Q5_1");
     // 4 wavefronts x 2 rows per 256-thread workgroup (the reference's grid, qwen35.rs:3086)
     return moe_mv_launch(who, std::string("moe_matvec_") + fmt_tag(fmt) + "_repacked_f32", 8, fmt, slab, nullptr, ids, xq,
                          y, in_dim, out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, s);
@@ -685,7 +700,7 @@ int rein_moe_down(int fmt, const void* slab, const int32_t* ids, const void* xq,
                   unsigned n_used, unsigned n_tok, rein_stream_t s)
 {
     const char* who = "rein_moe_down";
-    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0, Q5_1");
     if (in_dim / 32 > 32)       // long contraction: the full-wavefront mapping wastes nothing
         return rein_moe_expert_matvec(fmt, slab, ids, xq, y, in_dim, out_dim, bytes_per_expert, xq_tok_stride,
                                       xq_slot_stride, n_used, n_tok, s);

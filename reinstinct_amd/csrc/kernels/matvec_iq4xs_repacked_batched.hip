@@ -6,3 +6,7 @@
 
 REIN_DEFINE_MATVEC_BATCHED(matvec_iq4xs_repacked_batched_f32, REIN_IQ4_XS, 2, 4)
 REIN_DEFINE_MATVEC_BATCHED(matvec_iq4xs_repacked_batched16_f32, REIN_IQ4_XS, 1, 16)
+
+// the same kernels with the IQ3_S codebook (src/runtime/prefill.rs:473-474)
+REIN_DEFINE_MATVEC_BATCHED(matvec_iq3s_repacked_batched_f32, REIN_IQ3_S, 2, 4)
+REIN_DEFINE_MATVEC_BATCHED(matvec_iq3s_repacked_batched16_f32, REIN_IQ3_S, 1, 16)

@@ -67,12 +67,6 @@ struct __attribute__((packed, aligned(2))) ReinU16x8 { uint16_t v[8]; };
 struct __attribute__((packed, aligned(4))) ReinU32x8 { uint32_t v[8]; };
 struct __attribute__((packed, aligned(8))) ReinU64x8 { uint2 v[8]; };
 
-// (x - c) per byte for bytes x in [0,127], c < 128: no borrow crosses a byte
-__device__ __forceinline__ int rein_sub_bytes(uint32_t x, uint32_t c4)
-{
-    return (int)(((x | 0x80808080u) - c4) ^ 0x80808080u);
-}
-
 // Weight side of one superblock chunk (8 sub-blocks) for lane (row, half h).
 // The 16-byte-per-sub-block plane (nibbles; Q8_0: the lane half's quant plane) is
 // kept apart from the small words (aux bits, scales, fp16 pair), because the tuned
@@ -103,7 +97,7 @@ template <int FMT, class Self> struct MmqChunkBase {
 };
 
 template <> struct MmqChunk<REIN_Q4_K> : MmqChunkBase<REIN_Q4_K, MmqChunk<REIN_Q4_K>> {
-    static constexpr bool kTwoScales = false, kHasMin = true;
+    static constexpr bool kTwoScales = false, kHasMin = true, kMinSplit = false;
     struct Small { ReinU16x8 sm; uint32_t dd; };
     struct Raw { uint4 q[8]; Small sm; };
     float sc[4], ndmin;
@@ -152,7 +146,7 @@ template <> struct MmqChunk<REIN_Q4_K> : MmqChunkBase<REIN_Q4_K, MmqChunk<REIN_Q
 };
 
 template <> struct MmqChunk<REIN_Q5_K> : MmqChunkBase<REIN_Q5_K, MmqChunk<REIN_Q5_K>> {
-    static constexpr bool kTwoScales = false, kHasMin = true;
+    static constexpr bool kTwoScales = false, kHasMin = true, kMinSplit = false;
     struct Small { ReinU32x8 qh; ReinU16x8 sm; uint32_t dd; };
     struct Raw { uint4 q[8]; Small sm; };
     float sc[4], ndmin;
@@ -187,6 +181,73 @@ template <> struct MmqChunk<REIN_Q5_K> : MmqChunkBase<REIN_Q5_K, MmqChunk<REIN_Q
         m4.w = rein_bf16_of_u8(r.sm.v[6] >> 8) | (rein_bf16_of_u8(r.sm.v[7] >> 8) << 16);
         mb = __builtin_bit_cast(rein_v8bf, m4);
         ndmin = -dmin;
+    }
+    static __device__ __forceinline__ rein_v4i operand(const uint4& q, const Small& r, int s, unsigned h)
+    {
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        rein_v4i o;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            o[j] = (int)(((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | (rein_spread4(r.qh.v[s] >> (8 * j + 4 * h)) << 4));
+        return o;
+    }
+    __device__ __forceinline__ void rotate(Small& r)
+    {
+        sc[0] = sc[1]; sc[1] = sc[2]; sc[2] = sc[3];
+#pragma unroll
+        for (int i = 0; i < 6; i++) r.qh.v[i] = r.qh.v[i + 2];
+    }
+};
+
+// Q5_1: the Q5_K operand with a raw fp16 (d, m) per sub-block.  The minimum term
+// sum_s m_s * xsum_s goes through the bf16 MFMA like Q5_K's, but m_s is an fp16 value, not
+// a 6-bit integer under a shared dmin: it is split into a bf16 head (8 significant bits)
+// and the exact remainder (the other 3), so the products stay exact.  in_dim is only a
+// multiple of 32: sub-blocks past the end are clamped and zero-scaled.
+template <> struct MmqChunk<REIN_Q5_1> : MmqChunkBase<REIN_Q5_1, MmqChunk<REIN_Q5_1>> {
+    static constexpr bool kTwoScales = false, kHasMin = true, kMinSplit = true;
+    struct Small { ReinU32x8 qh; ReinU32x8 dm; };
+    struct Raw { uint4 q[8]; Small sm; };
+    float sc[4], ndmin;
+    rein_v8bf mb, mb_lo;
+    static __device__ __forceinline__ const uint4* plane(const Fmt<REIN_Q5_1>& f, unsigned) { return f.nib; }
+    static __device__ __forceinline__ void fetch_small(Small& r, const Fmt<REIN_Q5_1>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned)
+    {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const size_t i = (size_t)row * f.nsp + rein_clamp_sb(sb0 + s, n_sub);
+            r.qh.v[s] = f.qhp[i];
+            r.dm.v[s] = f.dmp[i];
+        }
+    }
+    static __device__ __forceinline__ void fetch(Raw& r, const Fmt<REIN_Q5_1>& f, unsigned row, unsigned sb0, unsigned n_sub, unsigned h)
+    {
+#pragma unroll
+        for (int s = 0; s < 8; s++) r.q[s] = f.nib[(size_t)row * f.nsp + rein_clamp_sb(sb0 + s, n_sub)];
+        fetch_small(r.sm, f, row, sb0, n_sub, h);
+    }
+    __device__ __forceinline__ void prepare(const Small& r, unsigned sb0, unsigned n_sub, unsigned h)
+    {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t v = h ? r.dm.v[2 * p + 1] : r.dm.v[2 * p];
+            sc[p] = sb0 + 2 * p + h < n_sub ? rein_h2f((uint16_t)(v & 0xFFFFu)) : 0.0f;
+        }
+        uint32_t hi[8], lo[8];
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const float m = sb0 + s < n_sub ? rein_h2f((uint16_t)(r.dm.v[s] >> 16)) : 0.0f;
+            const uint32_t head = __builtin_bit_cast(uint32_t, m) & 0xFFFF0000u;
+            const float rest = m - __builtin_bit_cast(float, head);          // at most 3 significant bits: exact in bf16
+            hi[s] = head >> 16;
+            lo[s] = __builtin_bit_cast(uint32_t, rest) >> 16;
+        }
+        uint4 m4;
+        m4.x = hi[0] | (hi[1] << 16); m4.y = hi[2] | (hi[3] << 16); m4.z = hi[4] | (hi[5] << 16); m4.w = hi[6] | (hi[7] << 16);
+        mb = __builtin_bit_cast(rein_v8bf, m4);
+        m4.x = lo[0] | (lo[1] << 16); m4.y = lo[2] | (lo[3] << 16); m4.z = lo[4] | (lo[5] << 16); m4.w = lo[6] | (lo[7] << 16);
+        mb_lo = __builtin_bit_cast(rein_v8bf, m4);
+        ndmin = 1.0f;                                                        // the term is + m * xsum (deff = -m)
     }
     static __device__ __forceinline__ rein_v4i operand(const uint4& q, const Small& r, int s, unsigned h)
     {
@@ -255,7 +316,7 @@ template <> struct MmqChunk<REIN_Q6_K> : MmqChunkBase<REIN_Q6_K, MmqChunk<REIN_Q
     }
 };
 
-// Q8_0 / Q4_0 / IQ4_XS: one fp16 scale per sub-block, the chunk may be ragged
+// Q8_0 / Q4_0 / IQ4_XS / IQ3_S: one fp16 scale per sub-block, the chunk may be ragged
 // (in_dim is only a multiple of 32): sub-blocks past the end are clamped and
 // their scale is forced to zero.
 template <int FMT> struct MmqChunkD16 : MmqChunkBase<FMT, MmqChunk<FMT>> {
@@ -293,7 +354,7 @@ template <int FMT> struct MmqChunkD16 : MmqChunkBase<FMT, MmqChunk<FMT>> {
         for (int j = 0; j < 4; j++) {
             if constexpr (FMT == REIN_Q8_0) o[j] = (int)w[j];
             else if constexpr (FMT == REIN_Q4_0) o[j] = rein_sub_bytes((w[j] >> (4 * h)) & 0x0F0F0F0Fu, 0x08080808u);
-            else o[j] = rein_iq4_lut4((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
+            else o[j] = rein_codebook4<FMT>((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
         }
         return o;
     }
@@ -302,6 +363,7 @@ template <int FMT> struct MmqChunkD16 : MmqChunkBase<FMT, MmqChunk<FMT>> {
 template <> struct MmqChunk<REIN_Q8_0> : MmqChunkD16<REIN_Q8_0> {};
 template <> struct MmqChunk<REIN_Q4_0> : MmqChunkD16<REIN_Q4_0> {};
 template <> struct MmqChunk<REIN_IQ4_XS> : MmqChunkD16<REIN_IQ4_XS> {};
+template <> struct MmqChunk<REIN_IQ3_S> : MmqChunkD16<REIN_IQ3_S> {};
 
 // LDS image of one activation chunk: TM tokens x 8 sub-blocks.  xsb holds each
 // block's xsum split into three bf16 (truncated head, then the exact remainders),
@@ -447,6 +509,7 @@ __device__ __forceinline__ void rein_mmq_chunk_math(const MmqLds<TM>& lds, const
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (C::kHasMin && DOTS == 0) {
+            static_assert(!C::kMinSplit, "split minimums are handled by the pipelined tile only");
             // sum over the 8 sub-blocks of m * xsum: lane half 0 carries the heads of
             // the xsum splits, half 1 the first remainders, a second MFMA the last
             // remainders (its half 1 multiplies zeros)
@@ -724,19 +787,37 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
         ck.rotate(sm);
     }
     if constexpr (C::kHasMin) {
-        const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
-        const rein_v8bf mb2 = h ? __builtin_bit_cast(rein_v8bf, z4) : ck.mb;
         rein_v16f z16;
 #pragma unroll
         for (int v = 0; v < 16; v++) z16[v] = 0.0f;
+        if constexpr (C::kMinSplit) {
+            // fp16 minimums as head + remainder: six (xsum split, minimum part) products
+            // of eight sub-blocks each, two per MFMA (one per lane half)
+            const rein_v8bf b_mid = h ? ck.mb_lo : ck.mb;
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const uint4 x01 = *reinterpret_cast<const uint4*>(lds.xsb[h][t * 32 + j]);
-            const uint4 x2  = *reinterpret_cast<const uint4*>(lds.xsb[2][t * 32 + j]);
-            rein_v16f m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x01), ck.mb, z16, 0, 0, 0);
-            m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x2), mb2, m, 0, 0, 0);
+            for (int t = 0; t < NT; t++) {
+                const uint4 x0 = *reinterpret_cast<const uint4*>(lds.xsb[0][t * 32 + j]);
+                const uint4 x1 = *reinterpret_cast<const uint4*>(lds.xsb[1][t * 32 + j]);
+                const uint4 x2 = *reinterpret_cast<const uint4*>(lds.xsb[2][t * 32 + j]);
+                const uint4 a1 = h ? x1 : x0, a2 = h ? x0 : x2, a3 = h ? x2 : x1;
+                rein_v16f m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, a1), ck.mb, z16, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, a2), b_mid, m, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, a3), ck.mb_lo, m, 0, 0, 0);
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[t][v] = fmaf(m[v], ck.ndmin, acc[t][v]);
+                for (int v = 0; v < 16; v++) acc[t][v] = fmaf(m[v], ck.ndmin, acc[t][v]);
+            }
+        } else {
+            const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
+            const rein_v8bf mb2 = h ? __builtin_bit_cast(rein_v8bf, z4) : ck.mb;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 x01 = *reinterpret_cast<const uint4*>(lds.xsb[h][t * 32 + j]);
+                const uint4 x2  = *reinterpret_cast<const uint4*>(lds.xsb[2][t * 32 + j]);
+                rein_v16f m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x01), ck.mb, z16, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rein_v8bf, x2), mb2, m, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[t][v] = fmaf(m[v], ck.ndmin, acc[t][v]);
+            }
         }
     }
 }

@@ -167,6 +167,7 @@ template <int FMT> struct SkinnyD16 {
 template <> struct SkinnyFmt<REIN_Q8_0> : SkinnyD16<REIN_Q8_0> {};
 template <> struct SkinnyFmt<REIN_Q4_0> : SkinnyD16<REIN_Q4_0> {};
 template <> struct SkinnyFmt<REIN_IQ4_XS> : SkinnyD16<REIN_IQ4_XS> {};
+template <> struct SkinnyFmt<REIN_IQ3_S> : SkinnyD16<REIN_IQ3_S> {};
 
 // ---- the 16-byte weight plane(s) of one chunk: 32 rows x 8 sub-blocks -------------
 // In registers as loaded: lane l of load i holds row 8i + l/8, sub-block l%8.

@@ -28,3 +28,7 @@ REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q8_0_v1, REIN_Q8_0, 1, 3)
 REIN_DEFINE_MMQ_SKINNY(rein_mmqs_q8_0_v2, REIN_Q8_0, 2, 3)
 REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq4xs_v1, REIN_IQ4_XS, 1, 3)
 REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq4xs_v2, REIN_IQ4_XS, 2, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq3s_v1, REIN_IQ3_S, 1, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq3s_v2, REIN_IQ3_S, 2, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq3s_v4, REIN_IQ3_S, 4, 3)
+REIN_DEFINE_MMQ_SKINNY(rein_mmqs_iq3s_v8, REIN_IQ3_S, 8, 2)

@@ -131,6 +131,10 @@ REIN_DEFINE_MOE_MV(moe_matvec_q8_0_repacked_f32, REIN_Q8_0, 2, 64)
 REIN_DEFINE_MOE_MV(moe_matvec_q5k_down_f32, REIN_Q5_K, 2, 32)
 REIN_DEFINE_MOE_MV(moe_matvec_q6k_down_f32, REIN_Q6_K, 2, 32)
 REIN_DEFINE_MOE_MV(moe_matvec_q8_0_repacked_down_f32, REIN_Q8_0, 2, 32)
+// Q5_1 experts: the Q5_K kernels with the raw (d, m) scale decode (the reference's second
+// compilation with Q5_1_SCALES, qwen35.rs:3082,3116)
+REIN_DEFINE_MOE_MV(moe_matvec_q5_1_repacked_f32, REIN_Q5_1, 2, 64)
+REIN_DEFINE_MOE_MV(moe_matvec_q5_1_down_f32, REIN_Q5_1, 2, 32)
 // the same for the format the reference has no down kernel for (it falls back to the
 // generic one, qwen35.rs:3118-3120)
 REIN_DEFINE_MOE_MV(rein_moe_matvec_q4k_down_f32, REIN_Q4_K, 2, 32)

@@ -27,6 +27,9 @@ enum ReinFmt : int {
     REIN_Q5_K   = 13,
     REIN_Q6_K   = 14,
     REIN_IQ4_XS = 23,
+    // relabelled formats: another format's planes and kernels with one decode step swapped
+    REIN_Q5_1   = 7,    // Q5_K's nibble and qh planes, raw fp16 (d, m) per sub-block (src/quant/q5_1.rs:12-20)
+    REIN_IQ3_S  = 21,   // IQ4_XS's planes, codebook value 2n - 15 (src/quant/iq3_s.rs:13-19)
 };
 
 // Unpacked sub-block.
@@ -79,6 +82,19 @@ __device__ __forceinline__ int rein_iq4_lut4(uint32_t n4)
     const uint32_t hi  = __builtin_amdgcn_perm(REIN_KV_12_15, REIN_KV_8_11, sel);
     const uint32_t m   = ((n4 >> 3) & 0x01010101u) * 0xFFu;
     return (int)((hi & m) | (lo & ~m));
+}
+
+// (x - c) per byte for bytes x in [0,127], c < 128: no borrow crosses a byte
+__device__ __forceinline__ int rein_sub_bytes(uint32_t x, uint32_t c4)
+{
+    return (int)(((x | 0x80808080u) - c4) ^ 0x80808080u);
+}
+
+// four nibbles (one per byte) -> the four int8 weight values of a codebook format
+template <int FMT> __device__ __forceinline__ int rein_codebook4(uint32_t n4)
+{
+    if constexpr (FMT == REIN_IQ3_S) return rein_sub_bytes(n4 << 1, 0x0F0F0F0Fu);   // KVALUES_IQ3S[n] = 2n - 15 (iq3_s.rs:161-162)
+    else return rein_iq4_lut4(n4);
 }
 
 // Streaming (nontemporal) loads for the matvec weight planes: every weight byte is
@@ -345,13 +361,14 @@ template <> struct Fmt<REIN_Q4_0> {
 };
 
 // ---------------------------------------------------------------- IQ4_XS
-template <> struct Fmt<REIN_IQ4_XS> {
+// IQ4_XS and IQ3_S share planes and arithmetic; FMT selects the codebook.
+template <int FMT> struct FmtCodebook16 {
     static constexpr bool kNeedsXSums = false;
     struct Raw { uint4 q; uint16_t d; };
     const uint4*    nib;
     const uint16_t* dp;
     unsigned nsp;
-    __device__ Fmt(const uint8_t* w, unsigned n_sub, unsigned out_dim)
+    __device__ FmtCodebook16(const uint8_t* w, unsigned n_sub, unsigned out_dim)
     {
         nsp = rein_nsp(n_sub);
         const size_t n = (size_t)out_dim * nsp;
@@ -371,8 +388,8 @@ template <> struct Fmt<REIN_IQ4_XS> {
         const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            s.w[j]     = rein_iq4_lut4(q[j] & 0x0F0F0F0Fu);
-            s.w[j + 4] = rein_iq4_lut4((q[j] >> 4) & 0x0F0F0F0Fu);
+            s.w[j]     = rein_codebook4<FMT>(q[j] & 0x0F0F0F0Fu);
+            s.w[j + 4] = rein_codebook4<FMT>((q[j] >> 4) & 0x0F0F0F0Fu);
         }
         s.s0 = rein_h2f(r.d);
         s.s1 = 0.0f;
@@ -381,6 +398,55 @@ template <> struct Fmt<REIN_IQ4_XS> {
     static __device__ __forceinline__ float term(const SubW& s, int i0, int i1, float dx, float, XSums)
     {
         return s.s0 * dx * (float)(i0 + i1);
+    }
+    static constexpr int kDotParts = 1;
+    static __device__ __forceinline__ void parts(int i0, int i1, XSums, int out[2]) { out[0] = i0 + i1; out[1] = 0; }
+};
+template <> struct Fmt<REIN_IQ4_XS> : FmtCodebook16<REIN_IQ4_XS> { using FmtCodebook16<REIN_IQ4_XS>::FmtCodebook16; };
+template <> struct Fmt<REIN_IQ3_S> : FmtCodebook16<REIN_IQ3_S> { using FmtCodebook16<REIN_IQ3_S>::FmtCodebook16; };
+
+// ------------------------------------------------------------------ Q5_1
+// The Q5_K unpack with the scale decode of the reference's Q5_1_SCALES build
+// (kernels/moe_matvec_q5k_repacked.cpp:57-60,86-91): dsc = d, deff = -m, both raw fp16
+// per sub-block.  in_dim is a multiple of 32 only.
+template <> struct Fmt<REIN_Q5_1> {
+    static constexpr bool kNeedsXSums = false;
+    struct Raw { uint4 q; uint32_t qh; uint32_t dm; };
+    const uint4*    nib;
+    const uint32_t* qhp;
+    const uint32_t* dmp;
+    unsigned nsp;
+    __device__ Fmt(const uint8_t* w, unsigned n_sub, unsigned out_dim)
+    {
+        nsp = rein_nsp(n_sub);
+        const size_t n = (size_t)out_dim * nsp;
+        nib = reinterpret_cast<const uint4*>(w);
+        qhp = reinterpret_cast<const uint32_t*>(w + n * 16);
+        dmp = reinterpret_cast<const uint32_t*>(w + n * 20);
+    }
+    __device__ __forceinline__ Raw load(unsigned row, unsigned sb) const
+    {
+        const size_t i = (size_t)row * nsp + sb;
+        Raw r;
+        r.q  = rein_ldw(&nib[i]);
+        r.qh = rein_ldw(&qhp[i]);
+        r.dm = rein_ldw(&dmp[i]);
+        return r;
+    }
+    static __device__ __forceinline__ void unpack(const Raw& r, SubW& s)
+    {
+        const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            s.w[j]     = (int)((q[j] & 0x0F0F0F0Fu) | (rein_spread4(r.qh >> (8 * j)) << 4));
+            s.w[j + 4] = (int)(((q[j] >> 4) & 0x0F0F0F0Fu) | (rein_spread4(r.qh >> (8 * j + 4)) << 4));
+        }
+        s.s0 = rein_h2f((uint16_t)(r.dm & 0xFFFFu));
+        s.s1 = -rein_h2f((uint16_t)(r.dm >> 16));
+    }
+    static __device__ __forceinline__ float term(const SubW& s, int i0, int i1, float dx, float xsum, XSums)
+    {
+        return s.s0 * dx * (float)(i0 + i1) - s.s1 * xsum;
     }
     static constexpr int kDotParts = 1;
     static __device__ __forceinline__ void parts(int i0, int i1, XSums, int out[2]) { out[0] = i0 + i1; out[1] = 0; }

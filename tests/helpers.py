@@ -63,6 +63,11 @@ def random_raw_weights(fmt, in_dim, out_dim, seed):
         put(0, ((blk % 29) - 14) * 0.0005)
     elif fmt == orc.IQ4_XS:
         put(0, ((blk % 23) - 11) * 0.005)
+    elif fmt == orc.IQ3_S:
+        put(0, ((blk % 23) - 11) * 0.0008)
+    elif fmt == orc.Q5_1:
+        put(0, ((blk % 29) - 14) * 0.003)
+        put(2, ((blk % 17) - 8) * 0.0123)
     return raw.reshape(-1)
 
 

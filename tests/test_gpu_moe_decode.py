@@ -16,8 +16,8 @@ from oracle import orc
 from helpers import assert_close_f32, random_raw_weights
 
 pytestmark = pytest.mark.gpu
-FMTS = [rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0]
-NAME = {rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k", rein.Q8_0: "q8_0"}
+FMTS = [rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.Q5_1]
+NAME = {rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k", rein.Q8_0: "q8_0", rein.Q5_1: "q5_1"}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -36,7 +36,7 @@ def expert_slabs(fmt, in_dim, out_dim, n_expert, seed, gaussian=True):
     # out_dim a multiple of 8 keeps every expert's slab 16-byte aligned (the library checks it)
     slabs = []
     for e in range(n_expert):
-        if gaussian:
+        if gaussian and fmt != rein.Q5_1:               # no synthetic quantizer for Q5_1
             w = (np.random.default_rng(seed + e).standard_normal((out_dim, in_dim)) * 0.02).astype(np.float32)
             raw = quant.quantize_weights(fmt, w)
         else:

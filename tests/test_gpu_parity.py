@@ -19,9 +19,10 @@ from helpers import Lcg, assert_close_f32, random_raw_weights, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-ALL = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS]
+# the six formats plus IQ3_S, which runs the IQ4_XS kernels with its own codebook (dense paths only)
+ALL = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS, rein.IQ3_S]
 NAME = {rein.Q4_0: "q4_0", rein.Q8_0: "q8_0", rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k",
-        rein.IQ4_XS: "iq4xs"}
+        rein.IQ4_XS: "iq4xs", rein.IQ3_S: "iq3s", rein.Q5_1: "q5_1"}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -38,7 +39,7 @@ def dev(a):
 
 
 def make_weights(fmt, in_dim, out_dim, seed, gaussian=False):
-    if gaussian:
+    if gaussian and fmt not in (rein.IQ3_S, rein.Q5_1):       # no synthetic quantizer for the relabelled formats
         w = (np.random.default_rng(seed).standard_normal((out_dim, in_dim)) * 0.02).astype(np.float32)
         raw = quant.quantize_weights(fmt, w)
     else:
@@ -397,9 +398,10 @@ def test_moe_gather_scatter_swiglu_combine():
     assert np.array_equal(d_out.to_host(np.float32).reshape(n_tok, dim), orc.moe_combine(experts, ids, w, s))
 
 
-@pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0])
-def test_grouped_gemm_parity(fmt):
-    in_dim, out_dim, n_expert, n_tok, n_used = 512, 136, 6, 40, 2
+@pytest.mark.parametrize("fmt,in_dim", [(rein.Q4_K, 512), (rein.Q5_K, 512), (rein.Q6_K, 512), (rein.Q8_0, 512),
+                                        (rein.Q5_1, 512), (rein.Q5_1, 352), (rein.Q5_1, 96), (rein.Q8_0, 352)])
+def test_grouped_gemm_parity(fmt, in_dim):
+    out_dim, n_expert, n_tok, n_used = 136, 6, 40, 2
     bpe = quant.repacked_len(fmt, in_dim, out_dim)
     slabs = [make_weights(fmt, in_dim, out_dim, seed=200 + e)[1] for e in range(n_expert)]
     slab = np.concatenate(slabs)
