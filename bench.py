@@ -39,7 +39,7 @@ INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 CACHE_BYTES = 512 << 20        # rotate over more than L2 (32 MB) + Infinity Cache (256 MB)
 
 FMT_NAME = {rein.Q4_0: "q4_0", rein.Q4_K: "q4_k", rein.Q5_K: "q5_k", rein.Q6_K: "q6_k", rein.Q8_0: "q8_0",
-            rein.IQ4_XS: "iq4_xs"}
+            rein.IQ4_XS: "iq4_xs", rein.IQ3_S: "iq3_s"}
 
 
 def log(*a):
@@ -49,6 +49,13 @@ def log(*a):
 def synth_weights(fmt, in_dim, out_dim, seed):
     """fp32 ~N(0,0.02) -> on-disk blocks -> repacked-v2 slab (host)."""
     rng = np.random.default_rng(seed)
+    if fmt == rein.IQ3_S:
+        # no fp32 -> IQ3_S quantizer exists (the reference has none either): seeded random
+        # blocks with a tame fp16 scale; the kernels' speed does not depend on the values
+        raw = rng.integers(0, 256, (out_dim * in_dim // 256, 110), dtype=np.uint8)
+        raw[:, 0:2] = np.frombuffer(np.float16(0.002).tobytes(), np.uint8)
+        raw = raw.reshape(-1)
+        return raw, quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     w = (rng.standard_normal((out_dim, in_dim), dtype=np.float32) * np.float32(0.02))
     raw = quant.quantize_weights(fmt, w)
     return raw, quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
@@ -526,7 +533,7 @@ def main():
 
     if args.sweep:
         sweep = []
-        for f in (rein.Q4_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.IQ4_XS):
+        for f in (rein.Q4_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.IQ4_XS, rein.IQ3_S):
             for (k, n) in HEADLINE_SHAPES:
                 _, packed = synth_weights(f, k, n, seed=5)
                 for b in (1, 2, 4, 8):

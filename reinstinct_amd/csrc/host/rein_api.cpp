@@ -234,6 +234,35 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     return launch(name, grid, 1, 1, wpb * 64, 0, s, args);
 }
 
+// Grouped GEMM launch.  The tile count lives on the device; the grid covers its upper bound
+// (qwen35.rs:3051).  One tile per workgroup (rein_mmq_<fmt>_grouped_t32, grid.z = 2 when a
+// second slab / output pair is given) as long as that bound fits grid.y; beyond it the
+// reference-named kernel, which strides over tiles, once per slab.
+int launch_grouped(int fmt, const void* slab0, const void* slab1, unsigned bytes_per_expert, const int32_t* expert_off,
+                   const int32_t* tile_off, unsigned n_expert, const void* xq, float* y0, float* y1, unsigned in_dim,
+                   unsigned out_dim, unsigned n_entries, rein_stream_t s)
+{
+    const unsigned bn = rein_moe_gemm_bn();
+    const unsigned tile_ub = (n_entries + bn - 1) / bn + n_expert;
+    const unsigned gx = (out_dim + 127) / 128;
+    if (tile_ub <= 65535 && env_u("REIN_GROUPED_STRIDED", 0) == 0) {
+        const void* s1 = slab1 ? slab1 : slab0;
+        float* o1 = y1 ? y1 : y0;
+        void* a[] = {(void*)&slab0, (void*)&s1, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off,
+                     (void*)&n_expert, (void*)&xq, (void*)&y0, (void*)&o1, (void*)&in_dim, (void*)&out_dim};
+        return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_grouped_t32", gx, tile_ub, slab1 ? 2 : 1, 256, 0, s, a);
+    }
+    const std::string name = std::string("mmq_gemm_") + fmt_tag(fmt) + "_grouped_f32";
+    for (int z = 0; z < (slab1 ? 2 : 1); z++) {
+        const void* slab = z ? slab1 : slab0;
+        float* y = z ? y1 : y0;
+        void* a[] = {(void*)&slab, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off, (void*)&n_expert,
+                     (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim};
+        if (int rc = launch(name, gx, std::min(tile_ub, 65535u), 1, 256, 0, s, a)) return rc;
+    }
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -644,14 +673,8 @@ int rein_moe_grouped_gemm(int fmt, const void* slab, unsigned bytes_per_expert, 
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     if (int rc = check_ptr(who, expert_off, 4, "expert_off")) return rc;
     if (int rc = check_ptr(who, tile_off, 4, "tile_off")) return rc;
-    // the tile count lives on the device; launch its upper bound (qwen35.rs:3051)
-    const unsigned bn = rein_moe_gemm_bn();
-    unsigned tile_ub = (n_entries + bn - 1) / bn + n_expert;
-    if (tile_ub > 65535) tile_ub = 65535;       // the kernel strides over tiles
-    const std::string name = std::string("mmq_gemm_") + fmt_tag(fmt) + "_grouped_f32";
-    void* a[] = {(void*)&slab, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off, (void*)&n_expert,
-                 (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim};
-    return launch(name, (out_dim + 127) / 128, tile_ub, 1, 256, 0, s, a);
+    return launch_grouped(fmt, slab, nullptr, bytes_per_expert, expert_off, tile_off, n_expert, xq, y, nullptr, in_dim,
+                          out_dim, n_entries, s);
 }
 
 namespace {
@@ -845,19 +868,8 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     }
     if (int rc = rein_moe_gather_xq(base + w.xq_in, perm, base + w.g_in, sh.hidden / 32, sh.n_used, ne, s)) return rc;
     // gate and up projections in one launch (grid.z = 2)
-    {
-        const unsigned bn = rein_moe_gemm_bn();
-        unsigned tile_ub = (ne + bn - 1) / bn + sh.n_expert;
-        if (tile_ub > 65535) tile_ub = 65535;
-        const unsigned bpe = (unsigned)bpe_gu;
-        const void* xq_in = base + w.g_in;
-        float* y0 = (float*)(base + w.e_gate);
-        float* y1 = (float*)(base + w.e_up);
-        const std::string name = std::string("rein_mmq_") + fmt_tag(sh.gate_up_fmt) + "_grouped_pair";
-        void* a[] = {(void*)&gate_exps, (void*)&up_exps, (void*)&bpe, (void*)&eoff, (void*)&toff, (void*)&sh.n_expert,
-                     (void*)&xq_in, (void*)&y0, (void*)&y1, (void*)&sh.hidden, (void*)&sh.expert_ff};
-        if (int rc = launch(name, (sh.expert_ff + 127) / 128, tile_ub, 2, 256, 0, s, a)) return rc;
-    }
+    if (int rc = launch_grouped(sh.gate_up_fmt, gate_exps, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert, base + w.g_in,
+                                (float*)(base + w.e_gate), (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;
     // SwiGLU straight into the down projection's BlockQ8 rows (rows are expert_ff long,
     // a multiple of 32, so the flat array quantizes as one vector)
     for (size_t e0 = 0; e0 < (size_t)ne * sh.expert_ff; e0 += (size_t)1 << 30) {

@@ -966,20 +966,36 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     }
 }
 
-// Two grouped GEMMs over the same sorted activations in one launch (the gate and up
-// projections of an expert FFN): blockIdx.z selects the slab and its output.  Twice
-// the workgroups per launch fill the machine better than two launches of half the
-// size, and the second launch's fill / drain disappears.
+// The library's own launch of the grouped GEMM: exactly one tile per workgroup --
+// blockIdx.x = 128-row block, blockIdx.y = token tile (the host launches an upper bound of
+// the tile count; surplus workgroups leave at once), blockIdx.z selects one of two slabs
+// with its output, so that the gate and the up projection of an expert FFN run in one
+// launch (twice the workgroups fill the machine better than two launches of half the
+// size, and the second launch's fill / drain disappears).  Without the grid-stride loops
+// of rein_mmq_grouped around it the tile keeps to the register budget of three
+// wavefronts per SIMD, which is what hides the pipeline fill of the short contractions
+// of expert FFNs (24 to 64 sub-blocks).  Requires gridDim.x >= ceil(out_dim / 128) and
+// gridDim.y >= tile_off[n_expert].
 template <int FMT>
-__device__ __forceinline__ void rein_mmq_grouped_pair(const uint8_t* __restrict__ slab0, const uint8_t* __restrict__ slab1,
-                                                      unsigned bytes_per_expert, const int* __restrict__ expert_off,
-                                                      const int* __restrict__ tile_off, unsigned n_expert,
-                                                      const BlockQ8* __restrict__ xq, float* __restrict__ y0,
-                                                      float* __restrict__ y1, unsigned in_dim, unsigned out_dim)
+__device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__ slab0, const uint8_t* __restrict__ slab1,
+                                                     unsigned bytes_per_expert, const int* __restrict__ expert_off,
+                                                     const int* __restrict__ tile_off, unsigned n_expert,
+                                                     const BlockQ8* __restrict__ xq, float* __restrict__ y0,
+                                                     float* __restrict__ y1, unsigned in_dim, unsigned out_dim)
 {
-    for (unsigned z = blockIdx.z; z < 2u; z += gridDim.z)
-        rein_mmq_grouped<FMT>(z ? slab1 : slab0, bytes_per_expert, expert_off, tile_off, n_expert, xq, z ? y1 : y0,
-                              in_dim, out_dim);
+    const unsigned tile = blockIdx.y, rb = blockIdx.x;
+    if (blockDim.x != 256u || rb * 128u >= out_dim || tile >= (unsigned)tile_off[n_expert]) return;
+    unsigned lo = 0, hi = n_expert;                // largest e with tile_off[e] <= tile
+    while (hi - lo > 1) {
+        const unsigned mid = (lo + hi) >> 1;
+        if ((unsigned)tile_off[mid] <= tile) lo = mid; else hi = mid;
+    }
+    const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
+    const unsigned tok_end = (unsigned)expert_off[lo + 1];
+    if (tok_base >= tok_end) return;
+    const uint8_t* slab = blockIdx.z ? slab1 : slab0;
+    rein_mmq_pipelined_tile<FMT, 32>(slab + (size_t)lo * bytes_per_expert, xq, blockIdx.z ? y1 : y0, in_dim, out_dim, rb,
+                                     tok_base, min(tok_end, tok_base + 32u));
 }
 
 // Two wavefronts per SIMD: a 256-register budget, which makes the compiler keep
@@ -1022,13 +1038,13 @@ __device__ __forceinline__ void rein_mmq_grouped_pair(const uint8_t* __restrict_
                               in_dim, out_dim);                                                  \
     }
 
-#define REIN_DEFINE_MMQ_GROUPED_PAIR(name, FMT)                                                  \
+#define REIN_DEFINE_MMQ_GROUPED_ONE(name, FMT)                                                   \
     extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                         \
         const unsigned char* __restrict__ slab0, const unsigned char* __restrict__ slab1,        \
         unsigned int bytes_per_expert, const int* __restrict__ expert_off,                       \
         const int* __restrict__ tile_off, unsigned int n_expert, const BlockQ8* __restrict__ xq, \
         float* __restrict__ y0, float* __restrict__ y1, unsigned int in_dim, unsigned int out_dim) \
     {                                                                                            \
-        rein_mmq_grouped_pair<FMT>(slab0, slab1, bytes_per_expert, expert_off, tile_off,         \
-                                   n_expert, xq, y0, y1, in_dim, out_dim);                       \
+        rein_mmq_grouped_one<FMT>(slab0, slab1, bytes_per_expert, expert_off, tile_off,          \
+                                  n_expert, xq, y0, y1, in_dim, out_dim);                        \
     }

@@ -5,5 +5,5 @@
 #include "mmq_gemm.h"
 
 REIN_DEFINE_MMQ_GROUPED(mmq_gemm_q4k_grouped_f32, REIN_Q4_K)
-// gate and up of an expert FFN in one launch (grid.z = 2)
-REIN_DEFINE_MMQ_GROUPED_PAIR(rein_mmq_q4k_grouped_pair, REIN_Q4_K)
+// the library's launch: one tile per workgroup; grid.z = 2 runs gate and up of an expert FFN at once
+REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q4k_grouped_t32, REIN_Q4_K)

@@ -5,10 +5,10 @@
 #include "mmq_gemm.h"
 
 REIN_DEFINE_MMQ_GROUPED(mmq_gemm_q5k_grouped_f32, REIN_Q5_K)
-// gate and up of an expert FFN in one launch (grid.z = 2)
-REIN_DEFINE_MMQ_GROUPED_PAIR(rein_mmq_q5k_grouped_pair, REIN_Q5_K)
+// the library's launch: one tile per workgroup; grid.z = 2 runs gate and up of an expert FFN at once
+REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q5k_grouped_t32, REIN_Q5_K)
 
 // Q5_1 experts: the reference compiles this file a second time with Q5_1_SCALES
 // (src/quant/q5_1.rs:58-60, qwen35.rs:3045) and looks up the same symbol in that module.
 REIN_DEFINE_MMQ_GROUPED(mmq_gemm_q5_1_grouped_f32, REIN_Q5_1)
-REIN_DEFINE_MMQ_GROUPED_PAIR(rein_mmq_q5_1_grouped_pair, REIN_Q5_1)
+REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q5_1_grouped_t32, REIN_Q5_1)
