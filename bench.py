@@ -383,6 +383,55 @@ def extras_decode_stream(stream):
     return res
 
 
+def extras_decode_ffn(stream):
+    """The FFN half of a dense decoder layer at batch 1 with the fused producers in place
+    (hidden 5120, FFN 17408, Q4_K): add_rmsnorm_q8 -> gate+up matvec -> swiglu_q8 -> down matvec,
+    four launches, against the six-launch chain without the fusion (norm, quantize, matvec,
+    swiglu, quantize, matvec).  Eight layers with their own weights in one hipGraph, so every
+    matvec streams from HBM."""
+    n_layers, hidden, ffn = 8, 5120, 17408
+    wgu = tiled_weights(rein.Q4_K, hidden, 2 * ffn, seed=1)
+    wdn = tiled_weights(rein.Q4_K, ffn, hidden, seed=2)
+    gu_w = [hip.DeviceBuf.from_host(wgu) for _ in range(n_layers)]
+    dn_w = [hip.DeviceBuf.from_host(wdn) for _ in range(n_layers)]
+    rng = np.random.default_rng(3)
+    dev = hip.DeviceBuf.from_host
+    h = dev(rng.standard_normal(hidden).astype(np.float32))
+    attn = dev((rng.standard_normal(hidden) * 0.1).astype(np.float32))
+    wn = dev(np.ones(hidden, np.float32))
+    yn, q1 = hip.DeviceBuf(hidden * 4), hip.DeviceBuf(hidden // 32 * 40)
+    gu = hip.DeviceBuf(2 * ffn * 4)
+    up = gu.ptr + ffn * 4                               # the up half of the fused gate+up output
+    act, q2 = hip.DeviceBuf(ffn * 4), hip.DeviceBuf(ffn // 32 * 40)
+    out = hip.DeviceBuf(hidden * 4)
+
+    def fused():
+        for layer in range(n_layers):
+            runtime.add_rmsnorm_q8(h, attn, wn, None, q1, hidden, 1, 1e-6, stream)
+            runtime.matvec_xq8(rein.Q4_K, gu_w[layer], q1, gu, hidden, 2 * ffn, stream)
+            runtime.swiglu_q8(gu, up, None, q2, ffn, stream)
+            runtime.matvec_xq8(rein.Q4_K, dn_w[layer], q2, out, ffn, hidden, stream)
+
+    def chain():
+        for layer in range(n_layers):
+            runtime.add_rmsnorm_q8(h, attn, wn, yn, q1, hidden, 1, 1e-6, stream)     # stands in for the fp32-only norm
+            runtime.quantize_q8(yn, q1, hidden, 1, stream)
+            runtime.matvec_xq8(rein.Q4_K, gu_w[layer], q1, gu, hidden, 2 * ffn, stream)
+            runtime.swiglu_mul(gu, up, act, ffn, stream)
+            runtime.quantize_q8(act, q2, ffn, 1, stream)
+            runtime.matvec_xq8(rein.Q4_K, dn_w[layer], q2, out, ffn, hidden, stream)
+
+    t_fused = time_graph(stream, fused, n_layers, steps=5)
+    t_chain = time_graph(stream, chain, n_layers, steps=5)
+    nbytes = wgu.nbytes + wdn.nbytes
+    res = {"workload": "dense decoder FFN half-layer, batch 1, hidden 5120, FFN 17408, Q4_K, 8 layers per hipGraph",
+           "us_per_layer_fused_4_launches": round(t_fused * 1e6, 2), "us_per_layer_unfused_6_launches": round(t_chain * 1e6, 2),
+           "weight_bytes_per_layer": nbytes, "GBs_fused": round(nbytes / t_fused / 1e9, 0),
+           "frac_hbm_peak_fused": round(nbytes / t_fused / 1e9 / HBM_PEAK_GBS, 4)}
+    log("decode ffn", res)
+    return res
+
+
 def extras_fused(stream):
     """The producers in front of the matvecs: fused (one launch writes the BlockQ8 blocks) against the
     two-launch chain they replace, at the decode shapes (hidden 5120, FFN 17408) and the MoE
@@ -549,7 +598,8 @@ def main():
     if args.extras:
         out["extras"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
                          "decode_stream_configs4": extras_decode_stream(stream), "fused_producers": extras_fused(stream),
-                         "moe_decode": extras_moe_decode(stream), "other_matvec_sites": extras_ondisk(stream)}
+                         "moe_decode": extras_moe_decode(stream), "other_matvec_sites": extras_ondisk(stream),
+                         "decode_ffn_chain": extras_decode_ffn(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)
