@@ -142,12 +142,19 @@ constexpr unsigned kCUs = 256;    // MI355X
 // flight.  Measured on MI355X (Q4_K, batch 1): 4 rows win once that still leaves
 // ~32 waves per CU (N = 34816), 2 rows down to ~8 waves per CU (N = 5120), 1 row
 // below that.
-unsigned pick_rows_per_wave(unsigned out_dim, unsigned batch)
+unsigned pick_rows_per_wave(int fmt, unsigned out_dim, unsigned batch)
 {
     const unsigned forced = env_u("REIN_MV_ROWS", 0);
     unsigned r = 1;
     if ((out_dim + 3) / 4 >= kCUs * 32) r = 4;
     else if ((out_dim + 1) / 2 >= kCUs * 8) r = 2;
+    // Per-format corrections, measured at 5120 -> 34816, 5120 -> 5120 and 17408 -> 5120: the
+    // formats with the most work per sub-block run out of issue slots before bandwidth, and
+    // there fewer rows per wave (more waves) or more rows (fewer activation reads) can win.
+    if (fmt == REIN_TYPE_Q8_0 && r == 4 && batch <= 2) r = 2;        // 34.9 -> 32.3 us (b1), 43.1 -> 37.0 (b2)
+    if (fmt == REIN_TYPE_Q6_K && r == 4 && batch == 2) r = 2;        // 48.1 -> 38.6 us
+    if (fmt == REIN_TYPE_Q6_K && r == 2 && batch == 4) r = 1;        // 15.8 -> 14.0, 42.7 -> 39.4 us
+    if (fmt == REIN_TYPE_Q5_K && r == 2 && batch == 4) r = 4;        // 13.9 -> 12.9, 39.2 -> 32.1 us
     if (forced == 1 || forced == 2 || forced == 4) r = forced;
     while (r > 1 && r * batch > 16) r >>= 1;
     return r;
@@ -203,13 +210,12 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
 // skinny MMQ.  v_dot4 is a quarter-rate instruction on this part, so every extra row
 // costs the dot4 kernels ~7 us at 5120 -> 34816 (Q4_K: 21 / 28 / 39 us at 1 / 2 / 3-4
 // rows) while the skinny MMQ takes 27 / 30 / 33 us for up to 2 / 4 / 8 rows.  Two rows
-// stay on dot4 (level at large N, faster at small N) except for Q8_0 at large N;
-// Q6_K (two MFMAs and the most aux words per sub-block) switches at 5.
-unsigned skinny_from_rows(int fmt, unsigned out_dim)
+// stay on dot4 (level at large N, faster at small N); Q6_K (two MFMAs and the most aux
+// words per sub-block) switches at 5.
+unsigned skinny_from_rows(int fmt)
 {
     unsigned dflt = 3;
     if (fmt == REIN_TYPE_Q6_K) dflt = 5;
-    if (fmt == REIN_TYPE_Q8_0 && out_dim >= 16384) dflt = 2;
     return env_u("REIN_SKINNY_FROM", dflt);
 }
 
@@ -223,9 +229,9 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
-    if (n_rows >= skinny_from_rows(fmt, out_dim) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
-    const unsigned r = pick_rows_per_wave(out_dim, b);
+    const unsigned r = pick_rows_per_wave(fmt, out_dim, b);
     const unsigned wpb = 4;
     const unsigned groups = (out_dim + r - 1) / r;
     const unsigned grid = (groups + wpb - 1) / wpb;
@@ -517,7 +523,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt, out_dim) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // Token tile.  The 64-token tile does about 6 % more work per cycle when the
     // machine is evenly loaded (the weight unpack is shared by two MFMA tiles), but two
     // of its workgroups fit a CU against three of the 32-token tile (registers), so the
