@@ -207,16 +207,37 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
 }
 
 // Activation rows from which the batched decode leaves the dot4 kernels for the
-// skinny MMQ.  v_dot4 is a quarter-rate instruction on this part, so every extra row
-// costs the dot4 kernels ~7 us at 5120 -> 34816 (Q4_K: 21 / 28 / 39 us at 1 / 2 / 3-4
+// skinny MMQ.  Every extra row is eight more v_dot4 and one more fp32 term per sub-block
+// and lane, which costs the dot4 kernels ~7 us at 5120 -> 34816 (Q4_K: 21 / 28 / 39 us at 1 / 2 / 3-4
 // rows) while the skinny MMQ takes 27 / 30 / 33 us for up to 2 / 4 / 8 rows.  Two rows
-// stay on dot4 (level at large N, faster at small N); Q6_K (two MFMAs and the most aux
-// words per sub-block) switches at 5.
+// stay on dot4 (level at large N, faster at small N).  Q6_K would switch at 5 (two MFMAs and
+// the most aux words per sub-block), but use_quad sends its 3+ rows elsewhere first.
 unsigned skinny_from_rows(int fmt)
 {
     unsigned dflt = 3;
     if (fmt == REIN_TYPE_Q6_K) dflt = 5;
     return env_u("REIN_SKINNY_FROM", dflt);
+}
+
+// Whether a batched decode of n_rows (<= 8) activation rows runs on the 4x4x4 int8 matrix
+// instruction (rein_mvq_*: four weight rows x four activation rows per instruction chain,
+// every weight sub-block unpacked once).  From measurements at 5120 -> 34816, 5120 -> 5120
+// and 17408 -> 5120 against the dot4 kernels and the skinny MMQ:
+//   Q6_K    3..8 rows everywhere   (34816 rows: 58 -> 41 us at 3-4 rows, 64 -> 57 at 5-8)
+//   Q5_K    3..4 rows everywhere   (44 -> 38 us, 12.7 -> 10.2, 30.0 -> 27.9)
+//   IQ4_XS  3..4 rows everywhere   (13.2 -> 9.7 us, 32.1 -> 25.6), 5..8 rows below 16384 output rows
+// The formats with a cheap unpack (Q4_K, Q4_0, Q8_0, IQ3_S) stay on dot4 / skinny MMQ.
+bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
+{
+    const unsigned forced = env_u("REIN_QUAD_FROM", 0);
+    if (forced) return n_rows >= forced;
+    if (n_rows < 3) return false;
+    switch (fmt) {
+    case REIN_TYPE_Q6_K:   return true;
+    case REIN_TYPE_Q5_K:   return n_rows <= 4;
+    case REIN_TYPE_IQ4_XS: return n_rows <= 4 || out_dim < 16384;
+    default:               return false;
+    }
 }
 
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
@@ -228,6 +249,12 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    if (use_quad(fmt, out_dim, n_rows)) {
+        // four output rows per wavefront, four wavefronts per workgroup
+        const std::string name = std::string("rein_mvq_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
+        void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+        return launch(name, ((out_dim + 3) / 4 + 3) / 4, 1, 1, 256, 0, s, args);
+    }
     // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
     if (n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);

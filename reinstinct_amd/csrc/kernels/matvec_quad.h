@@ -1,0 +1,227 @@
+// Batched decode matvec on the small int8 matrix instruction: 3 to 8 activation rows for
+// the formats whose weight unpack is expensive (Q6_K, Q5_K, IQ4_XS).
+//
+// On the dot4 matvec every activation row costs eight v_dot4_i32_i8 per weight sub-block
+// and lane, and the weight unpack is repeated per output row.  v_mfma_i32_4x4x4_16b_i8
+// multiplies, in each of the 16 four-lane blocks of a wavefront, a 4x4 int8 matrix A
+// (lane j of the block supplies row j: four consecutive k) with a 4x4 matrix B (lane j
+// supplies column j) in 8 cycles (measured), so the dots of four weight rows with four
+// activation rows cost what one row pair costs on dot4, and every (row, sub-block) is
+// unpacked exactly once.  What remains per output is the fp32 scaling, as in every
+// formulation of this path.  Mapping:
+//
+//   block  b = lane / 4   -> sub-block b (+16 per trip) of the contraction
+//   lane   j = lane % 4   -> weight row 4g + j  (A side)  and  activation row 4t + j  (B side)
+//
+// so lane (b, j) works on exactly one (row, sub-block) of the weights -- 16 bytes of the
+// nibble plane plus its scale words, through the same Fmt<FMT>::load / unpack as the dot4
+// kernels -- and one BlockQ8 of one activation row.  Eight chained instructions walk the
+// 32 k of the sub-block; D register r of lane j then holds the int32 dot of weight row r
+// with activation row j.  The scales of the four rows are spread over the block with DPP
+// quad broadcasts, the fp32 term is the format's own (Fmt<FMT>::term), partial sums over
+// sub-blocks stay in registers and are reduced across the 16 blocks at the end.
+//
+// The integer offsets of Q6_K (-32) and Q4_0 (-8) are folded into the weight bytes, which
+// gives the same integers as the dot4 kernels' "dot - offset * sum of activation quants".
+//
+// A wavefront owns four output rows and NT groups of four activation rows; weights are read
+// once per wavefront whatever NT.  Correct for any grid (grid-stride over row groups); the
+// block must be 256 threads.  No counterpart in the reference, whose
+// batched kernels are dot4 loops (kernels/matvec_*_repacked_batched.cpp); same arguments.
+#pragma once
+
+#include "rein_formats.h"
+
+typedef int rein_quad_v4i __attribute__((ext_vector_type(4)));
+
+template <int FMT> __device__ __forceinline__ int rein_fold_offset(int w)
+{
+    if constexpr (FMT == REIN_Q6_K) return rein_sub_bytes((uint32_t)w, 0x20202020u);
+    else if constexpr (FMT == REIN_Q4_0) return rein_sub_bytes((uint32_t)w, 0x08080808u);
+    else return w;
+}
+
+// value of lane R of every four-lane block, in all four lanes of the block
+template <int R> __device__ __forceinline__ float rein_quad_bcast(float v)
+{
+    return rein_dpp_f32<R * 0x55>(0.0f, v);
+}
+
+// One trip of a wavefront through LDS.  Memory wants lane l to read row l / 16, sub-block
+// l % 16 (16 lanes x 16 B contiguous per row and load); the matrix instruction wants lane
+// 4b + j to hold row j, sub-block b.  Each wavefront turns its 4 x 16 tile of 16-byte
+// entries through a private LDS image: entry e is stored at e + 4 (e / 16), which makes
+// both the row-major store and the column-major load conflict-free (a quarter-wave pass
+// of 16 lanes covers all 64 banks once).  LDS operations of one wavefront execute in
+// order, so no barrier is involved.
+template <int FMT, int NT>
+struct QuadStage {
+    static constexpr int kRawParts = (sizeof(typename Fmt<FMT>::Raw) + 15) / 16;
+    uint4 raw[kRawParts][76];
+    uint4 qs[NT][2][76];
+    uint2 hdr[NT][76];
+};
+
+template <int FMT> struct QuadRawBits {
+    static constexpr int kParts = (sizeof(typename Fmt<FMT>::Raw) + 15) / 16;
+    uint4 p[kParts];
+};
+
+template <int FMT>
+__device__ __forceinline__ QuadRawBits<FMT> rein_quad_raw_bits(const typename Fmt<FMT>::Raw& r)
+{
+    QuadRawBits<FMT> b;
+#pragma unroll
+    for (int i = 0; i < QuadRawBits<FMT>::kParts; i++) b.p[i] = make_uint4(0u, 0u, 0u, 0u);
+    __builtin_memcpy(&b, &r, sizeof(r));
+    return b;
+}
+
+struct QuadAct {
+    uint2 hdr;           // fp32 d, fp32 xsum
+    uint4 lo, hi;        // quants 0-15, 16-31
+};
+
+template <int FMT, int NT>
+__device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                      float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                      unsigned n_rows)
+{
+    using F = Fmt<FMT>;
+    using Raw = typename F::Raw;
+    constexpr bool kTwo = F::kDotParts == 2;          // Q6_K: one scale per 16 weights
+    constexpr int kParts = QuadRawBits<FMT>::kParts;
+    __shared__ QuadStage<FMT, NT> stages[4];
+    if (blockDim.x != 256u) return;                   // four wavefronts, four LDS images
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned j = lane & 3u, blk = lane >> 2;    // compute side: row / activation row j, sub-block slot blk
+    const unsigned lr = lane >> 4, ls = lane & 15u;   // memory side: row lr, sub-block slot ls
+    const unsigned put = lane + 4u * lr;              // entry 16 lr + ls
+    const unsigned get = 16u * j + blk + 4u * j;      // entry 16 j + blk
+    QuadStage<FMT, NT>& st = stages[wave];
+    const unsigned n_sub = in_dim >> 5;
+    const F fmt(w, n_sub, out_dim);
+    const unsigned n_groups = (out_dim + 3u) / 4u;
+    const XSums no_xs = {0, 0};
+
+    for (unsigned g = blockIdx.x * 4u + wave; g < n_groups; g += gridDim.x * 4u) {
+        const unsigned row = min(g * 4u + lr, out_dim - 1u);
+        float acc[NT][4];
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+
+        Raw rq;
+        QuadAct aq[NT];
+        auto fetch = [&](Raw& raw, QuadAct (&act)[NT], unsigned sb0) {
+            const unsigned sb = min(sb0 + ls, n_sub - 1u);             // loads stay unconditional
+            raw = fmt.load(row, sb);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const BlockQ8* p = xq + (size_t)min(4u * t + lr, n_rows - 1u) * n_sub + sb;
+                act[t].hdr = *reinterpret_cast<const uint2*>(p);
+                act[t].lo = make_uint4((uint32_t)p->qs[0], (uint32_t)p->qs[1], (uint32_t)p->qs[2], (uint32_t)p->qs[3]);
+                act[t].hi = make_uint4((uint32_t)p->qs[4], (uint32_t)p->qs[5], (uint32_t)p->qs[6], (uint32_t)p->qs[7]);
+            }
+        };
+        auto step = [&](const Raw& raw, const QuadAct (&act)[NT], unsigned sb0) {
+            // through LDS: what lane (lr, ls) fetched goes to lane (blk, j)
+            const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(raw);
+#pragma unroll
+            for (int i = 0; i < kParts; i++) st.raw[i][put] = bits.p[i];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                st.hdr[t][put] = act[t].hdr;
+                st.qs[t][0][put] = act[t].lo;
+                st.qs[t][1][put] = act[t].hi;
+            }
+            __builtin_amdgcn_wave_barrier();          // (no instruction: keeps the compiler from moving the reads up)
+            QuadRawBits<FMT> mine;
+#pragma unroll
+            for (int i = 0; i < kParts; i++) mine.p[i] = st.raw[i][get];
+            QuadAct ma[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                ma[t].hdr = st.hdr[t][get];
+                ma[t].lo = st.qs[t][0][get];
+                ma[t].hi = st.qs[t][1][get];
+            }
+            __builtin_amdgcn_wave_barrier();
+
+            Raw my;
+            __builtin_memcpy(&my, &mine, sizeof(my));
+            SubW sw;
+            F::unpack(my, sw);
+            const bool live = sb0 + blk < n_sub;
+            int a[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) a[k] = rein_fold_offset<FMT>(sw.w[k]);
+            // the scales of the block's four rows, in every lane of the block
+            float s0[4], s1[4];
+            s0[0] = rein_quad_bcast<0>(sw.s0); s0[1] = rein_quad_bcast<1>(sw.s0);
+            s0[2] = rein_quad_bcast<2>(sw.s0); s0[3] = rein_quad_bcast<3>(sw.s0);
+            s1[0] = rein_quad_bcast<0>(sw.s1); s1[1] = rein_quad_bcast<1>(sw.s1);
+            s1[2] = rein_quad_bcast<2>(sw.s1); s1[3] = rein_quad_bcast<3>(sw.s1);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const bool on = live && 4u * t + j < n_rows;
+                const float dx = on ? __builtin_bit_cast(float, ma[t].hdr.x) : 0.0f;
+                const float xsum = on ? __builtin_bit_cast(float, ma[t].hdr.y) : 0.0f;
+                const int q[8] = {(int)ma[t].lo.x, (int)ma[t].lo.y, (int)ma[t].lo.z, (int)ma[t].lo.w,
+                                  (int)ma[t].hi.x, (int)ma[t].hi.y, (int)ma[t].hi.z, (int)ma[t].hi.w};
+                rein_quad_v4i d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};
+#pragma unroll
+                for (int k = 0; k < 4; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
+                if (kTwo) {
+#pragma unroll
+                    for (int k = 4; k < 8; k++) d1 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d1, 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int k = 4; k < 8; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    SubW sc;
+                    sc.s0 = s0[r];
+                    sc.s1 = s1[r];
+                    acc[t][r] += F::term(sc, d0[r], d1[r], dx, xsum, no_xs);
+                }
+            }
+        };
+
+        // One trip (16 sub-blocks x 4 rows, 1 KiB of the nibble plane) per iteration; its loads
+        // are issued at the end of the trip before, and the other wavefronts of the SIMD (five
+        // fit) cover their latency.  Deeper register queues were measured and lose to the
+        // registers they cost.  Past the end the fetch repeats the last sub-blocks and is never
+        // used: no load sits under a branch.
+        fetch(rq, aq, 0u);
+        for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) {
+            step(rq, aq, sb0);
+            fetch(rq, aq, sb0 + 16u);
+        }
+
+        // sum over the 16 blocks (lane bits 2..5); lanes 0..3 (block 0) store
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float v = acc[t][r];
+                v += __shfl_xor(v, 4);
+                v += __shfl_xor(v, 8);
+                v += __shfl_xor(v, 16);
+                v += __shfl_xor(v, 32);
+                const unsigned tok = 4u * t + j, orow = g * 4u + r;
+                if (blk == 0u && tok < n_rows && orow < out_dim) y[(size_t)tok * out_dim + orow] = v;
+            }
+    }
+}
+
+// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows), n_rows <= 4 * NT
+#define REIN_DEFINE_MATVEC_QUAD(name, FMT, NT)                                                    \
+    extern "C" __global__ __launch_bounds__(256) void name(                                       \
+        const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y,    \
+        unsigned int in_dim, unsigned int out_dim, unsigned int n_rows)                           \
+    {                                                                                             \
+        rein_matvec_quad_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows);                        \
+    }

@@ -354,7 +354,7 @@ template <int FMT> struct MmqChunkD16 : MmqChunkBase<FMT, MmqChunk<FMT>> {
         for (int j = 0; j < 4; j++) {
             if constexpr (FMT == REIN_Q8_0) o[j] = (int)w[j];
             else if constexpr (FMT == REIN_Q4_0) o[j] = rein_sub_bytes((w[j] >> (4 * h)) & 0x0F0F0F0Fu, 0x08080808u);
-            else o[j] = rein_codebook4<FMT>((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
+            else o[j] = rein_codebook4<FMT>(w[j], 4 * h);
         }
         return o;
     }

@@ -74,27 +74,30 @@ __device__ __forceinline__ uint32_t rein_spread2(uint32_t h)
 #define REIN_KV_8_11  0x26190d01u
 #define REIN_KV_12_15 0x71594535u
 
-// four nibbles (one per byte, each < 16) -> four codebook int8
-__device__ __forceinline__ int rein_iq4_lut4(uint32_t n4)
-{
-    const uint32_t sel = n4 & 0x07070707u;
-    const uint32_t lo  = __builtin_amdgcn_perm(REIN_KV_4_7, REIN_KV_0_3, sel);
-    const uint32_t hi  = __builtin_amdgcn_perm(REIN_KV_12_15, REIN_KV_8_11, sel);
-    const uint32_t m   = ((n4 >> 3) & 0x01010101u) * 0xFFu;
-    return (int)((hi & m) | (lo & ~m));
-}
-
 // (x - c) per byte for bytes x in [0,127], c < 128: no borrow crosses a byte
 __device__ __forceinline__ int rein_sub_bytes(uint32_t x, uint32_t c4)
 {
     return (int)(((x | 0x80808080u) - c4) ^ 0x80808080u);
 }
 
-// four nibbles (one per byte) -> the four int8 weight values of a codebook format
-template <int FMT> __device__ __forceinline__ int rein_codebook4(uint32_t n4)
+// The four int8 weight values of a codebook format from the nibbles at bit `shift` (0 or 4)
+// of the four bytes of w.
+//   IQ4_XS: two byte permutes look the low three index bits up in either half of the
+//   codebook, a third picks per byte between the halves (selector byte i = i or 4 + i by
+//   index bit 3); no nibble is ever isolated.
+//   IQ3_S:  KVALUES_IQ3S[n] = 2n - 15 (src/quant/iq3_s.rs:161-162), computed per byte.
+template <int FMT> __device__ __forceinline__ int rein_codebook4(uint32_t w, unsigned shift)
 {
-    if constexpr (FMT == REIN_IQ3_S) return rein_sub_bytes(n4 << 1, 0x0F0F0F0Fu);   // KVALUES_IQ3S[n] = 2n - 15 (iq3_s.rs:161-162)
-    else return rein_iq4_lut4(n4);
+    const uint32_t v = w >> shift;
+    if constexpr (FMT == REIN_IQ3_S) {
+        return rein_sub_bytes((v << 1) & 0x1E1E1E1Eu, 0x0F0F0F0Fu);
+    } else {
+        const uint32_t sel  = v & 0x07070707u;
+        const uint32_t lo   = __builtin_amdgcn_perm(REIN_KV_4_7, REIN_KV_0_3, sel);
+        const uint32_t hi   = __builtin_amdgcn_perm(REIN_KV_12_15, REIN_KV_8_11, sel);
+        const uint32_t pick = ((v >> 1) & 0x04040404u) | 0x03020100u;
+        return (int)__builtin_amdgcn_perm(hi, lo, pick);
+    }
 }
 
 // Streaming (nontemporal) loads for the matvec weight planes: every weight byte is
@@ -388,8 +391,8 @@ template <int FMT> struct FmtCodebook16 {
         const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            s.w[j]     = rein_codebook4<FMT>(q[j] & 0x0F0F0F0Fu);
-            s.w[j + 4] = rein_codebook4<FMT>((q[j] >> 4) & 0x0F0F0F0Fu);
+            s.w[j]     = rein_codebook4<FMT>(q[j], 0);
+            s.w[j + 4] = rein_codebook4<FMT>(q[j], 4);
         }
         s.s0 = rein_h2f(r.d);
         s.s1 = 0.0f;

@@ -1,0 +1,77 @@
+"""The batched decode matvec on the 4x4x4 int8 matrix instruction (rein_mvq_*) against the
+oracle, for every dense format, every row count 1..8, output row counts that are not
+multiples of four and contractions that are not multiples of 16 sub-blocks.  The library
+picks these kernels for some formats only; REIN_QUAD_FROM forces them here."""
+import numpy as np
+import pytest
+
+import reinstinct_amd as rein
+from reinstinct_amd import hip, quant, runtime
+from reinstinct_amd._lib import init
+from oracle import orc
+from helpers import assert_close_f32, random_raw_weights
+
+pytestmark = pytest.mark.gpu
+
+DENSE = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS, rein.IQ3_S]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def gpu():
+    init()
+    hip.set_device(0)
+    yield
+    hip.synchronize()
+
+
+def dev(a):
+    return hip.DeviceBuf.from_host(np.ascontiguousarray(a))
+
+
+def run(fmt, packed, xq, in_dim, out_dim, n_rows):
+    dw, dq = dev(packed), dev(xq)
+    dy = dev(np.full(n_rows * out_dim, np.nan, np.float32))
+    if n_rows == 1:
+        runtime.matvec_xq8(fmt, dw, dq, dy, in_dim, out_dim)
+    else:
+        runtime.matvec_batched_xq8(fmt, dw, dq, dy, in_dim, out_dim, n_rows)
+    hip.synchronize()
+    return dy.to_host(np.float32).reshape(n_rows, out_dim)
+
+
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (256, 64), (5120, 130), (4096, 33)])
+def test_quad_matvec_parity(fmt, in_dim, out_dim, monkeypatch):
+    monkeypatch.setenv("REIN_QUAD_FROM", "1")
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + in_dim)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in range(1, 9):
+        print("quad", fmt, in_dim, out_dim, n_rows, flush=True)
+        x = np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32)
+        xq = orc.quantize_q8(x)
+        want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
+        assert_close_f32(run(fmt, packed, xq, in_dim, out_dim, n_rows), want, what=f"quad fmt {fmt} rows {n_rows}")
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])       # 32-weight blocks: any multiple of 32
+@pytest.mark.parametrize("in_dim", [32, 96, 352, 544, 1056])
+def test_quad_matvec_ragged_contraction(fmt, in_dim, monkeypatch):
+    monkeypatch.setenv("REIN_QUAD_FROM", "1")
+    out_dim = 37
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=in_dim)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in (1, 4, 7):
+        xq = orc.quantize_q8(np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32))
+        want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
+        assert_close_f32(run(fmt, packed, xq, in_dim, out_dim, n_rows), want, what=f"quad ragged {in_dim}")
+
+
+@pytest.mark.parametrize("fmt,n_rows", [(rein.Q6_K, 3), (rein.Q6_K, 8), (rein.Q5_K, 4), (rein.IQ4_XS, 3), (rein.IQ4_XS, 6)])
+def test_default_dispatch_at_benchmark_width(fmt, n_rows):
+    # the row counts the library sends to these kernels by itself, at the K of the decode shapes
+    in_dim, out_dim = 5120, 1100
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
+    want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
+    assert_close_f32(run(fmt, packed, xq, in_dim, out_dim, n_rows), want, what="default dispatch")
