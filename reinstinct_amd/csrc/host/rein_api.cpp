@@ -221,12 +221,16 @@ unsigned skinny_from_rows(int fmt)
 
 // Whether a batched decode of n_rows (<= 8) activation rows runs on the 4x4x4 int8 matrix
 // instruction (rein_mvq_*: four weight rows x four activation rows per instruction chain,
-// every weight sub-block unpacked once).  From measurements at 5120 -> 34816, 5120 -> 5120
-// and 17408 -> 5120 against the dot4 kernels and the skinny MMQ:
-//   Q6_K    3..8 rows everywhere   (34816 rows: 58 -> 41 us at 3-4 rows, 64 -> 57 at 5-8)
-//   Q5_K    3..4 rows everywhere   (44 -> 38 us, 12.7 -> 10.2, 30.0 -> 27.9)
-//   IQ4_XS  3..4 rows everywhere   (13.2 -> 9.7 us, 32.1 -> 25.6), 5..8 rows below 16384 output rows
-// The formats with a cheap unpack (Q4_K, Q4_0, Q8_0, IQ3_S) stay on dot4 / skinny MMQ.
+// every weight sub-block unpacked once).  From one run of all three kernel families at
+// 5120 -> 34816, 5120 -> 5120 and 17408 -> 5120 (us, best of dot4 / skinny MMQ -> this):
+//   Q6_K    3..8 rows everywhere           3-4 rows: 58.3 -> 40.5, 13.8 -> 13.2, 38.7 -> 37.5
+//                                          5-8 rows: 63.6 -> 58.2, 18.2 -> 15.5, 44.5 -> 43.0
+//   Q5_K    3..4 rows everywhere           43.6 -> 37.4, 12.6 -> 10.1, 29.8 -> 27.8
+//           5..8 rows below 16384 rows     13.2 -> 12.0, 31.8 -> 31.7 (34816 rows: 46.7 vs 50.8, stays)
+//   IQ4_XS  3..4 rows everywhere           34.1 -> 31.1, 13.1 -> 10.1, 31.9 -> 25.7
+//           5..8 rows below 16384 rows     13.3 -> 12.4, 32.4 -> 32.3 (34816 rows: 35.3 vs 45.6, stays)
+// The formats with a cheap unpack (Q4_K, Q4_0, Q8_0, IQ3_S) stay on dot4 / skinny MMQ
+// (Q4_K 4 rows at 34816 output rows: skinny 29.6, this 34.3).
 bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
 {
     const unsigned forced = env_u("REIN_QUAD_FROM", 0);
@@ -234,7 +238,7 @@ bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
     if (n_rows < 3) return false;
     switch (fmt) {
     case REIN_TYPE_Q6_K:   return true;
-    case REIN_TYPE_Q5_K:   return n_rows <= 4;
+    case REIN_TYPE_Q5_K:
     case REIN_TYPE_IQ4_XS: return n_rows <= 4 || out_dim < 16384;
     default:               return false;
     }

@@ -125,7 +125,7 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
                 act[t].hi = make_uint4((uint32_t)p->qs[4], (uint32_t)p->qs[5], (uint32_t)p->qs[6], (uint32_t)p->qs[7]);
             }
         };
-        auto step = [&](const Raw& raw, const QuadAct (&act)[NT], unsigned sb0) {
+        auto step = [&](Raw& raw, QuadAct (&act)[NT], unsigned sb0) {
             // through LDS: what lane (lr, ls) fetched goes to lane (blk, j)
             const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(raw);
 #pragma unroll
@@ -136,7 +136,15 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
                 st.qs[t][0][put] = act[t].lo;
                 st.qs[t][1][put] = act[t].hi;
             }
-            __builtin_amdgcn_wave_barrier();          // (no instruction: keeps the compiler from moving the reads up)
+            // The load registers are free again: request the next trip now, so that it is in
+            // flight while this one is read back and multiplied (past the end the fetch repeats
+            // the last sub-blocks and is never used: no load sits under a branch).  The
+            // scheduling barriers pin that order; left alone the compiler sinks the loads to
+            // where their results are needed and the kernel loses a third of its speed (measured,
+            // as were the placements behind the read-back and behind the arithmetic: both slower).
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(raw, act, sb0 + 16u);
+            __builtin_amdgcn_sched_barrier(0);
             QuadRawBits<FMT> mine;
 #pragma unroll
             for (int i = 0; i < kParts; i++) mine.p[i] = st.raw[i][get];
@@ -147,7 +155,6 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
                 ma[t].lo = st.qs[t][0][get];
                 ma[t].hi = st.qs[t][1][get];
             }
-            __builtin_amdgcn_wave_barrier();
 
             Raw my;
             __builtin_memcpy(&my, &mine, sizeof(my));
@@ -190,16 +197,12 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
             }
         };
 
-        // One trip (16 sub-blocks x 4 rows, 1 KiB of the nibble plane) per iteration; its loads
-        // are issued at the end of the trip before, and the other wavefronts of the SIMD (five
-        // fit) cover their latency.  Deeper register queues were measured and lose to the
-        // registers they cost.  Past the end the fetch repeats the last sub-blocks and is never
-        // used: no load sits under a branch.
+        // One trip (16 sub-blocks x 4 rows, 1 KiB of the nibble plane) per iteration and one
+        // trip of loads in flight per wavefront; the other wavefronts of the SIMD cover the rest
+        // of the latency.  Deeper register queues were measured and lose to the registers they
+        // cost.
         fetch(rq, aq, 0u);
-        for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) {
-            step(rq, aq, sb0);
-            fetch(rq, aq, sb0 + 16u);
-        }
+        for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) step(rq, aq, sb0);
 
         // sum over the 16 blocks (lane bits 2..5); lanes 0..3 (block 0) store
 #pragma unroll

@@ -17,3 +17,4 @@ REIN_DEFINE_MATVEC_QUAD(rein_mvq_iq4xs_t8, REIN_IQ4_XS, 2)
 REIN_DEFINE_MATVEC_QUAD(rein_mvq_iq3s_t4, REIN_IQ3_S, 1)
 REIN_DEFINE_MATVEC_QUAD(rein_mvq_iq3s_t8, REIN_IQ3_S, 2)
 
+
