@@ -303,8 +303,7 @@ template <> struct MmqChunk<REIN_Q6_K> : MmqChunkBase<REIN_Q6_K, MmqChunk<REIN_Q
         for (int j = 0; j < 4; j++) {
             // hi2 byte 2j+h holds the 2-bit fields of this half's word j
             const uint32_t hw = j < 2 ? r.h2.v[s].x : r.h2.v[s].y;
-            const uint32_t hb = (hw >> (16 * (j & 1) + 8 * h)) & 0xFFu;
-            const uint32_t q6 = ((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | rein_spread2(hb);
+            const uint32_t q6 = ((w[j] >> (4 * h)) & 0x0F0F0F0Fu) | rein_spread2(hw, 16 * (j & 1) + 8 * h);
             o[j] = rein_sub_bytes(q6, 0x20202020u);
         }
         return o;

@@ -60,12 +60,16 @@ __device__ __forceinline__ uint32_t rein_spread4(uint32_t h)
     return __umul24(h & 0xFu, 0x204081u) & 0x01010101u;
 }
 
-// four 2-bit fields of byte h -> bits 4,5 of bytes 0..3
-__device__ __forceinline__ uint32_t rein_spread2(uint32_t h)
+// The four 2-bit fields of the byte at bit `shift` of word hw -> bits 4,5 of bytes 0..3.
+// Two 24-bit multiplies place fields (0, 2) and (1, 3) -- the masks go on before the
+// multiply (so the copies cannot run into each other) and after it (to drop the copies
+// that landed elsewhere); no field is ever shifted into place on its own.
+__device__ __forceinline__ uint32_t rein_spread2(uint32_t hw, unsigned shift)
 {
-    const uint32_t even = __umul24(h & 0x33u, 0x10010u) & 0x00300030u;          // fields 0,2
-    const uint32_t odd  = __umul24((h >> 2) & 0x33u, 0x10010u) & 0x00300030u;   // fields 1,3
-    return even | (odd << 8);
+    const uint32_t h = hw >> shift;
+    const uint32_t even = __umul24(h & 0x33u, 0x10010u) & 0x00300030u;          // field 0 -> bit 4, field 2 -> bit 20
+    const uint32_t odd  = __umul24(h & 0xCCu, 0x400400u);                        // field 1 -> bit 12, field 3 -> bit 28
+    return (odd & 0x30003000u) | even;
 }
 
 // IQ4_NL / IQ4_XS codebook (src/quant/iq4_xs.rs:28-31), four entries per word.
@@ -253,10 +257,9 @@ template <> struct Fmt<REIN_Q6_K> {
             // byte g of the hi2 plane holds dot group g's four 2-bit fields;
             // group 2j -> low nibbles of word j, group 2j+1 -> high nibbles
             // (kernels/matvec_q6k_repacked.cpp:97-103)
-            const uint32_t he = ((j < 2 ? r.h2.x : r.h2.y) >> (16 * (j & 1))) & 0xFFu;
-            const uint32_t ho = ((j < 2 ? r.h2.x : r.h2.y) >> (16 * (j & 1) + 8)) & 0xFFu;
-            s.w[j]     = (int)((q[j] & 0x0F0F0F0Fu) | rein_spread2(he));
-            s.w[j + 4] = (int)(((q[j] >> 4) & 0x0F0F0F0Fu) | rein_spread2(ho));
+            const uint32_t hw = j < 2 ? r.h2.x : r.h2.y;
+            s.w[j]     = (int)((q[j] & 0x0F0F0F0Fu) | rein_spread2(hw, 16 * (j & 1)));
+            s.w[j + 4] = (int)(((q[j] >> 4) & 0x0F0F0F0Fu) | rein_spread2(hw, 16 * (j & 1) + 8));
         }
         const float d = rein_h2f(r.d);
         s.s0 = d * (float)(int)(int8_t)(r.sm & 0xFFu);
