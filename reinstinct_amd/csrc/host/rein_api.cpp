@@ -151,6 +151,7 @@ unsigned pick_rows_per_wave(int fmt, unsigned out_dim, unsigned batch)
     // Per-format corrections, measured at 5120 -> 34816, 5120 -> 5120 and 17408 -> 5120: the
     // formats with the most work per sub-block run out of issue slots before bandwidth, and
     // there fewer rows per wave (more waves) or more rows (fewer activation reads) can win.
+    if ((fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0) && batch == 1 && out_dim >= 7168) r = 4;   // 7168 rows: 7.6 -> 7.1 us, 16384: 12.4 -> 11.8
     if (fmt == REIN_TYPE_Q8_0 && r == 4 && batch <= 2) r = 2;        // 34.9 -> 32.3 us (b1), 43.1 -> 37.0 (b2)
     if (fmt == REIN_TYPE_Q6_K && r == 4 && batch == 2) r = 2;        // 48.1 -> 38.6 us
     if (fmt == REIN_TYPE_Q6_K && r == 2 && batch == 4) r = 1;        // 15.8 -> 14.0, 42.7 -> 39.4 us
