@@ -284,6 +284,11 @@ int rein_matmul(int fmt, const void *w, const float *x, float *y, unsigned in_di
                 unsigned out_dim, unsigned n_rows, void *xq_scratch, rein_stream_t s);
 /* Which path rein_matmul takes: 0 matvec, 1 batched matvec, 2 MMQ; <0 on error. */
 int rein_matmul_path(int fmt, unsigned n_rows);
+/* How rein_mmq_xq8 tiles the tokens of a P-row GEMM above 16 rows: the number of 64-token
+ * tiles per 128-row block; the remaining tokens run in 32-token tiles (0: all of them).
+ * The reference launches one fixed tile shape (prefill.rs:536-560); this choice has no
+ * counterpart there.  <0 on error. */
+int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows);
 
 /* Debug / parity: per-block int32 dots exactly as the kernels form them.
  * out [n_rows][out_dim][in_dim/32][parts], parts = rein_block_dot_parts(fmt)

@@ -12,6 +12,7 @@
 #include <algorithm>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include "../../../include/rein.h"
 #include "hip_api.h"
@@ -546,6 +547,54 @@ int rein_matvec_q8_0_splitk(const void* w, const void* xq, float* y_partials, un
     return launch("matvec_q8_0_repacked_splitk_f32", (out_dim + 1) / 2, n_split, 1, 64, 0, s, a);
 }
 
+// How many 64-token tiles per row block the MMQ launch uses (0 = the 32-token kernel).
+// A 64-token tile costs 1.68 times a 32-token tile of the 32-token kernel (one weight unpack
+// feeds two MFMA tiles); a 32-token tile inside the mixed kernel costs 1.17 (two workgroups
+// per CU there, three in its own kernel) -- ratios measured at 5120 x 17408 and 5120 x 5120.
+// Workgroups are handed to CUs in launch order, 64-token tiles first; a CU's finish time is
+// the sum of what it was handed.  The candidate with the earliest last finish wins.  Up to
+// three 32-token workgroups per CU (everything resident at once) nothing beats the fine
+// grain.  The estimate walks at most a few thousand workgroups, so it is kept per shape.
+static unsigned mmq_pick_n64(unsigned out_dim, unsigned p_rows)
+{
+    const unsigned n_rb = (out_dim + 127) / 128, t32 = (p_rows + 31) / 32;
+    const unsigned long long wg32 = (unsigned long long)n_rb * t32;
+    if (p_rows < 64 || wg32 <= 3ull * kCUs) return 0;
+    static std::mutex mu;
+    static std::unordered_map<unsigned long long, unsigned> memo;
+    const unsigned long long key = ((unsigned long long)out_dim << 32) | p_rows;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = memo.find(key);
+        if (it != memo.end()) return it->second;
+    }
+    const double c64 = 1.68, c32mix = 1.17;
+    const unsigned a_max = p_rows / 64;
+    unsigned best_n64 = a_max;                                 // very large grids: granularity no longer matters
+    if (wg32 <= 64ull * kCUs) {
+        double best = std::ceil((double)wg32 / kCUs);          // the 32-token kernel
+        best_n64 = 0;
+        std::vector<double> load(kCUs);
+        for (unsigned a = a_max > 6 ? a_max - 6 : 1; a <= a_max; a++) {
+            const unsigned long long big = (unsigned long long)n_rb * a;
+            const unsigned long long small = (unsigned long long)n_rb * ((p_rows - a * 64 + 31) / 32);
+            for (unsigned c = 0; c < kCUs; c++) load[c] = -c64 * (double)(big / kCUs + (c < big % kCUs ? 1 : 0));
+            std::make_heap(load.begin(), load.end());          // max-heap of negated loads: top = least loaded CU
+            for (unsigned long long i = 0; i < small; i++) {
+                std::pop_heap(load.begin(), load.end());
+                load.back() -= c32mix;
+                std::push_heap(load.begin(), load.end());
+            }
+            const double finish = -*std::min_element(load.begin(), load.end());
+            if (finish < best - 1e-9) { best = finish; best_n64 = a; }
+        }
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (memo.size() > 4096) memo.clear();
+    memo[key] = best_n64;
+    return best_n64;
+}
+
 int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
                  unsigned p_rows, rein_stream_t s)
 {
@@ -556,30 +605,40 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
-    // Token tile.  The 64-token tile does about 6 % more work per cycle when the
-    // machine is evenly loaded (the weight unpack is shared by two MFMA tiles), but two
-    // of its workgroups fit a CU against three of the 32-token tile (registers), so the
-    // choice goes by how full the last round of resident workgroups is.
-    unsigned tm = 32;
-    if (p_rows > 32 && fmt != REIN_TYPE_Q6_K) {
-        const double n_rb128 = (out_dim + 127) / 128;
-        const double wg32 = n_rb128 * ((p_rows + 31) / 32), wg64 = n_rb128 * ((p_rows + 63) / 64);
-        const double slots32 = kCUs * 3.0, slots64 = kCUs * 2.0;
-        const double eff32 = 1.00 * (wg32 / slots32) / std::ceil(wg32 / slots32);
-        const double eff64 = 1.06 * (wg64 / slots64) / std::ceil(wg64 / slots64);
-        if (eff64 > eff32) tm = 64;
+    // Token tiles: 32 tokens (rein_mmq_<fmt>_t32, three workgroups per CU) or the mixed launch
+    // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).
+    const unsigned n_rb = (out_dim + 127) / 128;
+    unsigned n64 = fmt == REIN_TYPE_Q6_K ? 0 : mmq_pick_n64(out_dim, p_rows);   // Q6_K: two int8 MFMAs per sub-block,
+                                                                                // the 64-token tile does not fit the register file
+    const unsigned forced_tm = env_u("REIN_MMQ_TM", 0), forced_n64 = env_u("REIN_MMQ_N64", 0xFFFFFFFFu);
+    if (fmt != REIN_TYPE_Q6_K && forced_n64 != 0xFFFFFFFFu) n64 = std::min(forced_n64, p_rows / 64);
+    if (forced_tm == 32) n64 = 0;
+    if (forced_tm == 64 && fmt != REIN_TYPE_Q6_K) {
+        const unsigned long long g = 8ull * ((n_rb + 7) / 8) * ((p_rows + 63) / 64);
+        if (g > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many tiles for one launch");
+        void* a[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
+        return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_t64", (unsigned)g, 1, 1, 256, 0, s, a);
     }
-    const unsigned forced = env_u("REIN_MMQ_TM", 0);
-    if (forced == 32 || forced == 64) tm = forced;
-    if (fmt == REIN_TYPE_Q6_K) tm = 32;          // two int8 MFMAs per sub-block: the 64-token tile does not fit the register file
-    const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + tm - 1) / tm;
-    // 1-D grid; workgroup i runs on XCD i % 8 and the kernel maps it to
-    // (row block, token tile) so that one weight block stays on one XCD
-    const unsigned long long grid = 8ull * ((n_rb + 7) / 8) * n_tt;
+    // 1-D grids; workgroup i runs on XCD i % 8 and the kernels map it to (row block, token
+    // tile) so that one weight block stays on one XCD
+    if (n64 > 0 || forced_n64 != 0xFFFFFFFFu) {
+        const unsigned n32 = (p_rows - n64 * 64 + 31) / 32;
+        const unsigned long long g = 8ull * ((n_rb + 7) / 8) * (n64 + n32);
+        if (g > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many tiles for one launch");
+        void* a[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&n64};
+        return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_mix", (unsigned)g, 1, 1, 256, 0, s, a);
+    }
+    const unsigned long long grid = 8ull * ((n_rb + 7) / 8) * ((p_rows + 31) / 32);
     if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many tiles for one launch");
-    const std::string name = std::string("rein_mmq_") + fmt_tag(fmt) + "_t" + std::to_string(tm);
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
-    return launch(name, (unsigned)grid, 1, 1, 256, 0, s, args);
+    return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_t32", (unsigned)grid, 1, 1, 256, 0, s, args);
+}
+
+int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows)
+{
+    if (!rein_block_size(fmt)) return fail(REIN_E_BAD_FORMAT, "rein_mmq_tile_plan: unknown format " + std::to_string(fmt));
+    if (out_dim == 0 || p_rows == 0) return fail(REIN_E_BAD_SHAPE, "rein_mmq_tile_plan: empty shape");
+    return fmt == REIN_TYPE_Q6_K ? 0 : (int)mmq_pick_n64(out_dim, p_rows);
 }
 
 int rein_matmul_path(int fmt, unsigned n_rows)

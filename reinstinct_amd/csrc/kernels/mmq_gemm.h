@@ -60,6 +60,32 @@ __device__ __forceinline__ rein_v16f rein_mmq_unbias(rein_v16i c)
     return __builtin_bit_cast(rein_v16f, c) - REIN_MMQ_MAGIC_F;
 }
 
+// The tuned kernels bias the int8 MFMA through its accumulator operand with the inline
+// constant 1/(2 pi) = 0x3E22F983 instead: no registers hold the bias.  Integer addition of
+// `dot` to that bit pattern stays inside the binade [1/8, 1/4) for -2292099 <= dot <=
+// 6096508 (every format's 32-element dot is below 2^20), whose ulp is 2^-26, so the result
+// read as fp32 is exactly 1/(2 pi) + dot * 2^-26 and the subtraction below returns
+// dot * 2^-26 exactly.  The activation scales are staged multiplied by 2^26
+// (rein_mmq_xstore), a power of two, so every product and sum rounds as without the trick.
+// The instruction is written as asm because the compiler does not fold a splat of that
+// constant into the operand.  The compiler cannot see that this is an MFMA, so the wait
+// states it would have placed are written out: two between a VALU write of an operand and
+// the MFMA that reads it, twelve between an 8-pass MFMA and a read of its result.
+#define REIN_MMQ_INV2PI 0.15915494f
+#define REIN_MMQ_XSCALE 67108864.0f
+// SBIAS: subtract the constant out of a scalar register (four-byte encodings) instead of a
+// literal; measured per tile shape, the 64-token tile gains 4 % from it, the 32-token tile
+// loses 1 %.
+template <bool SBIAS>
+__device__ __forceinline__ rein_v16f rein_mmq_dot_tile(rein_v4i a, rein_v4i b)
+{
+    rein_v16f r;
+    asm("s_nop 1\n\tv_mfma_i32_32x32x32_i8 %0, %1, %2, 0.15915494\n\ts_nop 11" : "=&v"(r) : "v"(a), "v"(b));
+    float c0 = REIN_MMQ_INV2PI;
+    if constexpr (SBIAS) asm("" : "+s"(c0));
+    return r - c0;
+}
+
 // bf16 bit pattern of a small non-negative integer (exact below 256)
 __device__ __forceinline__ uint32_t rein_bf16_of_u8(uint32_t v) { return __builtin_bit_cast(uint32_t, (float)v) >> 16; }
 
@@ -85,7 +111,16 @@ template <int FMT> struct MmqChunk;
 __device__ __forceinline__ unsigned rein_clamp_sb(unsigned sb, unsigned n_sub) { return sb < n_sub ? sb : n_sub - 1; }
 
 template <int FMT, class Self> struct MmqChunkBase {
+    // kSplitK: the lane halves of the tuned kernel split a sub-block's contraction as
+    // {0..7, 16..23} / {8..15, 24..31} instead of {0..15} / {16..31} (rein_mmq_act_operand
+    // reads the activations to match); operand_at() then reads only its 8 plane bytes
+    static constexpr bool kSplitK = false;
     rein_v4i b[8];
+    template <class Small>
+    static __device__ __forceinline__ rein_v4i operand_at(const uint4* e, const Small& sm, int s, unsigned h)
+    {
+        return Self::operand(*e, sm, s, h);
+    }
     template <class Raw>
     __device__ __forceinline__ void expand(const Raw& r, unsigned sb0, unsigned n_sub, unsigned h)
     {
@@ -138,6 +173,19 @@ template <> struct MmqChunk<REIN_Q4_K> : MmqChunkBase<REIN_Q4_K, MmqChunk<REIN_Q
         rein_v4i o;
 #pragma unroll
         for (int j = 0; j < 4; j++) o[j] = (int)((w[j] >> (4 * h)) & 0x0F0F0F0Fu);
+        return o;
+    }
+    // Plane byte i holds weights i (low nibble) and 16 + i (high nibble): the 8 bytes
+    // 8h..8h+7 give weights {8h..8h+7, 16+8h..16+8h+7} with two masks and two shifts + masks.
+    static constexpr bool kSplitK = true;
+    static __device__ __forceinline__ rein_v4i operand_at(const uint4* e, const Small&, int, unsigned h)
+    {
+        const uint2 q = reinterpret_cast<const uint2*>(e)[h];
+        rein_v4i o;
+        o[0] = (int)(q.x & 0x0F0F0F0Fu);
+        o[1] = (int)(q.y & 0x0F0F0F0Fu);
+        o[2] = (int)((q.x >> 4) & 0x0F0F0F0Fu);
+        o[3] = (int)((q.y >> 4) & 0x0F0F0F0Fu);
         return o;
     }
     // next sub-block pair to the front (the rolled loop of the tuned kernel only
@@ -601,8 +649,7 @@ __device__ __forceinline__ void rein_mmq_tile(const uint8_t* __restrict__ w, con
 template <int TM>
 struct MmqXRegs {
     static constexpr int kPer = TM * 8 / 256;            // activation blocks per thread per chunk
-    uint2 hdr[kPer];
-    uint4 lo[kPer], hi[kPer];
+    uint2 w[kPer][5];                                    // the block's 40 bytes as 8-byte words
 };
 
 template <int TM>
@@ -618,14 +665,14 @@ __device__ __forceinline__ void rein_mmq_xfetch(MmqXRegs<TM>& r, const BlockQ8* 
         const unsigned tok = tok_base + tl, sb = sb0 + s;
         const uint2* p = reinterpret_cast<const uint2*>(
             xq + (size_t)(tok < tok_end ? tok : tok_end - 1) * n_sub + (sb < n_sub ? sb : n_sub - 1));
-        const uint2 w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];   // 8-byte aligned words
-        r.hdr[k] = w0;
-        r.lo[k].x = w1.x; r.lo[k].y = w1.y; r.lo[k].z = w2.x; r.lo[k].w = w2.y;
-        r.hi[k].x = w3.x; r.hi[k].y = w3.y; r.hi[k].z = w4.x; r.hi[k].w = w4.y;
+#pragma unroll
+        for (int i = 0; i < 5; i++) r.w[k][i] = p[i];   // 8-byte aligned words
     }
 }
 
-// rows past tok_end / sub-blocks past n_sub get zero scales here
+// rows past tok_end / sub-blocks past n_sub get zero scales here; dx is staged times 2^26
+// (see rein_mmq_dot_tile).  Words 1..4 of a block are its quants 0..7, 8..15, 16..23, 24..31;
+// they go out in the grouping the 16-byte loads deliver, {1,2} to qs[0] and {3,4} to qs[1].
 template <int TM>
 __device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM>& r, unsigned n_sub,
                                                 unsigned tok_base, unsigned tok_end, unsigned sb0)
@@ -635,11 +682,15 @@ __device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM
         const unsigned e = threadIdx.x + k * 256;
         const unsigned tl = e >> 3, s = e & 7;
         const bool ok = tok_base + tl < tok_end && sb0 + s < n_sub;
-        l.qs[0][s][tl] = r.lo[k];
-        l.qs[1][s][tl] = r.hi[k];
-        l.dx[s][tl]    = ok ? __builtin_bit_cast(float, r.hdr[k].x) : 0.0f;
+        uint2* q0 = reinterpret_cast<uint2*>(&l.qs[0][s][tl]);
+        uint2* q1 = reinterpret_cast<uint2*>(&l.qs[1][s][tl]);
+        q0[0] = r.w[k][1];
+        q0[1] = r.w[k][2];
+        q1[0] = r.w[k][3];
+        q1[1] = r.w[k][4];
+        l.dx[s][tl]    = ok ? __builtin_bit_cast(float, r.w[k][0].x) * REIN_MMQ_XSCALE : 0.0f;
         uint16_t sp[3];
-        rein_mmq_split_xsum(ok ? __builtin_bit_cast(float, r.hdr[k].y) : 0.0f, sp);
+        rein_mmq_split_xsum(ok ? __builtin_bit_cast(float, r.w[k][0].y) : 0.0f, sp);
         l.xsb[0][tl][s] = sp[0];
         l.xsb[1][tl][s] = sp[1];
         l.xsb[2][tl][s] = sp[2];
@@ -699,6 +750,23 @@ __device__ __forceinline__ void rein_mmq_wload(MmqWLds<FMT>& dst, unsigned half,
 // s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding)
 #define REIN_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
 
+// int8 MFMA operand of token `tok`, sub-block `blk` for lane half h: quants 16h..16h+15, or
+// {8h..8h+7, 16+8h..16+8h+7} when the format splits the contraction that way (kSplitK).
+template <bool SPLITK, int TM>
+__device__ __forceinline__ rein_v4i rein_mmq_act_operand(const MmqLds<TM>& lds, unsigned h, unsigned blk, unsigned tok)
+{
+    rein_v4i a;
+    if constexpr (SPLITK) {
+        const uint2 lo = reinterpret_cast<const uint2*>(&lds.qs[0][blk][tok])[h];
+        const uint2 hi = reinterpret_cast<const uint2*>(&lds.qs[1][blk][tok])[h];
+        a[0] = (int)lo.x; a[1] = (int)lo.y; a[2] = (int)hi.x; a[3] = (int)hi.y;
+    } else {
+        const uint4 a4 = lds.qs[h][blk][tok];
+        a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
+    }
+    return a;
+}
+
 // The chunk math of the tuned kernel: one rolled iteration per sub-block pair so
 // that only one pair's tiles (two int32 dot tiles, one 2-block scale tile) are
 // live at a time.  Pairs 0,1 read ring slot 0 and pairs 2,3 slot 1; as soon as a
@@ -717,15 +785,15 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
     using C = MmqChunk<FMT>;
     constexpr int NT = TM / 32;
     constexpr int kDma = 2 * MmqWLds<FMT>::kPlanes;
-    rein_v16i cinit;
-#pragma unroll
-    for (int v = 0; v < 16; v++) cinit[v] = REIN_MMQ_MAGIC_I;
     rein_v32f z32;
 #pragma unroll
     for (int v = 0; v < 32; v++) z32[v] = 0.0f;
     const unsigned rot = j >> 1;
 
-#pragma unroll 1
+    // two pairs per trip at 32 tokens (the ring addresses of a slot become four adds and
+    // the branches on the pair's parity go); at 64 tokens that would spill
+    constexpr int kPairUnroll = (NT == 1 && !C::kTwoScales) ? 2 : 1;
+#pragma unroll kPairUnroll
     for (unsigned p = 0; p < 4; p++) {
         if (p == 2) {
             // slot 1 of this chunk: only the refill of slot 0 (if any) is younger
@@ -733,8 +801,8 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
         }
         const uint4* slot = wl.q[wsel][p >> 1];
         const unsigned s4 = 2u * (p & 1u);
-        const rein_v4i b0 = C::operand(slot[4u * j + ((s4 + rot) & 3u)], sm, 0, h);
-        const rein_v4i b1 = C::operand(slot[4u * j + ((s4 + 1u + rot) & 3u)], sm, 1, h);
+        const rein_v4i b0 = C::operand_at(&slot[4u * j + ((s4 + rot) & 3u)], sm, 0, h);
+        const rein_v4i b1 = C::operand_at(&slot[4u * j + ((s4 + 1u + rot) & 3u)], sm, 1, h);
         if (more && (p & 1u)) {
             // both pairs of the slot are in registers: refill it.  The LDS reads above
             // must have returned before the DMA may overwrite the slot.
@@ -750,16 +818,12 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
                 for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : bs[k]; bhi[k] = h ? bs[k] : 0; }
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
-                    const uint4 a4 = lds.qs[h][2 * p + s][t * 32 + j];
-                    rein_v4i a;
-                    a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
+                    const rein_v4i a = rein_mmq_act_operand<C::kSplitK>(lds, h, 2 * p + s, t * 32 + j);
                     const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
-                    const rein_v16i clo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, cinit, 0, 0, 0);
-                    const rein_v16f flo = rein_mmq_unbias(clo);
+                    const rein_v16f flo = rein_mmq_dot_tile<NT == 2>(a, blo);
 #pragma unroll
                     for (int v = 0; v < 16; v++) acc[t][v] = fmaf(flo[v], sx[v], acc[t][v]);
-                    const rein_v16i chi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, cinit, 0, 0, 0);
-                    const rein_v16f fhi = rein_mmq_unbias(chi);
+                    const rein_v16f fhi = rein_mmq_dot_tile<NT == 2>(a, bhi);
 #pragma unroll
                     for (int v = 0; v < 16; v++) acc[t][v] = fmaf(fhi[v], sx[16 + v], acc[t][v]);
                 }
@@ -767,18 +831,13 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
         } else {
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                const uint4 a40 = lds.qs[h][2 * p][t * 32 + j];
-                const uint4 a41 = lds.qs[h][2 * p + 1][t * 32 + j];
-                rein_v4i a0, a1;
-                a0[0] = (int)a40.x; a0[1] = (int)a40.y; a0[2] = (int)a40.z; a0[3] = (int)a40.w;
-                a1[0] = (int)a41.x; a1[1] = (int)a41.y; a1[2] = (int)a41.z; a1[3] = (int)a41.w;
+                const rein_v4i a0 = rein_mmq_act_operand<C::kSplitK>(lds, h, 2 * p, t * 32 + j);
+                const rein_v4i a1 = rein_mmq_act_operand<C::kSplitK>(lds, h, 2 * p + 1, t * 32 + j);
                 const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[0], z32, 0, 0, 0);
-                const rein_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0, cinit, 0, 0, 0);
-                const rein_v16f f0 = rein_mmq_unbias(c0);
+                const rein_v16f f0 = rein_mmq_dot_tile<NT == 2>(a0, b0);
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[t][v] = fmaf(f0[v], sx[v], acc[t][v]);
-                const rein_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1, cinit, 0, 0, 0);
-                const rein_v16f f1 = rein_mmq_unbias(c1);
+                const rein_v16f f1 = rein_mmq_dot_tile<NT == 2>(a1, b1);
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[t][v] = fmaf(f1[v], sx[16 + v], acc[t][v]);
             }
@@ -824,7 +883,20 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
 // One workgroup tile of the tuned kernel: 256 threads, rows 128*rb .., tokens
 // tok_base .. tok_end (at most TM) of xq / y.  Ends on a barrier, so a workgroup may
 // run several tiles in a row.
+// LDS of one tile: two activation images and the four wavefronts' weight rings.  The
+// buffer is one variable per size, so a kernel that runs tiles of both token counts
+// (LDSB = the larger size for both) holds one buffer, not two.
 template <int FMT, int TM>
+constexpr int rein_mmq_tile_lds_bytes() { return 2 * (int)sizeof(MmqLds<TM>) + 4 * (int)sizeof(MmqWLds<FMT>); }
+
+template <int BYTES>
+__device__ __forceinline__ unsigned char* rein_mmq_tile_lds()
+{
+    __shared__ __attribute__((aligned(16))) unsigned char raw[BYTES];
+    return raw;
+}
+
+template <int FMT, int TM, int LDSB = rein_mmq_tile_lds_bytes<FMT, TM>()>
 __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
                                                         float* __restrict__ y, unsigned in_dim, unsigned out_dim,
                                                         unsigned rb, unsigned tok_base, unsigned tok_end)
@@ -833,8 +905,11 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     using C = MmqChunk<FMT>;
     constexpr int NT = TM / 32;
     constexpr int kDma = 2 * MmqWLds<FMT>::kPlanes;
-    __shared__ MmqLds<TM> lds[2];
-    __shared__ MmqWLds<FMT> wlds[4];
+    static_assert(LDSB >= rein_mmq_tile_lds_bytes<FMT, TM>(), "tile LDS buffer too small");
+    static_assert(sizeof(MmqLds<TM>) % 16 == 0, "weight rings must stay 16-byte aligned");
+    unsigned char* const raw = rein_mmq_tile_lds<LDSB>();
+    MmqLds<TM>* const lds = reinterpret_cast<MmqLds<TM>*>(raw);
+    MmqWLds<FMT>* const wlds = reinterpret_cast<MmqWLds<FMT>*>(raw + 2 * sizeof(MmqLds<TM>));
 
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned j = lane & 31u, h = lane >> 5;
@@ -886,6 +961,10 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
         rein_mmq_chunk_math_rolled<FMT, TM>(lds[buf], wl, wsel, ck, cur, acc, j, h, more, [&](unsigned half) {
             if (half == 0) {
                 rein_mmq_xstore<TM>(nxt, xr, n_sub, tok_base, tok_end, sb0 + 8);
+                // The loads below land in the registers the stores above have just read.  Without
+                // the fence the compiler issues them first, into other registers, and copies them
+                // over after the stores -- a wait for the loads in the middle of the chunk.
+                __builtin_amdgcn_sched_barrier(0);
                 // past the last chunk the fetch repeats on clamped addresses and is never stored
                 rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, more2 ? sb0 + 16 : sb0 + 8);
             }
@@ -916,6 +995,37 @@ __device__ __forceinline__ void rein_mmq_pipelined(const uint8_t* __restrict__ w
     const unsigned rb = (k / n_tt) * 8u + xcd, tt = k % n_tt;
     if (rb >= n_rb) return;
     rein_mmq_pipelined_tile<FMT, TM>(w, xq, y, in_dim, out_dim, rb, tt * TM, min(p_rows, tt * TM + TM));
+}
+
+// The same with token tiles of two sizes in one launch: per row block the first n64
+// tiles take 64 tokens, the rest of the tokens goes in 32-token tiles.  The 64-token tile
+// costs less per token (one weight unpack feeds two MFMA tiles) but its coarser grain
+// leaves the last round of workgroups badly filled at a few hundred tokens; launched
+// first, with the small tiles behind them as fillers, the machine drains evenly.  The
+// host picks n64.  Workgroup -> tile keeps one weight block on one XCD, as above.
+template <int FMT>
+__device__ __forceinline__ void rein_mmq_pipelined_mixed(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                         float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                         unsigned p_rows, unsigned n64)
+{
+    constexpr int kLds = rein_mmq_tile_lds_bytes<FMT, 64>();
+    const unsigned n_rb = (out_dim + 127u) / 128u, n_rbg = (n_rb + 7u) / 8u;
+    const unsigned tok64 = min(p_rows, n64 * 64u);
+    const unsigned n32 = (p_rows - tok64 + 31u) / 32u;
+    const unsigned xcd = blockIdx.x & 7u;
+    unsigned k = blockIdx.x >> 3;
+    if (k < n_rbg * n64) {
+        const unsigned rb = (k / n64) * 8u + xcd, tt = k % n64;
+        if (rb >= n_rb || tt * 64u >= tok64) return;
+        rein_mmq_pipelined_tile<FMT, 64, kLds>(w, xq, y, in_dim, out_dim, rb, tt * 64u, min(tok64, tt * 64u + 64u));
+        return;
+    }
+    k -= n_rbg * n64;
+    if (n32 == 0u) return;
+    const unsigned rb = (k / n32) * 8u + xcd, tt = k % n32;
+    if (rb >= n_rb) return;
+    const unsigned t0 = tok64 + tt * 32u;
+    rein_mmq_pipelined_tile<FMT, 32, kLds>(w, xq, y, in_dim, out_dim, rb, t0, min(p_rows, t0 + 32u));
 }
 
 // Dense GEMM: grid-stride over (row block, token tile).
@@ -1016,6 +1126,12 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
     extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(REIN_MMQ_ARGS)                        \
     {                                                                                            \
         rein_mmq_pipelined<FMT, TM>(w, xq, y, in_dim, out_dim, p_rows);                          \
+    }
+
+#define REIN_DEFINE_MMQ_MIXED(name, FMT)                                                         \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(REIN_MMQ_ARGS, unsigned int n64) \
+    {                                                                                            \
+        rein_mmq_pipelined_mixed<FMT>(w, xq, y, in_dim, out_dim, p_rows, n64);                   \
     }
 
 #define REIN_DEFINE_MMQ_DOTS(name, FMT)                                                          \

@@ -10,4 +10,5 @@ REIN_DEFINE_MMQ(mmq_gemm_q4k_repacked_f32, REIN_Q4_K, 64)
 REIN_DEFINE_MMQ(mmq_gemm_q4k_repacked_narrow_f32, REIN_Q4_K, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_q4k_t32, REIN_Q4_K, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_q4k_t64, REIN_Q4_K, 64)
+REIN_DEFINE_MMQ_MIXED(rein_mmq_q4k_mix, REIN_Q4_K)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q4k, REIN_Q4_K)

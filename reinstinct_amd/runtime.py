@@ -88,6 +88,14 @@ def matmul_path(fmt, n_rows):
     return ("matvec", "batched_matvec", "mmq")[rc]
 
 
+def mmq_tile_plan(fmt, out_dim, p_rows):
+    """64-token tiles per 128-row block that mmq_xq8 launches for this shape (0: 32-token tiles only)"""
+    rc = lib.rein_mmq_tile_plan(fmt, out_dim, p_rows)
+    if rc < 0:
+        check(rc)
+    return rc
+
+
 def block_dots(fmt, w, xq, out, in_dim, out_dim, n_rows, via_mfma=False, stream=None):
     check(lib.rein_block_dots(fmt, _p(w), _p(xq), _p(out), in_dim, out_dim, n_rows, int(via_mfma), _s(stream)))
 

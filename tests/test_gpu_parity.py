@@ -285,6 +285,30 @@ def test_mmq_odd_sub_block_count(fmt):
                          dy.to_host(np.float32).reshape(p_rows, out_dim), p_rows, x)
 
 
+# The mixed launch (64-token tiles first, 32-token tiles behind them): every split of the
+# tokens, including a ragged last tile of either size and a split that leaves no small tile.
+@pytest.mark.parametrize("fmt", [f for f in ALL if f != rein.Q6_K])
+@pytest.mark.parametrize("p_rows,n64", [(200, 1), (200, 3), (128, 2), (100, 0), (91, 1)])
+def test_mmq_mixed_tiles_parity(fmt, p_rows, n64, monkeypatch):
+    in_dim, out_dim = 1024, 300
+    raw, packed = make_weights(fmt, in_dim, out_dim, seed=0x3131 + fmt)
+    x = Lcg(0x0BADCAFE + p_rows).acts(p_rows * in_dim).reshape(p_rows, in_dim)
+    dq = gpu_quantize(x)
+    dw = dev(packed)
+    monkeypatch.setenv("REIN_MMQ_TM", "32")
+    d32 = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    runtime.mmq_xq8(fmt, dw, dq, d32, in_dim, out_dim, p_rows)
+    monkeypatch.delenv("REIN_MMQ_TM")
+    monkeypatch.setenv("REIN_MMQ_N64", str(n64))
+    dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    runtime.mmq_xq8(fmt, dw, dq, dy, in_dim, out_dim, p_rows)
+    hip.synchronize()
+    y = dy.to_host(np.float32).reshape(p_rows, out_dim)
+    check_matvec_outputs(fmt, raw, packed, dq.to_host(np.uint8), in_dim, out_dim, y, p_rows, x)
+    # both tile sizes add the same terms in the same order
+    assert np.array_equal(y, d32.to_host(np.float32).reshape(p_rows, out_dim))
+
+
 @pytest.mark.parametrize("fmt", ALL)
 def test_mmq_reference_symbols_and_geometry(fmt):
     in_dim, out_dim = 512, 150
