@@ -112,8 +112,8 @@ __device__ __forceinline__ unsigned rein_clamp_sb(unsigned sb, unsigned n_sub) {
 
 template <int FMT, class Self> struct MmqChunkBase {
     // kSplitK: the lane halves of the tuned kernel split a sub-block's contraction as
-    // {0..7, 16..23} / {8..15, 24..31} instead of {0..15} / {16..31} (rein_mmq_act_operand
-    // reads the activations to match); operand_at() then reads only its 8 plane bytes
+    // {0..7, 16..23} / {8..15, 24..31} instead of {0..15} / {16..31} (rein_mmq_xstore stages
+    // the activations to match); operand_at() then reads only its 8 plane bytes
     static constexpr bool kSplitK = false;
     rein_v4i b[8];
     template <class Small>
@@ -646,10 +646,13 @@ __device__ __forceinline__ void rein_mmq_tile(const uint8_t* __restrict__ w, con
 //     over the 8 XCDs, each with its own L2), so a weight block is pulled from
 //     HBM once and re-read from that L2.
 // Grid: 8 * ceil(n_row_blocks / 8) * n_token_tiles workgroups of 256 threads.
+struct __attribute__((packed, aligned(8))) ReinQ8Words { uint32_t v[4]; };   // 16 bytes at 8-byte alignment
+
 template <int TM>
 struct MmqXRegs {
     static constexpr int kPer = TM * 8 / 256;            // activation blocks per thread per chunk
-    uint2 w[kPer][5];                                    // the block's 40 bytes as 8-byte words
+    uint2 hdr[kPer];                                     // d, xsum
+    rein_v4i lo[kPer], hi[kPer];                         // quants 0..15, 16..31: the two 16-byte loads
 };
 
 template <int TM>
@@ -663,18 +666,24 @@ __device__ __forceinline__ void rein_mmq_xfetch(MmqXRegs<TM>& r, const BlockQ8* 
         const unsigned e = threadIdx.x + k * 256;
         const unsigned tl = e >> 3, s = e & 7;
         const unsigned tok = tok_base + tl, sb = sb0 + s;
-        const uint2* p = reinterpret_cast<const uint2*>(
+        const char* p = reinterpret_cast<const char*>(
             xq + (size_t)(tok < tok_end ? tok : tok_end - 1) * n_sub + (sb < n_sub ? sb : n_sub - 1));
+        const ReinQ8Words lo = *reinterpret_cast<const ReinQ8Words*>(p + 8), hi = *reinterpret_cast<const ReinQ8Words*>(p + 24);
 #pragma unroll
-        for (int i = 0; i < 5; i++) r.w[k][i] = p[i];   // 8-byte aligned words
+        for (int i = 0; i < 4; i++) { r.lo[k][i] = (int)lo.v[i]; r.hi[k][i] = (int)hi.v[i]; }
+        // keeps the header out of the two 16-byte loads above (merged with it they would be
+        // cut at offsets 0 / 16 / 32 and the quads would have to be reassembled)
+        asm volatile("" ::: "memory");
+        r.hdr[k] = *reinterpret_cast<const uint2*>(p);
     }
 }
 
 // rows past tok_end / sub-blocks past n_sub get zero scales here; dx is staged times 2^26
-// (see rein_mmq_dot_tile).  Words 1..4 of a block are its quants 0..7, 8..15, 16..23, 24..31;
-// they go out in the grouping the 16-byte loads deliver, {1,2} to qs[0] and {3,4} to qs[1].
-template <int TM>
-__device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM>& r, unsigned n_sub,
+// (see rein_mmq_dot_tile).  Lane half 0 / 1 of the math reads quants 0..15 / 16..31, or
+// {0..7, 16..23} / {8..15, 24..31} when the format splits the contraction that way
+// (MmqChunkBase::kSplitK).
+template <int TM, bool SPLITK>
+__device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, MmqXRegs<TM>& r, unsigned n_sub,
                                                 unsigned tok_base, unsigned tok_end, unsigned sb0)
 {
 #pragma unroll
@@ -682,15 +691,21 @@ __device__ __forceinline__ void rein_mmq_xstore(MmqLds<TM>& l, const MmqXRegs<TM
         const unsigned e = threadIdx.x + k * 256;
         const unsigned tl = e >> 3, s = e & 7;
         const bool ok = tok_base + tl < tok_end && sb0 + s < n_sub;
-        uint2* q0 = reinterpret_cast<uint2*>(&l.qs[0][s][tl]);
-        uint2* q1 = reinterpret_cast<uint2*>(&l.qs[1][s][tl]);
-        q0[0] = r.w[k][1];
-        q0[1] = r.w[k][2];
-        q1[0] = r.w[k][3];
-        q1[1] = r.w[k][4];
-        l.dx[s][tl]    = ok ? __builtin_bit_cast(float, r.w[k][0].x) * REIN_MMQ_XSCALE : 0.0f;
+        if constexpr (SPLITK) {
+            // Pin the two quads as loaded: the regrouping then happens here, on values that
+            // arrived a chunk ago, and the next fetch lands in these registers directly.
+            // Left to itself the compiler keeps the store grouping across the loop and
+            // regroups right behind the loads, which waits for them in mid-chunk.
+            asm volatile("" : "+v"(r.lo[k]), "+v"(r.hi[k]));
+            l.qs[0][s][tl] = make_uint4((unsigned)r.lo[k][0], (unsigned)r.lo[k][1], (unsigned)r.hi[k][0], (unsigned)r.hi[k][1]);
+            l.qs[1][s][tl] = make_uint4((unsigned)r.lo[k][2], (unsigned)r.lo[k][3], (unsigned)r.hi[k][2], (unsigned)r.hi[k][3]);
+        } else {
+            l.qs[0][s][tl] = __builtin_bit_cast(uint4, r.lo[k]);
+            l.qs[1][s][tl] = __builtin_bit_cast(uint4, r.hi[k]);
+        }
+        l.dx[s][tl]    = ok ? __builtin_bit_cast(float, r.hdr[k].x) * REIN_MMQ_XSCALE : 0.0f;
         uint16_t sp[3];
-        rein_mmq_split_xsum(ok ? __builtin_bit_cast(float, r.w[k][0].y) : 0.0f, sp);
+        rein_mmq_split_xsum(ok ? __builtin_bit_cast(float, r.hdr[k].y) : 0.0f, sp);
         l.xsb[0][tl][s] = sp[0];
         l.xsb[1][tl][s] = sp[1];
         l.xsb[2][tl][s] = sp[2];
@@ -722,27 +737,64 @@ __device__ __forceinline__ void rein_lds_dma16(const void* gptr, unsigned lds_ba
                  : "memory", "m0");
 }
 
-// HBM -> LDS, asynchronous (counted by vmcnt), sub-blocks sb_first .. sb_first+3 of
-// rows row_base .. row_base+31 into slot `half`.  Lane l of load k covers row
-// 16k + l/4 (four lanes walk the row's 64 contiguous bytes).  2 * kPlanes loads.
-template <int FMT>
-__device__ __forceinline__ void rein_mmq_wload(MmqWLds<FMT>& dst, unsigned half, const Fmt<FMT>& fmt,
-                                               unsigned row_base, unsigned out_dim, unsigned sb_first, unsigned n_sub,
-                                               unsigned lane)
+// The same with the address as scalar base + 32-bit lane offset: the per-transfer address
+// arithmetic of the tuned kernel then runs on the scalar unit.
+__device__ __forceinline__ void rein_lds_dma16_s(unsigned voff, const void* sbase, unsigned lds_base)
 {
-    typedef __attribute__((address_space(3))) void* lptr_t;
-#pragma unroll
-    for (int pl = 0; pl < MmqWLds<FMT>::kPlanes; pl++) {
-        const uint4* plane = MmqChunk<FMT>::plane(fmt, (unsigned)pl);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+// Where a wavefront's ring transfers come from and go to.  row_off[k]: byte offset of lane
+// l's row in transfer k (row 16k + l/4 of the wavefront's 32, clamped to the matrix)
+// relative to the wavefront's first row; s4: which of the half chunk's four sub-blocks the
+// lane fetches (four lanes walk a row's 64 contiguous bytes; the rotation by row / 2 is the
+// ring's bank swizzle); lds: LDS address of the wavefront's ring.  K-quant rows hold whole
+// chunks, so the lane offset is constant and only the scalar base moves; the 32-weight
+// formats clamp the sub-block to the row (ragged last chunk).
+template <int FMT>
+struct MmqWSrc {
+    static constexpr bool kRagged = !(FMT == REIN_Q4_K || FMT == REIN_Q5_K || FMT == REIN_Q6_K);
+    unsigned row_off[2], s4[2], lds;
+    size_t wave_off;                               // byte offset of the wavefront's first row in a plane
+    __device__ __forceinline__ void init(const MmqWLds<FMT>& ring, const Fmt<FMT>& fmt, unsigned row_base, unsigned out_dim,
+                                         unsigned lane)
+    {
+        typedef __attribute__((address_space(3))) const void* lptr_t;
+        lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)&ring);
+        // a wavefront whose rows all lie past the matrix reads the last row (and stores nothing)
+        const unsigned first = min(row_base, out_dim - 1u);
+        wave_off = (size_t)first * fmt.nsp * 16u;
 #pragma unroll
         for (int k = 0; k < 2; k++) {
             const unsigned n = 16u * k + (lane >> 2);
-            const unsigned s4 = ((lane & 3u) - (n >> 1)) & 3u;
-            const unsigned row = min(row_base + n, out_dim - 1u);
-            const unsigned sb = rein_clamp_sb(sb_first + s4, n_sub);
-            const unsigned lds_base =
-                __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)&dst.q[pl][half][64 * k]);
-            rein_lds_dma16(plane + (size_t)row * fmt.nsp + sb, lds_base);
+            s4[k] = ((lane & 3u) - (n >> 1)) & 3u;
+            const unsigned nrow = min(row_base + n, out_dim - 1u) - first;
+            row_off[k] = nrow * fmt.nsp * 16u + (kRagged ? 0u : s4[k] * 16u);
+        }
+    }
+};
+
+// HBM -> LDS, asynchronous (counted by vmcnt), sub-blocks sb_first .. sb_first+3 of
+// the wavefront's 32 rows into slot `half`.  2 * kPlanes transfers.
+template <int FMT>
+__device__ __forceinline__ void rein_mmq_wload(const MmqWSrc<FMT>& src, unsigned half, const Fmt<FMT>& fmt,
+                                               unsigned sb_first, unsigned n_sub)
+{
+#pragma unroll
+    for (int pl = 0; pl < MmqWLds<FMT>::kPlanes; pl++) {
+        const char* plane = reinterpret_cast<const char*>(MmqChunk<FMT>::plane(fmt, (unsigned)pl));
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const unsigned lds_base = src.lds + (((unsigned)pl * 2u + half) * 128u + 64u * k) * 16u;
+            if constexpr (MmqWSrc<FMT>::kRagged) {
+                const unsigned sb = rein_clamp_sb(sb_first + src.s4[k], n_sub);
+                rein_lds_dma16_s(src.row_off[k] + sb * 16u, plane + src.wave_off, lds_base);
+            } else {
+                rein_lds_dma16_s(src.row_off[k], plane + src.wave_off + (size_t)sb_first * 16u, lds_base);
+            }
         }
     }
 }
@@ -750,20 +802,14 @@ __device__ __forceinline__ void rein_mmq_wload(MmqWLds<FMT>& dst, unsigned half,
 // s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding)
 #define REIN_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
 
-// int8 MFMA operand of token `tok`, sub-block `blk` for lane half h: quants 16h..16h+15, or
-// {8h..8h+7, 16+8h..16+8h+7} when the format splits the contraction that way (kSplitK).
-template <bool SPLITK, int TM>
+// int8 MFMA operand of token `tok`, sub-block `blk` for lane half h (the 16 quants staged
+// for that half by rein_mmq_xstore)
+template <int TM>
 __device__ __forceinline__ rein_v4i rein_mmq_act_operand(const MmqLds<TM>& lds, unsigned h, unsigned blk, unsigned tok)
 {
+    const uint4 a4 = lds.qs[h][blk][tok];
     rein_v4i a;
-    if constexpr (SPLITK) {
-        const uint2 lo = reinterpret_cast<const uint2*>(&lds.qs[0][blk][tok])[h];
-        const uint2 hi = reinterpret_cast<const uint2*>(&lds.qs[1][blk][tok])[h];
-        a[0] = (int)lo.x; a[1] = (int)lo.y; a[2] = (int)hi.x; a[3] = (int)hi.y;
-    } else {
-        const uint4 a4 = lds.qs[h][blk][tok];
-        a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
-    }
+    a[0] = (int)a4.x; a[1] = (int)a4.y; a[2] = (int)a4.z; a[3] = (int)a4.w;
     return a;
 }
 
@@ -818,7 +864,7 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
                 for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : bs[k]; bhi[k] = h ? bs[k] : 0; }
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
-                    const rein_v4i a = rein_mmq_act_operand<C::kSplitK>(lds, h, 2 * p + s, t * 32 + j);
+                    const rein_v4i a = rein_mmq_act_operand(lds, h, 2 * p + s, t * 32 + j);
                     const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
                     const rein_v16f flo = rein_mmq_dot_tile<NT == 2>(a, blo);
 #pragma unroll
@@ -831,8 +877,8 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
         } else {
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                const rein_v4i a0 = rein_mmq_act_operand<C::kSplitK>(lds, h, 2 * p, t * 32 + j);
-                const rein_v4i a1 = rein_mmq_act_operand<C::kSplitK>(lds, h, 2 * p + 1, t * 32 + j);
+                const rein_v4i a0 = rein_mmq_act_operand(lds, h, 2 * p, t * 32 + j);
+                const rein_v4i a1 = rein_mmq_act_operand(lds, h, 2 * p + 1, t * 32 + j);
                 const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.sc[0], z32, 0, 0, 0);
                 const rein_v16f f0 = rein_mmq_dot_tile<NT == 2>(a0, b0);
 #pragma unroll
@@ -911,7 +957,7 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     MmqLds<TM>* const lds = reinterpret_cast<MmqLds<TM>*>(raw);
     MmqWLds<FMT>* const wlds = reinterpret_cast<MmqWLds<FMT>*>(raw + 2 * sizeof(MmqLds<TM>));
 
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned j = lane & 31u, h = lane >> 5;
     const unsigned n_sub = in_dim >> 5;
     const F fmt(w, n_sub, out_dim);
@@ -920,6 +966,8 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     const unsigned rowc = row < out_dim ? row : out_dim - 1;
     const unsigned wsel = FMT == REIN_Q8_0 ? h : 0u;
     MmqWLds<FMT>& wl = wlds[wave];
+    MmqWSrc<FMT> wsrc;
+    wsrc.init(wl, fmt, row_base, out_dim, lane);
 
     rein_v16f acc[NT];
 #pragma unroll
@@ -943,10 +991,10 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     MmqXRegs<TM> xr;
     C::fetch_small(small, fmt, rowc, 0, n_sub, h);
     rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 0);
-    rein_mmq_xstore<TM>(lds[0], xr, n_sub, tok_base, tok_end, 0);
+    rein_mmq_xstore<TM, C::kSplitK>(lds[0], xr, n_sub, tok_base, tok_end, 0);
     rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 8 < n_sub ? 8 : 0);
-    rein_mmq_wload<FMT>(wl, 0, fmt, row_base, out_dim, 0, n_sub, lane);
-    rein_mmq_wload<FMT>(wl, 1, fmt, row_base, out_dim, 4, n_sub, lane);
+    rein_mmq_wload<FMT>(wsrc, 0, fmt, 0, n_sub);
+    rein_mmq_wload<FMT>(wsrc, 1, fmt, 4, n_sub);
     REIN_WAIT_VMCNT(kDma);                           // slot 0 of chunk 0 has landed
     __syncthreads();
 
@@ -960,7 +1008,7 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
         MmqLds<TM>& nxt = lds[buf ^ 1u];
         rein_mmq_chunk_math_rolled<FMT, TM>(lds[buf], wl, wsel, ck, cur, acc, j, h, more, [&](unsigned half) {
             if (half == 0) {
-                rein_mmq_xstore<TM>(nxt, xr, n_sub, tok_base, tok_end, sb0 + 8);
+                rein_mmq_xstore<TM, C::kSplitK>(nxt, xr, n_sub, tok_base, tok_end, sb0 + 8);
                 // The loads below land in the registers the stores above have just read.  Without
                 // the fence the compiler issues them first, into other registers, and copies them
                 // over after the stores -- a wait for the loads in the middle of the chunk.
@@ -968,7 +1016,7 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
                 // past the last chunk the fetch repeats on clamped addresses and is never stored
                 rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, more2 ? sb0 + 16 : sb0 + 8);
             }
-            rein_mmq_wload<FMT>(wl, half, fmt, row_base, out_dim, sb0 + 8 + 4 * half, n_sub, lane);
+            rein_mmq_wload<FMT>(wsrc, half, fmt, sb0 + 8 + 4 * half, n_sub);
         });
         if (more) REIN_WAIT_VMCNT(kDma);             // slot 0 of the next chunk has landed
         __syncthreads();
