@@ -608,12 +608,11 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     // Token tiles: 32 tokens (rein_mmq_<fmt>_t32, three workgroups per CU) or the mixed launch
     // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).
     const unsigned n_rb = (out_dim + 127) / 128;
-    unsigned n64 = fmt == REIN_TYPE_Q6_K ? 0 : mmq_pick_n64(out_dim, p_rows);   // Q6_K: two int8 MFMAs per sub-block,
-                                                                                // the 64-token tile does not fit the register file
+    unsigned n64 = mmq_pick_n64(out_dim, p_rows);
     const unsigned forced_tm = env_u("REIN_MMQ_TM", 0), forced_n64 = env_u("REIN_MMQ_N64", 0xFFFFFFFFu);
-    if (fmt != REIN_TYPE_Q6_K && forced_n64 != 0xFFFFFFFFu) n64 = std::min(forced_n64, p_rows / 64);
+    if (forced_n64 != 0xFFFFFFFFu) n64 = std::min(forced_n64, p_rows / 64);
     if (forced_tm == 32) n64 = 0;
-    if (forced_tm == 64 && fmt != REIN_TYPE_Q6_K) {
+    if (forced_tm == 64) {
         const unsigned long long g = 8ull * ((n_rb + 7) / 8) * ((p_rows + 63) / 64);
         if (g > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many tiles for one launch");
         void* a[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
@@ -638,7 +637,7 @@ int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows)
 {
     if (!rein_block_size(fmt)) return fail(REIN_E_BAD_FORMAT, "rein_mmq_tile_plan: unknown format " + std::to_string(fmt));
     if (out_dim == 0 || p_rows == 0) return fail(REIN_E_BAD_SHAPE, "rein_mmq_tile_plan: empty shape");
-    return fmt == REIN_TYPE_Q6_K ? 0 : (int)mmq_pick_n64(out_dim, p_rows);
+    return (int)mmq_pick_n64(out_dim, p_rows);
 }
 
 int rein_matmul_path(int fmt, unsigned n_rows)

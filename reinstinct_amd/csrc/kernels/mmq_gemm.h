@@ -121,6 +121,12 @@ template <int FMT, class Self> struct MmqChunkBase {
     {
         return Self::operand(*e, sm, s, h);
     }
+    // what the tuned kernel needs of prepare(); the same unless a format says otherwise
+    template <class Small>
+    __device__ __forceinline__ void prepare_tuned(const Small& r, unsigned sb0, unsigned n_sub, unsigned h)
+    {
+        static_cast<Self*>(this)->prepare(r, sb0, n_sub, h);
+    }
     template <class Raw>
     __device__ __forceinline__ void expand(const Raw& r, unsigned sb0, unsigned n_sub, unsigned h)
     {
@@ -356,10 +362,40 @@ template <> struct MmqChunk<REIN_Q6_K> : MmqChunkBase<REIN_Q6_K, MmqChunk<REIN_Q
         }
         return o;
     }
+    // Tuned kernel.  The lane halves split a sub-block as {0..7, 16..23} / {8..15, 24..31}:
+    // operand registers 0,1 then belong to the first 16-weight scale group and 2,3 to the
+    // second in BOTH halves, so the two groups' dots come from two MFMAs whose other
+    // registers are constant zeros (no per-lane masking).  The int8 group scales combine the
+    // two int32 dots exactly (|dot| <= 16*32*127, |sum| < 2^24), which leaves one fp32 scale
+    // per sub-block, d * dx, as in the one-scale formats.  dq = d * 2^-26 undoes the factor
+    // the activation scales are staged with.  hi2 dword h holds this half's 2-bit fields:
+    // byte 0 -> weights 8h.., byte 2 -> 8h+4.., byte 1 -> 16+8h.., byte 3 -> 20+8h...
+    static constexpr bool kSplitK = true;
+    float dq;
+    __device__ __forceinline__ void prepare_tuned(const Small& r, unsigned, unsigned, unsigned)
+    {
+        dq = rein_h2f(r.d) * (1.0f / REIN_MMQ_XSCALE);
+    }
+    static __device__ __forceinline__ rein_v4i operand_at(const uint4* e, const Small& r, int s, unsigned h)
+    {
+        const uint2 q = reinterpret_cast<const uint2*>(e)[h];
+        const uint32_t hw = h ? r.h2.v[s].y : r.h2.v[s].x;
+        rein_v4i o;
+        o[0] = rein_sub_bytes((q.x & 0x0F0F0F0Fu) | rein_spread2(hw, 0), 0x20202020u);
+        o[1] = rein_sub_bytes((q.y & 0x0F0F0F0Fu) | rein_spread2(hw, 16), 0x20202020u);
+        o[2] = rein_sub_bytes(((q.x >> 4) & 0x0F0F0F0Fu) | rein_spread2(hw, 8), 0x20202020u);
+        o[3] = rein_sub_bytes(((q.y >> 4) & 0x0F0F0F0Fu) | rein_spread2(hw, 24), 0x20202020u);
+        return o;
+    }
+    // the int8 scales of sub-block s (0 or 1 after rotation) for the two groups
+    static __device__ __forceinline__ int group_scale(const Small& r, int s, int g)
+    {
+        return (int)(int8_t)(g ? (r.sm.v[s] >> 8) : (r.sm.v[s] & 0xFFu));
+    }
     __device__ __forceinline__ void rotate(Small& r)
     {
 #pragma unroll
-        for (int i = 0; i < 6; i++) { sc[i] = sc[i + 2]; r.h2.v[i] = r.h2.v[i + 2]; }
+        for (int i = 0; i < 6; i++) { sc[i] = sc[i + 2]; r.h2.v[i] = r.h2.v[i + 2]; r.sm.v[i] = r.sm.v[i + 2]; }
     }
 };
 
@@ -835,6 +871,17 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
 #pragma unroll
     for (int v = 0; v < 32; v++) z32[v] = 0.0f;
     const unsigned rot = j >> 1;
+    rein_v4i zlo[2], zhi[2];
+    if constexpr (C::kTwoScales) {
+        // opaque zeros: otherwise the compiler rebuilds the half-zero operands from
+        // constants for every MFMA
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            zlo[s] = rein_v4i{0, 0, 0, 0};
+            zhi[s] = rein_v4i{0, 0, 0, 0};
+            asm volatile("" : "+v"(zlo[s]), "+v"(zhi[s]));
+        }
+    }
 
     // two pairs per trip at 32 tokens (the ring addresses of a slot become four adds and
     // the branches on the pair's parity go); at 64 tokens that would spill
@@ -856,22 +903,27 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
             refill(p >> 1);
         }
         if constexpr (C::kTwoScales) {
+            rein_v16i zi;
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                const rein_v4i bs = s ? b1 : b0;
-                rein_v4i blo, bhi;
+            for (int v = 0; v < 16; v++) zi[v] = 0;
 #pragma unroll
-                for (int k = 0; k < 4; k++) { blo[k] = h ? 0 : bs[k]; bhi[k] = h ? bs[k] : 0; }
+            for (int t = 0; t < NT; t++) {
+                const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + h][t * 32 + j], ck.dq, z32, 0, 0, 0);
 #pragma unroll
-                for (int t = 0; t < NT; t++) {
+                for (int s = 0; s < 2; s++) {
+                    const rein_v4i bs = s ? b1 : b0;
+                    // the zero halves of the two operands live in the same registers all along
+                    zlo[s][0] = bs[0]; zlo[s][1] = bs[1];
+                    zhi[s][2] = bs[2]; zhi[s][3] = bs[3];
                     const rein_v4i a = rein_mmq_act_operand(lds, h, 2 * p + s, t * 32 + j);
-                    const rein_v32f sx = __builtin_amdgcn_mfma_f32_32x32x1f32(lds.dx[2 * p + s][t * 32 + j], ck.sc[s], z32, 0, 0, 0);
-                    const rein_v16f flo = rein_mmq_dot_tile<NT == 2>(a, blo);
+                    const rein_v16i ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, zlo[s], zi, 0, 0, 0);
+                    const rein_v16i ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, zhi[s], zi, 0, 0, 0);
+                    const int sl = C::group_scale(sm, s, 0), sh = C::group_scale(sm, s, 1);
 #pragma unroll
-                    for (int v = 0; v < 16; v++) acc[t][v] = fmaf(flo[v], sx[v], acc[t][v]);
-                    const rein_v16f fhi = rein_mmq_dot_tile<NT == 2>(a, bhi);
-#pragma unroll
-                    for (int v = 0; v < 16; v++) acc[t][v] = fmaf(fhi[v], sx[16 + v], acc[t][v]);
+                    for (int v = 0; v < 16; v++) {
+                        const int both = __mul24(ilo[v], sl) + __mul24(ihi[v], sh);
+                        acc[t][v] = fmaf((float)both, sx[16 * s + v], acc[t][v]);
+                    }
                 }
             }
         } else {
@@ -1001,7 +1053,7 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     unsigned buf = 0;
     for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 8, buf ^= 1u) {
         C ck;
-        ck.prepare(small, sb0, n_sub, h);
+        ck.prepare_tuned(small, sb0, n_sub, h);
         const typename C::Small cur = small;
         const bool more = sb0 + 8 < n_sub, more2 = sb0 + 16 < n_sub;
         if (more) C::fetch_small(small, fmt, rowc, sb0 + 8, n_sub, h);

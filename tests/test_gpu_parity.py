@@ -287,7 +287,7 @@ def test_mmq_odd_sub_block_count(fmt):
 
 # The mixed launch (64-token tiles first, 32-token tiles behind them): every split of the
 # tokens, including a ragged last tile of either size and a split that leaves no small tile.
-@pytest.mark.parametrize("fmt", [f for f in ALL if f != rein.Q6_K])
+@pytest.mark.parametrize("fmt", ALL)
 @pytest.mark.parametrize("p_rows,n64", [(200, 1), (200, 3), (128, 2), (100, 0), (91, 1)])
 def test_mmq_mixed_tiles_parity(fmt, p_rows, n64, monkeypatch):
     in_dim, out_dim = 1024, 300
