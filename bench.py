@@ -205,6 +205,13 @@ def time_graph(stream, launch_all, n_launches, steps=5):
     return e0.elapsed_ms(e1) * 1e-3 / (steps * n_launches)
 
 
+def mmq_kernel_name(fmt, out_dim, p_rows):
+    """the kernel mmq_xq8 launches for this shape (64-token tiles per row block, the rest in 32-token tiles)"""
+    n64 = runtime.mmq_tile_plan(fmt, out_dim, p_rows)
+    tag = {rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k"}.get(fmt, FMT_NAME[fmt])
+    return f"rein_mmq_{tag}_mix (n64 = {n64})" if n64 else f"rein_mmq_{tag}_t32"
+
+
 def extras_mmq(stream):
     """BASELINE configs[2]: B in {Q4_K, Q6_K, Q8_0} x M in {128, 512, 2048}, 5120 x 17408"""
     out = []
@@ -577,7 +584,8 @@ def main():
         out["mmq"] = {"workload": "Q4_K MMQ prefill GEMM 512x5120x17408 (BASELINE configs[2])",
                       "us_per_launch": round(sec * 1e6, 2), "value": round(tops, 2), "unit": "int8 TOPS",
                       "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                                   "frac": round(tops / INT8_PEAK_TOPS, 4)}}
+                                   "frac": round(tops / INT8_PEAK_TOPS, 4),
+                                   "kernel": mmq_kernel_name(rein.Q4_K, 17408, 512)}}
         del mm
 
     if args.sweep:
