@@ -83,7 +83,11 @@ __device__ __forceinline__ rein_v16f rein_mmq_dot_tile(rein_v4i a, rein_v4i b)
     asm("s_nop 1\n\tv_mfma_i32_32x32x32_i8 %0, %1, %2, 0.15915494\n\ts_nop 11" : "=&v"(r) : "v"(a), "v"(b));
     float c0 = REIN_MMQ_INV2PI;
     if constexpr (SBIAS) asm("" : "+s"(c0));
-    return r - c0;
+    rein_v16f f = r - c0;
+    // all sixteen subtractions (in place) before the first fma: independent fp32
+    // instructions issue faster than sixteen dependent subtract / fma pairs
+    asm("" : "+v"(f));
+    return f;
 }
 
 // bf16 bit pattern of a small non-negative integer (exact below 256)
