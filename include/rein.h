@@ -339,6 +339,22 @@ int rein_moe_down(int fmt, const void *slab, const int32_t *ids, const void *xq,
                   unsigned in_dim, unsigned out_dim, unsigned bytes_per_expert,
                   unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used, unsigned n_tok,
                   rein_stream_t s);
+/* The one-token expert FFN in two launches instead of the four of qwen35.rs:3071-3167 (no
+ * single counterpart in the reference; each is byte / bit identical to the launches it
+ * replaces).  rein_moe_gate_up_swiglu_q8: moe_gate_up_swiglu_q4k_repacked_f32 followed by
+ * quantize_q8_f32 -- xq_out[tok][slot] receives out_dim/32 BlockQ8 blocks of
+ * silu(gate . x) * (up . x); Q4_K experts, out_dim a multiple of 32.
+ * rein_moe_down_combine: moe_matvec_*_f32 (or its *_down form) followed by moe_combine_f32 --
+ * out[tok][i] = sum_j weights[tok][j] * down_exps_s[ids[tok][j]] * (W[ids[tok][j]] . xq[tok][j])[i]
+ * in slot order.  Formats Q4_K, Q5_K, Q6_K, Q8_0, Q5_1. */
+int rein_moe_gate_up_swiglu_q8(int fmt, const void *gate_slab, const void *up_slab, const int32_t *ids,
+                               const void *xq, void *xq_out, unsigned in_dim, unsigned out_dim,
+                               unsigned bytes_per_expert, unsigned xq_tok_stride, unsigned xq_slot_stride,
+                               unsigned n_used, unsigned n_tok, rein_stream_t s);
+int rein_moe_down_combine(int fmt, const void *slab, const int32_t *ids, const float *weights,
+                          const float *down_exps_s, const void *xq, float *out, unsigned in_dim,
+                          unsigned out_dim, unsigned bytes_per_expert, unsigned xq_tok_stride,
+                          unsigned xq_slot_stride, unsigned n_used, unsigned n_tok, rein_stream_t s);
 /* launch_moe_gate_up_swiglu (qwen35.rs:3141-3167; kernels/moe_gate_up_swiglu_q4k_repacked.cpp):
  * y = silu(Wgate . xq) * (Wup . xq) in one pass over both slabs.  fmt must be Q4_K. */
 int rein_moe_gate_up_swiglu(int fmt, const void *gate_slab, const void *up_slab, const int32_t *ids,

@@ -118,6 +118,8 @@ SIGNATURES = {
     "rein_moe_expert_matvec": (_i, [_i, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
     "rein_moe_down": (_i, [_i, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
     "rein_moe_gate_up_swiglu": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
+    "rein_moe_gate_up_swiglu_q8": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
+    "rein_moe_down_combine": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, _vp]),
     "rein_rmsnorm_q8": (_i, [_vp, _vp, _vp, _u, _u, C.c_float, _vp]),
     "rein_add_rmsnorm_q8": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _u, C.c_float, _vp]),
     "rein_swiglu_q8": (_i, [_vp, _vp, _vp, _vp, _u, _vp]),

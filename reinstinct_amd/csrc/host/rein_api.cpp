@@ -843,6 +843,60 @@ int rein_moe_gate_up_swiglu(int fmt, const void* gate_slab, const void* up_slab,
                          out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, s);
 }
 
+int rein_moe_gate_up_swiglu_q8(int fmt, const void* gate_slab, const void* up_slab, const int32_t* ids, const void* xq,
+                               void* xq_out, unsigned in_dim, unsigned out_dim, unsigned bytes_per_expert,
+                               unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used, unsigned n_tok,
+                               rein_stream_t s)
+{
+    const char* who = "rein_moe_gate_up_swiglu_q8";
+    if (fmt != REIN_TYPE_Q4_K) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": the fused form exists for Q4_K experts");
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_tok)) return rc;
+    if (out_dim % 32 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": out_dim must be a multiple of 32 (whole BlockQ8 blocks)");
+    if (n_used == 0 || n_used > 65535 || n_tok > 65535)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_used and n_tok must be in 1..65535");
+    if (bytes_per_expert < rein_repacked_len(fmt, in_dim, out_dim))
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert is smaller than one repacked expert");
+    if (bytes_per_expert % 16 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert must be a multiple of 16");
+    if (int rc = check_ptr(who, gate_slab, 16, "gate_slab")) return rc;
+    if (int rc = check_ptr(who, up_slab, 16, "up_slab")) return rc;
+    if (int rc = check_ptr(who, ids, 4, "ids")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, xq_out, 8, "xq_out")) return rc;
+    void* a[] = {(void*)&gate_slab, (void*)&up_slab, (void*)&ids, (void*)&xq, (void*)&xq_out, (void*)&in_dim, (void*)&out_dim,
+                 (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
+    return launch("rein_moe_gate_up_swiglu_q8_q4k", out_dim / 32, n_used, n_tok, 1024, 0, s, a);
+}
+
+int rein_moe_down_combine(int fmt, const void* slab, const int32_t* ids, const float* weights, const float* down_exps_s,
+                          const void* xq, float* out, unsigned in_dim, unsigned out_dim, unsigned bytes_per_expert,
+                          unsigned xq_tok_stride, unsigned xq_slot_stride, unsigned n_used, unsigned n_tok, rein_stream_t s)
+{
+    const char* who = "rein_moe_down_combine";
+    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0, Q5_1");
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_tok)) return rc;
+    if (n_used == 0 || n_used > 65535 || n_tok > 65535)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_used and n_tok must be in 1..65535");
+    if (bytes_per_expert < rein_repacked_len(fmt, in_dim, out_dim))
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert is smaller than one repacked expert");
+    if (bytes_per_expert % 16 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert must be a multiple of 16");
+    if (int rc = check_ptr(who, slab, 16, "slab")) return rc;
+    if (int rc = check_ptr(who, ids, 4, "ids")) return rc;
+    if (int rc = check_ptr(who, weights, 4, "weights")) return rc;
+    if (int rc = check_ptr(who, down_exps_s, 4, "down_exps_s")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, out, 4, "out")) return rc;
+    // a workgroup owns two rows, one team per slot: half-wavefront teams for contractions of at most
+    // 32 sub-blocks, whole wavefronts otherwise; as many teams as slots, up to 512 threads
+    const bool half = in_dim / 32 <= 32;
+    const unsigned lanes = half ? 32 : 64;
+    unsigned threads = ((n_used * lanes + 63) / 64) * 64;
+    if (threads > 512) threads = 512;
+    void* a[] = {(void*)&slab, (void*)&ids, (void*)&weights, (void*)&down_exps_s, (void*)&xq, (void*)&out, (void*)&in_dim,
+                 (void*)&out_dim, (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
+    return launch(std::string("rein_moe_down_combine_") + fmt_tag(fmt) + (half ? "_h" : ""),
+                  (out_dim + 1) / 2, 1, n_tok, threads, 0, s, a);
+}
+
 int rein_swiglu_mul(const float* gate, const float* up, float* out, unsigned n, rein_stream_t s)
 {
     if (n == 0) return fail(REIN_E_BAD_SHAPE, "rein_swiglu_mul: n is zero");

@@ -21,6 +21,73 @@
 #include "rein_formats.h"
 #include "q8_block.h"
 
+// Dot products of rows row0 .. row0+R-1 of one expert (w0; GATE_UP: also w1) with the
+// BlockQ8 row xqs, for a team of LANES lanes (lane = index in the team).  s0 / s1 are valid
+// in every lane of the team.  Rows past rmax are clamped (the caller stores nothing for them).
+template <int FMT, int R, int LANES, bool GATE_UP>
+__device__ __forceinline__ void rein_moe_row_sums(const Fmt<FMT>& w0, const Fmt<FMT>& w1, const BlockQ8* __restrict__ xqs,
+                                                  unsigned n_sub, unsigned row0, unsigned rmax, unsigned lane,
+                                                  float (&s0)[R], float (&s1)[R])
+{
+    using F = Fmt<FMT>;
+    float a0[R], a1[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) { a0[r] = 0.0f; a1[r] = 0.0f; }
+
+    for (unsigned sb0 = 0; sb0 < n_sub; sb0 += LANES) {
+        const bool live = sb0 + lane < n_sub;
+        const unsigned sb = live ? sb0 + lane : n_sub - 1;
+        typename F::Raw raw0[R], raw1[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            raw0[r] = w0.load(min(row0 + r, rmax), sb);
+            if (GATE_UP) raw1[r] = w1.load(min(row0 + r, rmax), sb);
+        }
+        const BlockQ8* p = xqs + sb;
+        const float dx = live ? p->d : 0.0f, xsum = live ? p->xsum : 0.0f;
+        int q[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) q[j] = p->qs[j];
+        XSums xs;
+        if (F::kNeedsXSums) xs = rein_xsums(q);
+        else { xs.lo = 0; xs.hi = 0; }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            SubW sw;
+            F::unpack(raw0[r], sw);
+            int i0 = 0, i1 = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) { i0 = rein_dot4(sw.w[j], q[j], i0); i1 = rein_dot4(sw.w[j + 4], q[j + 4], i1); }
+            a0[r] += F::term(sw, i0, i1, dx, xsum, xs);
+            if (GATE_UP) {
+                F::unpack(raw1[r], sw);
+                i0 = 0; i1 = 0;
+#pragma unroll
+                for (int j = 0; j < 4; j++) { i0 = rein_dot4(sw.w[j], q[j], i0); i1 = rein_dot4(sw.w[j + 4], q[j + 4], i1); }
+                a1[r] += F::term(sw, i0, i1, dx, xsum, xs);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        s1[r] = 0.0f;
+        if (LANES == 64) {
+            s0[r] = rein_wave_sum(a0[r]);
+            if (GATE_UP) s1[r] = rein_wave_sum(a1[r]);
+        } else {
+            // row sums of the four 16-lane rows; a half owns rows {0,1} or {2,3}
+            const float t = rein_row16_sum(a0[r]);
+            const int b = __builtin_bit_cast(int, t);
+            const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) +
+                             __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+            const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) +
+                             __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+            s0[r] = (threadIdx.x & 32u) ? hi : lo;
+        }
+    }
+}
+
 template <int FMT, int R, int LANES, bool GATE_UP>
 __device__ __forceinline__ void rein_moe_matvec(const uint8_t* __restrict__ slab0, const uint8_t* __restrict__ slab1,
                                                 const int* __restrict__ ids, const BlockQ8* __restrict__ xq,
@@ -49,63 +116,102 @@ __device__ __forceinline__ void rein_moe_matvec(const uint8_t* __restrict__ slab
     const unsigned wave_team0 = blockIdx.x * teams_per_block + (threadIdx.x >> 6) * (64 / LANES);
     for (unsigned g = team0, gw = wave_team0; gw < n_groups; g += gridDim.x * teams_per_block, gw += gridDim.x * teams_per_block) {
         const unsigned row0 = g * R;
-        float a0[R], a1[R];
+        float s0[R], s1[R];
+        rein_moe_row_sums<FMT, R, LANES, GATE_UP>(w0, w1, xqs, n_sub, row0, rmax, lane, s0, s1);
 #pragma unroll
-        for (int r = 0; r < R; r++) { a0[r] = 0.0f; a1[r] = 0.0f; }
+        for (int r = 0; r < R; r++)
+            if (lane == 0 && row0 + r < out_dim) yo[row0 + r] = GATE_UP ? rein_silu_det(s0[r]) * s1[r] : s0[r];
+    }
+}
 
-        for (unsigned sb0 = 0; sb0 < n_sub; sb0 += LANES) {
-            const bool live = sb0 + lane < n_sub;
-            const unsigned sb = live ? sb0 + lane : n_sub - 1;
-            typename F::Raw raw0[R], raw1[R];
+// gate + up + SwiGLU + quantize_q8 in one launch: xq_out[tok][slot][blk] is the BlockQ8 block
+// of outputs 32 blk .. 32 blk + 31 of silu(gate . x) * (up . x) -- byte for byte what
+// moe_gate_up_swiglu_*_f32 followed by quantize_q8_f32 writes (same per-row sums, same silu,
+// same block quantizer).  One workgroup of 1024 threads per block of 32 outputs: wavefront w
+// computes rows 2w, 2w + 1 (the mapping of the two-launch form), the 32 values meet in LDS and
+// one 16-lane row quantizes them.  grid = (out_dim / 32, n_used, n_tok); out_dim % 32 == 0.
+template <int FMT>
+__device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
+                                                           const int* __restrict__ ids, const BlockQ8* __restrict__ xq,
+                                                           BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
+                                                           unsigned bytes_per_expert, unsigned xq_tok_stride,
+                                                           unsigned xq_slot_stride, unsigned n_used)
+{
+    using F = Fmt<FMT>;
+    __shared__ float vals[32];
+    if (blockDim.x != 1024u) return;
+    const unsigned tok = blockIdx.z, slot = blockIdx.y, blk = blockIdx.x;
+    const unsigned n_blk = out_dim >> 5;
+    if (blk >= n_blk) return;
+    const unsigned eid = (unsigned)ids[(size_t)tok * n_used + slot];
+    const BlockQ8* xqs = xq + (size_t)tok * xq_tok_stride + (size_t)slot * xq_slot_stride;
+    const unsigned n_sub = in_dim >> 5;
+    const F w0(gate_slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
+    const F w1(up_slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned row0 = blk * 32u + wave * 2u;
+    float s0[2], s1[2];
+    rein_moe_row_sums<FMT, 2, 64, true>(w0, w1, xqs, n_sub, row0, out_dim - 1u, lane, s0, s1);
+    if (lane < 2u) vals[wave * 2u + lane] = lane ? rein_silu_det(s0[1]) * s1[1] : rein_silu_det(s0[0]) * s1[0];
+    __syncthreads();
+    if (threadIdx.x < 16u)
+        rein_q8_store_sub(xq_out + ((size_t)tok * n_used + slot) * n_blk + blk, threadIdx.x, vals[threadIdx.x], vals[threadIdx.x + 16u]);
+}
+
+// down projection + weighted combine in one launch:
+//   out[tok][i] = sum_j (weights[tok][j] * down_exps_s[ids[tok][j]]) * (W[ids[tok][j]] . xq[tok][j])[i]
+// in slot order j = 0 .. n_used-1, a multiply and an add per slot (no fma): bit for bit what
+// moe_matvec_*_f32 followed by moe_combine_f32 writes.  A workgroup owns R rows; its teams of
+// LANES lanes take one slot each (all slots of a row group are in flight at once, as in the
+// two-launch form), the per-slot results meet in LDS and thread r sums row r in slot order.
+// grid = (row groups, 1, n_tok); any grid.x is correct; block a multiple of 64, at most 512.
+template <int FMT, int R, int LANES>
+__device__ __forceinline__ void rein_moe_down_combine(const uint8_t* __restrict__ slab, const int* __restrict__ ids,
+                                                      const float* __restrict__ weights, const float* __restrict__ down_exps_s,
+                                                      const BlockQ8* __restrict__ xq, float* __restrict__ out, unsigned in_dim,
+                                                      unsigned out_dim, unsigned bytes_per_expert, unsigned xq_tok_stride,
+                                                      unsigned xq_slot_stride, unsigned n_used)
+{
+#pragma clang fp contract(off)
+    using F = Fmt<FMT>;
+    constexpr unsigned kMaxTeams = 512 / LANES;
+    __shared__ float vals[kMaxTeams][R];
+    const unsigned n_teams = blockDim.x / LANES;
+    if (n_teams == 0u || n_teams > kMaxTeams || (blockDim.x & 63u)) return;
+    const unsigned tok = blockIdx.z;
+    ids     += (size_t)tok * n_used;
+    weights += (size_t)tok * n_used;
+    out     += (size_t)tok * out_dim;
+    const unsigned n_sub = in_dim >> 5;
+    const unsigned lane = threadIdx.x & (LANES - 1u), team = threadIdx.x / LANES;
+    const unsigned n_groups = (out_dim + R - 1) / R;
+    const unsigned rmax = out_dim - 1;
+    for (unsigned g = blockIdx.x; g < n_groups; g += gridDim.x) {
+        const unsigned row0 = g * R;
+        float acc = 0.0f;                                        // thread r < R: row row0 + r
+        for (unsigned j0 = 0; j0 < n_used; j0 += n_teams) {
+            // a team past the last slot repeats the last slot and stores nothing
+            const unsigned j = min(j0 + team, n_used - 1u);
+            const unsigned eid = (unsigned)ids[j];
+            const F w(slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
+            const BlockQ8* xqs = xq + (size_t)tok * xq_tok_stride + (size_t)j * xq_slot_stride;
+            float s0[R], s1[R];
+            rein_moe_row_sums<FMT, R, LANES, false>(w, w, xqs, n_sub, row0, rmax, lane, s0, s1);
+            if (lane == 0u && j0 + team < n_used) {
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                raw0[r] = w0.load(min(row0 + r, rmax), sb);
-                if (GATE_UP) raw1[r] = w1.load(min(row0 + r, rmax), sb);
+                for (int r = 0; r < R; r++) vals[team][r] = s0[r];
             }
-            const BlockQ8* p = xqs + sb;
-            const float dx = live ? p->d : 0.0f, xsum = live ? p->xsum : 0.0f;
-            int q[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) q[j] = p->qs[j];
-            XSums xs;
-            if (F::kNeedsXSums) xs = rein_xsums(q);
-            else { xs.lo = 0; xs.hi = 0; }
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                SubW sw;
-                F::unpack(raw0[r], sw);
-                int i0 = 0, i1 = 0;
-#pragma unroll
-                for (int j = 0; j < 4; j++) { i0 = rein_dot4(sw.w[j], q[j], i0); i1 = rein_dot4(sw.w[j + 4], q[j + 4], i1); }
-                a0[r] += F::term(sw, i0, i1, dx, xsum, xs);
-                if (GATE_UP) {
-                    F::unpack(raw1[r], sw);
-                    i0 = 0; i1 = 0;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) { i0 = rein_dot4(sw.w[j], q[j], i0); i1 = rein_dot4(sw.w[j + 4], q[j + 4], i1); }
-                    a1[r] += F::term(sw, i0, i1, dx, xsum, xs);
+            __syncthreads();
+            if (threadIdx.x < (unsigned)R) {
+                const unsigned n_here = min(n_teams, n_used - j0);
+                for (unsigned t = 0; t < n_here; t++) {
+                    const float sc = weights[j0 + t] * down_exps_s[ids[j0 + t]];
+                    acc += sc * vals[t][threadIdx.x];
                 }
             }
+            __syncthreads();
         }
-
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            float s0, s1 = 0.0f;
-            if (LANES == 64) {
-                s0 = rein_wave_sum(a0[r]);
-                if (GATE_UP) s1 = rein_wave_sum(a1[r]);
-            } else {
-                // row sums of the four 16-lane rows; a half owns rows {0,1} or {2,3}
-                const float t = rein_row16_sum(a0[r]);
-                const int b = __builtin_bit_cast(int, t);
-                const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) +
-                                 __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
-                const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) +
-                                 __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
-                s0 = (threadIdx.x & 32u) ? hi : lo;
-            }
-            if (lane == 0 && row0 + r < out_dim) yo[row0 + r] = GATE_UP ? rein_silu_det(s0) * s1 : s0;
-        }
+        if (threadIdx.x < (unsigned)R && row0 + threadIdx.x < out_dim) out[row0 + threadIdx.x] = acc;
     }
 }
 
@@ -150,3 +256,40 @@ void moe_gate_up_swiglu_q4k_repacked_f32(const unsigned char* __restrict__ gate_
     rein_moe_matvec<REIN_Q4_K, 2, 64, true>(gate_slab, up_slab, ids, xq, y, in_dim, out_dim, bytes_per_expert,
                                             xq_tok_stride, xq_slot_stride, n_used);
 }
+
+// The two fused launches of the one-token expert FFN (no counterpart in the reference, which
+// runs the four-launch chain of src/runtime/qwen35.rs:3071-3167).
+#define REIN_DEFINE_MOE_GUQ8(name, FMT)                                                                   \
+    extern "C" __global__ __launch_bounds__(1024) void name(                                              \
+        const unsigned char* __restrict__ gate_slab, const unsigned char* __restrict__ up_slab,           \
+        const int* __restrict__ ids, const BlockQ8* __restrict__ xq, BlockQ8* __restrict__ xq_out,        \
+        unsigned int in_dim, unsigned int out_dim, unsigned int bytes_per_expert,                         \
+        unsigned int xq_tok_stride, unsigned int xq_slot_stride, unsigned int n_used)                     \
+    {                                                                                                     \
+        rein_moe_gate_up_swiglu_q8<FMT>(gate_slab, up_slab, ids, xq, xq_out, in_dim, out_dim,             \
+                                        bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used);         \
+    }
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k, REIN_Q4_K)
+
+#define REIN_DEFINE_MOE_DC(name, FMT, R, LANES)                                                           \
+    extern "C" __global__ __launch_bounds__(512) void name(                                               \
+        const unsigned char* __restrict__ slab, const int* __restrict__ ids, const float* __restrict__ weights, \
+        const float* __restrict__ down_exps_s, const BlockQ8* __restrict__ xq, float* __restrict__ out,   \
+        unsigned int in_dim, unsigned int out_dim, unsigned int bytes_per_expert,                         \
+        unsigned int xq_tok_stride, unsigned int xq_slot_stride, unsigned int n_used)                     \
+    {                                                                                                     \
+        rein_moe_down_combine<FMT, R, LANES>(slab, ids, weights, down_exps_s, xq, out, in_dim, out_dim,   \
+                                             bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used);    \
+    }
+// two rows per workgroup; short contractions (at most 32 sub-blocks): half-wavefront teams,
+// as the *_down symbols
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q4k_h, REIN_Q4_K, 2, 32)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5k_h, REIN_Q5_K, 2, 32)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q6k_h, REIN_Q6_K, 2, 32)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q8_0_h, REIN_Q8_0, 2, 32)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5_1_h, REIN_Q5_1, 2, 32)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q4k, REIN_Q4_K, 2, 64)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5k, REIN_Q5_K, 2, 64)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q6k, REIN_Q6_K, 2, 64)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q8_0, REIN_Q8_0, 2, 64)
+REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5_1, REIN_Q5_1, 2, 64)

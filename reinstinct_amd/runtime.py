@@ -144,6 +144,21 @@ def moe_gate_up_swiglu(fmt, gate_slab, up_slab, ids, xq, y, in_dim, out_dim, byt
                                       bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, _s(stream)))
 
 
+def moe_gate_up_swiglu_q8(fmt, gate_slab, up_slab, ids, xq, xq_out, in_dim, out_dim, bytes_per_expert, xq_tok_stride,
+                          xq_slot_stride, n_used, n_tok=1, stream=None):
+    """moe_gate_up_swiglu followed by quantize_q8 in one launch (BlockQ8 rows of the down projection's input)"""
+    check(lib.rein_moe_gate_up_swiglu_q8(fmt, _p(gate_slab), _p(up_slab), _p(ids), _p(xq), _p(xq_out), in_dim, out_dim,
+                                         bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok, _s(stream)))
+
+
+def moe_down_combine(fmt, slab, ids, weights, down_exps_s, xq, out, in_dim, out_dim, bytes_per_expert, xq_tok_stride,
+                     xq_slot_stride, n_used, n_tok=1, stream=None):
+    """moe_down followed by moe_combine in one launch"""
+    check(lib.rein_moe_down_combine(fmt, _p(slab), _p(ids), _p(weights), _p(down_exps_s), _p(xq), _p(out), in_dim,
+                                    out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used, n_tok,
+                                    _s(stream)))
+
+
 def swiglu_mul(gate, up, out, n, stream=None):
     check(lib.rein_swiglu_mul(_p(gate), _p(up), _p(out), n, _s(stream)))
 

@@ -193,3 +193,67 @@ def test_moe_decode_ffn_chain_config4_shapes():
     got = d_out.to_host(np.float32)
     assert rel_l2(got, want) < 2e-3
     assert_close_f32(got, want.reshape(-1), rel=2e-2, abs_=2e-3, what="moe decode ffn")
+
+
+# ------------------------------------------------------------------ the two fused launches
+@pytest.mark.parametrize("in_dim,out_dim,n_tok", [(2048, 768, 1), (2048, 96, 3), (256, 32, 2)])
+def test_gate_up_swiglu_q8_equals_the_two_launches(in_dim, out_dim, n_tok):
+    # gate + up + SwiGLU + quantize in one launch: byte for byte what the fused matvec
+    # followed by quantize_q8 writes, and that chain is what the oracle is compared with above
+    fmt, n_expert, n_used = rein.Q4_K, 10, 8
+    rng = np.random.default_rng(in_dim * 7 + out_dim)
+    gate, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=17)
+    up, _ = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=170)
+    ids = np.stack([rng.permutation(n_expert)[:n_used] for _ in range(n_tok)]).astype(np.int32)
+    xq = quantized_rows(rng, n_tok, 1, in_dim)
+    d_gate, d_up, d_ids, d_xq = dev(gate), dev(up), dev(ids), dev(xq)
+    d_act = dev(np.full((n_tok, n_used, out_dim), np.nan, np.float32))
+    runtime.moe_gate_up_swiglu(fmt, d_gate, d_up, d_ids, d_xq, d_act, in_dim, out_dim, bpe, in_dim // 32, 0, n_used, n_tok)
+    n_bytes = n_tok * n_used * (out_dim // 32) * 40
+    d_chain = dev(np.full(n_bytes, 0xAA, np.uint8))
+    runtime.quantize_q8(d_act, d_chain, out_dim, n_tok * n_used)
+    d_fused = dev(np.full(n_bytes, 0x55, np.uint8))
+    runtime.moe_gate_up_swiglu_q8(fmt, d_gate, d_up, d_ids, d_xq, d_fused, in_dim, out_dim, bpe, in_dim // 32, 0, n_used, n_tok)
+    hip.synchronize()
+    assert np.array_equal(d_fused.to_host(np.uint8), d_chain.to_host(np.uint8))
+    # and against the CPU chain: same quants up to the fp32 rounding of the sums in front of them
+    g = oracle_expert_matvec(fmt, gate, bpe, ids, xq, in_dim, out_dim, slot_rows=False)
+    u = oracle_expert_matvec(fmt, up, bpe, ids, xq, in_dim, out_dim, slot_rows=False)
+    want = orc.quantize_q8((orc.map_det("silu", g) * u).reshape(n_tok * n_used, out_dim)).reshape(-1, 40)
+    got = d_fused.to_host(np.uint8).reshape(-1, 40)
+    dq = np.abs(got[:, 8:].view(np.int8).astype(np.int32) - want[:, 8:].view(np.int8).astype(np.int32))
+    assert dq.max() <= 1 and np.mean(dq != 0) < 0.02
+    assert np.allclose(got[:, :4].copy().view(np.float32), want[:, :4].copy().view(np.float32), rtol=2e-3)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("in_dim,out_dim,n_tok", [(768, 2048, 1), (768, 56, 2), (256, 43, 1), (2048, 64, 1)])
+def test_down_combine_equals_the_two_launches(fmt, in_dim, out_dim, n_tok):
+    # down projection + weighted combine in one launch: bit for bit the two-launch result
+    # (both team widths: up to 32 sub-blocks half-wavefronts, 2048 the full wavefront)
+    if out_dim % 8 and fmt != rein.Q8_0:
+        out_dim += 8 - out_dim % 8          # slabs must stay 16-byte aligned
+    n_expert, n_used = 12, 8
+    rng = np.random.default_rng(in_dim * 5 + out_dim + fmt)
+    slab, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=fmt * 100 + 77)
+    if bpe % 16:
+        pytest.skip("expert slab not 16-byte aligned at this shape")
+    ids = np.stack([rng.permutation(n_expert)[:n_used] for _ in range(n_tok)]).astype(np.int32)
+    wts = rng.random((n_tok, n_used)).astype(np.float32)
+    scales = (0.5 + rng.random(n_expert)).astype(np.float32)
+    xq = quantized_rows(rng, n_tok, n_used, in_dim)
+    n_sub = in_dim // 32
+    d_slab, d_ids, d_wts, d_sc, d_xq = dev(slab), dev(ids), dev(wts), dev(scales), dev(xq)
+    d_eo = dev(np.full((n_tok, n_used, out_dim), np.nan, np.float32))
+    runtime.moe_down(fmt, d_slab, d_ids, d_xq, d_eo, in_dim, out_dim, bpe, n_used * n_sub, n_sub, n_used, n_tok)
+    d_chain = dev(np.full((n_tok, out_dim), np.nan, np.float32))
+    runtime.moe_combine(d_eo, d_ids, d_wts, d_sc, d_chain, n_tok, out_dim, n_used)
+    d_fused = dev(np.full((n_tok, out_dim), np.nan, np.float32))
+    runtime.moe_down_combine(fmt, d_slab, d_ids, d_wts, d_sc, d_xq, d_fused, in_dim, out_dim, bpe, n_used * n_sub, n_sub,
+                             n_used, n_tok)
+    hip.synchronize()
+    got = d_fused.to_host(np.float32)
+    assert np.array_equal(got.view(np.uint32), d_chain.to_host(np.float32).view(np.uint32))
+    eo = oracle_expert_matvec(fmt, slab, bpe, ids, xq, in_dim, out_dim, slot_rows=True)
+    want = orc.moe_combine(eo, ids, wts, scales)
+    assert_close_f32(got.reshape(want.shape), want, what=f"down+combine fmt {fmt}")
