@@ -313,6 +313,13 @@ int rein_moe_sort(const int32_t *ids, unsigned n_entries, unsigned n_expert, uns
 /* moe_gather_xq / moe_scatter_rows (kernels/moe_expert_sort.cpp:81-110) */
 int rein_moe_gather_xq(const void *xq_src, const int32_t *perm, void *xq_dst, unsigned nsub,
                        unsigned n_used, unsigned n_entries, rein_stream_t s);
+/* quantize_q8_f32 followed by moe_gather_xq in one launch (no single counterpart in the
+ * reference): every row of x [n_tok][in_dim] is quantized once and written to the places
+ * inv[tok * n_used + j] of its routing entries in the expert-sorted order (inv = the inverse
+ * of the sort's perm; negative = dropped entry); xq_dst [n_tok * n_used][in_dim/32] blocks.
+ * The same bytes as the two launches, without the quantized table between them. */
+int rein_moe_quantize_scatter(const float *x, const int32_t *inv, void *xq_dst, unsigned in_dim,
+                              unsigned n_used, unsigned n_tok, rein_stream_t s);
 int rein_moe_scatter_rows(const float *src, const int32_t *perm, float *dst, unsigned dim,
                           unsigned n_entries, rein_stream_t s);
 /* launch_moe_grouped_gemm (qwen35.rs:3036-3064; kernels/mmq_gemm_*_grouped.cpp):

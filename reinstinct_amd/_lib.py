@@ -89,6 +89,7 @@ SIGNATURES = {
     "rein_moe_topk": (_i, [_vp, _u, _u, _u, _vp, _vp, _vp]),
     "rein_moe_sort": (_i, [_vp, _u, _u, _u, _vp, _vp, _vp, _vp, _vp, _vp]),
     "rein_moe_gather_xq": (_i, [_vp, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_moe_quantize_scatter": (_i, [_vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_moe_scatter_rows": (_i, [_vp, _vp, _vp, _u, _u, _vp]),
     "rein_moe_grouped_gemm": (_i, [_i, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
     "rein_swiglu_mul": (_i, [_vp, _vp, _vp, _u, _vp]),

@@ -701,6 +701,15 @@ int rein_moe_topk(const float* logits, unsigned n_tok, unsigned n_expert, unsign
     return launch("moe_topk_f32", n_tok, 1, 1, 128, n_expert * 4, s, args);
 }
 
+namespace {
+// Small routing tables are sorted by one workgroup (one launch instead of four or five): the
+// 4096 entries of 512 tokens x top-8 take it ~5 us, about one launch of the split form.
+bool moe_sort_in_one_block(unsigned n_entries, unsigned n_expert)
+{
+    return n_entries <= 32768 && n_expert <= 2048 && env_u("REIN_MOE_SORT_SPLIT", 0) == 0;
+}
+}  // namespace
+
 int rein_moe_sort(const int32_t* ids, unsigned n_entries, unsigned n_expert, unsigned bn, int32_t* count,
                   int32_t* cursor, int32_t* perm, int32_t* expert_off, int32_t* tile_off, rein_stream_t s)
 {
@@ -709,6 +718,13 @@ int rein_moe_sort(const int32_t* ids, unsigned n_entries, unsigned n_expert, uns
     const void* ptrs[] = {ids, count, cursor, perm, expert_off, tile_off};
     for (const void* p : ptrs)
         if (int rc = check_ptr("rein_moe_sort", p, 4, "buffer")) return rc;
+    if (moe_sort_in_one_block(n_entries, n_expert)) {
+        // cursor is left as it is: the rank counters of the one-workgroup sort live in LDS
+        int32_t* inv = nullptr;
+        void* a[] = {(void*)&ids, (void*)&count, (void*)&expert_off, (void*)&tile_off, (void*)&perm, (void*)&inv,
+                     (void*)&n_entries, (void*)&n_expert, (void*)&bn};
+        return launch("rein_moe_sort_one_block", 1, 1, 1, 1024, 0, s, a);
+    }
     const unsigned ge = (n_expert + 255) / 256, gn = (n_entries + 255) / 256;
     {
         void* a[] = {(void*)&count, (void*)&n_expert};
@@ -740,6 +756,22 @@ int rein_moe_gather_xq(const void* xq_src, const int32_t* perm, void* xq_dst, un
     const unsigned gx = (nsub * 5 + 255) / 256, gy = n_entries < 65535 ? n_entries : 65535;
     void* a[] = {(void*)&xq_src, (void*)&perm, (void*)&xq_dst, (void*)&nsub, (void*)&n_used, (void*)&n_entries};
     return launch("moe_gather_xq", gx, gy, 1, 256, 0, s, a);
+}
+
+int rein_moe_quantize_scatter(const float* x, const int32_t* inv, void* xq_dst, unsigned in_dim, unsigned n_used,
+                              unsigned n_tok, rein_stream_t s)
+{
+    const char* who = "rein_moe_quantize_scatter";
+    if (in_dim == 0 || in_dim % 32 != 0 || n_used == 0 || n_tok == 0)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": in_dim must be a non-zero multiple of 32, the counts non-zero");
+    if (n_tok > 65535) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most 65535 tokens per call");
+    if (int rc = check_ptr(who, x, 4, "x")) return rc;
+    if (int rc = check_ptr(who, inv, 4, "inv")) return rc;
+    if (int rc = check_ptr(who, xq_dst, 8, "xq_dst")) return rc;
+    const unsigned gx = (in_dim + 511) / 512;
+    const unsigned n_entries = n_tok * n_used;
+    void* a[] = {(void*)&x, (void*)&inv, (void*)&xq_dst, (void*)&in_dim, (void*)&n_used, (void*)&n_entries};
+    return launch("rein_moe_quantize_scatter", gx, n_tok, 1, 256, 0, s, a);
 }
 
 int rein_moe_scatter_rows(const float* src, const int32_t* perm, float* dst, unsigned dim, unsigned n_entries,
@@ -997,14 +1029,17 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     const unsigned ne = sh.n_tok * sh.n_used;
 
     if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
-    if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
     // counting sort by expert (moe_expert_sort.hip), with the inverse permutation kept so
     // that the combine can read the sorted expert outputs in place
-    {
-        int32_t* count = (int32_t*)(base + w.count);
+    int32_t* count = (int32_t*)(base + w.count);
+    int32_t* inv = (int32_t*)(base + w.inv);
+    const unsigned bn = rein_moe_gemm_bn();
+    if (moe_sort_in_one_block(ne, sh.n_expert)) {
+        void* a[] = {(void*)&ids, (void*)&count, (void*)&eoff, (void*)&toff, (void*)&perm, (void*)&inv, (void*)&ne,
+                     (void*)&sh.n_expert, (void*)&bn};
+        if (int rc = launch("rein_moe_sort_one_block", 1, 1, 1, 1024, 0, s, a)) return rc;
+    } else {
         int32_t* cursor = (int32_t*)(base + w.cursor);
-        int32_t* inv = (int32_t*)(base + w.inv);
-        const unsigned bn = rein_moe_gemm_bn();
         const unsigned zn = (unsigned)((w.cursor - w.count) / 4) + sh.n_expert;     // count .. cursor are adjacent
         const unsigned gn = (ne + 255) / 256;
         void* a0[] = {(void*)&count, (void*)&zn};
@@ -1016,7 +1051,8 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
         void* a3[] = {(void*)&ids, (void*)&eoff, (void*)&cursor, (void*)&perm, (void*)&inv, (void*)&ne, (void*)&sh.n_expert};
         if (int rc = launch("rein_moe_sort_scatter_inv", gn, 1, 1, 256, 0, s, a3)) return rc;
     }
-    if (int rc = rein_moe_gather_xq(base + w.xq_in, perm, base + w.g_in, sh.hidden / 32, sh.n_used, ne, s)) return rc;
+    // the expert-sorted BlockQ8 rows straight from x (quantize_q8 + moe_gather_xq in one launch)
+    if (int rc = rein_moe_quantize_scatter(x, inv, base + w.g_in, sh.hidden, sh.n_used, sh.n_tok, s)) return rc;
     // gate and up projections in one launch (grid.z = 2)
     if (int rc = launch_grouped(sh.gate_up_fmt, gate_exps, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert, base + w.g_in,
                                 (float*)(base + w.e_gate), (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;

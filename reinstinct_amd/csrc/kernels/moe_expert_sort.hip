@@ -117,3 +117,57 @@ extern "C" __global__ void rein_moe_sort_scatter_inv(const int* __restrict__ ids
         inv[i] = pos;
     }
 }
+
+// The whole counting sort in one workgroup of 1024 threads, for routing tables small enough
+// that launches, not work, are what the four-kernel form costs (512 tokens x top-8 = 4096
+// entries): histogram and rank counters live in LDS, wavefront 0 scans, the same threads
+// scatter.  Writes count, expert_off, tile_off, perm and (if inv != nullptr) inv exactly as
+// moe_sort_zero + moe_sort_histogram + moe_sort_scan + rein_moe_sort_scatter_inv would
+// (the order inside one expert is as undetermined here as there).  n_expert <= 2048.
+#define REIN_SORT1_MAX_EXPERT 2048
+extern "C" __global__ __launch_bounds__(1024)
+void rein_moe_sort_one_block(const int* __restrict__ ids, int* __restrict__ count, int* __restrict__ expert_off,
+                             int* __restrict__ tile_off, int* __restrict__ perm, int* __restrict__ inv,
+                             unsigned int n_entries, unsigned int n_expert, unsigned int bn)
+{
+    __shared__ int cnt[REIN_SORT1_MAX_EXPERT], off[REIN_SORT1_MAX_EXPERT], cur[REIN_SORT1_MAX_EXPERT];
+    if (blockIdx.x != 0 || n_expert > REIN_SORT1_MAX_EXPERT) return;
+    for (unsigned e = threadIdx.x; e < n_expert; e += blockDim.x) { cnt[e] = 0; cur[e] = 0; }
+    __syncthreads();
+    for (unsigned i = threadIdx.x; i < n_entries; i += blockDim.x) {
+        const int e = ids[i];
+        if (e >= 0 && (unsigned)e < n_expert) atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const unsigned lane = threadIdx.x;
+        int ebase = 0, tbase = 0;
+        for (unsigned e0 = 0; e0 < n_expert; e0 += 64) {
+            const unsigned e = e0 + lane;
+            const int c = e < n_expert ? cnt[e] : 0;
+            const int t = (int)(((unsigned)c + bn - 1u) / bn);
+            const int ce = rein_wave_scan_incl(c, lane);
+            const int te = rein_wave_scan_incl(t, lane);
+            if (e < n_expert) {
+                off[e] = ebase + ce - c;
+                count[e] = c;
+                expert_off[e] = ebase + ce - c;
+                tile_off[e]   = tbase + te - t;
+            }
+            ebase += __shfl(ce, 63);
+            tbase += __shfl(te, 63);
+        }
+        if (lane == 0) {
+            expert_off[n_expert] = ebase;
+            tile_off[n_expert]   = tbase;
+        }
+    }
+    __syncthreads();
+    for (unsigned i = threadIdx.x; i < n_entries; i += blockDim.x) {
+        const int e = ids[i];
+        if (e < 0 || (unsigned)e >= n_expert) { if (inv) inv[i] = -1; continue; }
+        const int pos = off[e] + atomicAdd(&cur[e], 1);
+        perm[pos] = (int)i;
+        if (inv) inv[i] = pos;
+    }
+}

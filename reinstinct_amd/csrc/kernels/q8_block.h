@@ -53,7 +53,9 @@ __device__ __forceinline__ float rein_row_max(float lo, float hi)
 // inv = 127/amax are IEEE divisions; q = clamp(rint(v*inv), -127, 127), ties to
 // even; an all-zero block stores d = 1.  Same output as
 // kernels/quantize_q8.cpp:37-53 of the reference up to its use of v_rcp_f32 for inv.
-__device__ __forceinline__ void rein_q8_store_sub(BlockQ8* __restrict__ o, unsigned l, float lo, float hi)
+struct ReinQ8Lane { int w0, w1; float d, sum; };   // what lane l of a row holds of the finished block
+
+__device__ __forceinline__ ReinQ8Lane rein_q8_quantize_sub(float lo, float hi)
 {
 #pragma clang fp contract(off)
     const float amax = rein_row_max(fabsf(lo), fabsf(hi));
@@ -65,10 +67,23 @@ __device__ __forceinline__ void rein_q8_store_sub(BlockQ8* __restrict__ o, unsig
     // bytes of a lane quad -> one dword per 16-element half: pairs, then pairs of pairs
     int p = q0 | (q1 << 16);                                                          // [q0, -, q1, -]
     p = p | (__builtin_amdgcn_update_dpp(0, p, 0xB1, 0xF, 0xF, false) << 8);          // even lanes: + lane^1
-    const int w0 = (p & 0xFFFF) | (__builtin_amdgcn_update_dpp(0, p, 0x4E, 0xF, 0xF, false) << 16);
-    const int w1 = ((unsigned)p >> 16) | (__builtin_amdgcn_update_dpp(0, p, 0x4E, 0xF, 0xF, false) & 0xFFFF0000);
-    if ((l & 3u) == 0u) { o->qs[l >> 2] = w0; o->qs[4 + (l >> 2)] = w1; }
-    if (l == 0u) { o->d = d; o->xsum = sum; }
+    ReinQ8Lane r;
+    r.w0 = (p & 0xFFFF) | (__builtin_amdgcn_update_dpp(0, p, 0x4E, 0xF, 0xF, false) << 16);
+    r.w1 = ((unsigned)p >> 16) | (__builtin_amdgcn_update_dpp(0, p, 0x4E, 0xF, 0xF, false) & 0xFFFF0000);
+    r.d = d;
+    r.sum = sum;
+    return r;
+}
+
+__device__ __forceinline__ void rein_q8_store_lane(BlockQ8* __restrict__ o, unsigned l, const ReinQ8Lane& r)
+{
+    if ((l & 3u) == 0u) { o->qs[l >> 2] = r.w0; o->qs[4 + (l >> 2)] = r.w1; }
+    if (l == 0u) { o->d = r.d; o->xsum = r.sum; }
+}
+
+__device__ __forceinline__ void rein_q8_store_sub(BlockQ8* __restrict__ o, unsigned l, float lo, float hi)
+{
+    rein_q8_store_lane(o, l, rein_q8_quantize_sub(lo, hi));
 }
 
 // exp(x), |relative error| < 3e-7 on [-87, 88]; outside, x is clamped (the result

@@ -113,6 +113,11 @@ def moe_gather_xq(xq_src, perm, xq_dst, nsub, n_used, n_entries, stream=None):
     check(lib.rein_moe_gather_xq(_p(xq_src), _p(perm), _p(xq_dst), nsub, n_used, n_entries, _s(stream)))
 
 
+def moe_quantize_scatter(x, inv, xq_dst, in_dim, n_used, n_tok, stream=None):
+    """quantize_q8 + moe_gather_xq in one launch (inv = inverse of the sort's perm)"""
+    check(lib.rein_moe_quantize_scatter(_p(x), _p(inv), _p(xq_dst), in_dim, n_used, n_tok, _s(stream)))
+
+
 def moe_scatter_rows(src, perm, dst, dim, n_entries, stream=None):
     check(lib.rein_moe_scatter_rows(_p(src), _p(perm), _p(dst), dim, n_entries, _s(stream)))
 

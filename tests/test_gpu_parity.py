@@ -376,7 +376,12 @@ def gpu_sort(ids, n_expert, bn):
     return bufs[2], bufs[3], bufs[4]
 
 
-def test_moe_sort_invariants():
+@pytest.mark.parametrize("split", [False, True])
+def test_moe_sort_invariants(split, monkeypatch):
+    # both forms of the sort: one workgroup (small routing tables) and the reference's
+    # zero / histogram / scan / scatter launches
+    if split:
+        monkeypatch.setenv("REIN_MOE_SORT_SPLIT", "1")
     rng = np.random.default_rng(1)
     for n_tok, n_used, n_expert, bn in [(512, 8, 128, 32), (7, 2, 200, 16), (300, 4, 3, 32)]:
         ids = rng.integers(0, n_expert, (n_tok, n_used)).astype(np.int32)
@@ -391,6 +396,42 @@ def test_moe_sort_invariants():
         assert len(set(valid.tolist())) == valid.size and valid.min() >= 0 and valid.max() < flat.size
         for e in range(n_expert):     # the order inside one expert is free (qwen35.rs:2956-2987)
             assert np.all(flat[perm[eoff[e]: eoff[e + 1]]] == e)
+
+
+def test_moe_quantize_scatter_equals_the_two_launches():
+    rng = np.random.default_rng(12)
+    for n_tok, n_used, in_dim in [(37, 8, 2048), (5, 2, 96), (600, 4, 256)]:
+        n = n_tok * n_used
+        x = rng.standard_normal((n_tok, in_dim)).astype(np.float32)
+        x[0, :32] = 0.0                                   # an all-zero block
+        perm = rng.permutation(n).astype(np.int32)
+        inv = np.empty(n, np.int32)
+        inv[perm] = np.arange(n, dtype=np.int32)
+        d_x = dev(x)
+        d_xq = hip.DeviceBuf(n_tok * in_dim // 32 * 40)
+        runtime.quantize_q8(d_x, d_xq, in_dim, n_tok)
+        d_chain = dev(np.full(n * in_dim // 32 * 40, 0xAA, np.uint8))
+        runtime.moe_gather_xq(d_xq, dev(perm), d_chain, in_dim // 32, n_used, n)
+        d_fused = dev(np.full(n * in_dim // 32 * 40, 0x55, np.uint8))
+        runtime.moe_quantize_scatter(d_x, dev(inv), d_fused, in_dim, n_used, n_tok)
+        hip.synchronize()
+        got = d_fused.to_host(np.uint8)
+        assert np.array_equal(got, d_chain.to_host(np.uint8))
+        want = orc.quantize_q8(x).reshape(n_tok, -1)[perm // n_used].reshape(-1)
+        assert np.array_equal(got, want)
+    # dropped entries (inv < 0) are skipped: their rows keep the fill
+    n_tok, n_used, in_dim = 4, 2, 64
+    x = rng.standard_normal((n_tok, in_dim)).astype(np.float32)
+    inv = np.array([0, -1, 1, 2, -1, 3, 4, 5], np.int32)
+    d_fused = dev(np.full(8 * 2 * 40, 0x55, np.uint8))
+    runtime.moe_quantize_scatter(dev(x), dev(inv), d_fused, in_dim, n_used, n_tok)
+    hip.synchronize()
+    got = d_fused.to_host(np.uint8).reshape(8, 80)
+    xq = orc.quantize_q8(x).reshape(n_tok, 80)
+    for i, pos in enumerate(inv):
+        if pos >= 0:
+            assert np.array_equal(got[pos], xq[i // n_used])
+    assert np.all(got[6:] == 0x55)
 
 
 def test_moe_gather_scatter_swiglu_combine():
