@@ -1154,6 +1154,21 @@ __device__ __forceinline__ void rein_mmq_dense(const uint8_t* __restrict__ w, co
 // rows expert_off[e] + 32*local .. of the expert-sorted xq / y.  Each tile runs
 // the tuned 32-token workgroup tile; any grid is correct, the block must be 256
 // threads (src/runtime/qwen35.rs:3062).
+// Expert of a token tile: the largest e with tile_off[e] <= tile.  Every wavefront counts the
+// entries that are <= tile with one load per lane and 64 experts (a binary search would be
+// seven dependent loads deep at 128 experts, in front of every workgroup's first fetch).
+__device__ __forceinline__ unsigned rein_mmq_tile_expert(const int* __restrict__ tile_off, unsigned n_expert, unsigned tile)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    unsigned n_le = 0;
+    for (unsigned e0 = 0; e0 < n_expert; e0 += 64u) {
+        const unsigned e = e0 + lane;
+        const bool le = e < n_expert && (unsigned)tile_off[e < n_expert ? e : 0u] <= tile;
+        n_le += (unsigned)__popcll(__ballot(le));
+    }
+    return n_le - 1u;                              // tile_off[0] = 0 <= tile: at least one
+}
+
 template <int FMT>
 __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ slab, unsigned bytes_per_expert,
                                                  const int* __restrict__ expert_off, const int* __restrict__ tile_off,
@@ -1164,12 +1179,7 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     const unsigned n_rb = (out_dim + 127u) / 128u;
     const unsigned n_tiles = (unsigned)tile_off[n_expert];
     for (unsigned tile = blockIdx.y; tile < n_tiles; tile += gridDim.y) {
-        unsigned lo = 0, hi = n_expert;            // largest e with tile_off[e] <= tile
-        while (hi - lo > 1) {
-            const unsigned mid = (lo + hi) >> 1;
-            if ((unsigned)tile_off[mid] <= tile) lo = mid; else hi = mid;
-        }
-        const unsigned e = lo;
+        const unsigned e = rein_mmq_tile_expert(tile_off, n_expert, tile);
         const unsigned tok_base = (unsigned)expert_off[e] + (tile - (unsigned)tile_off[e]) * 32u;
         const unsigned tok_end = (unsigned)expert_off[e + 1];
         if (tok_base >= tok_end) continue;         // host counted tiles with a smaller bn
@@ -1198,11 +1208,7 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
 {
     const unsigned tile = blockIdx.y, rb = blockIdx.x;
     if (blockDim.x != 256u || rb * 128u >= out_dim || tile >= (unsigned)tile_off[n_expert]) return;
-    unsigned lo = 0, hi = n_expert;                // largest e with tile_off[e] <= tile
-    while (hi - lo > 1) {
-        const unsigned mid = (lo + hi) >> 1;
-        if ((unsigned)tile_off[mid] <= tile) lo = mid; else hi = mid;
-    }
+    const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
     const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
     const unsigned tok_end = (unsigned)expert_off[lo + 1];
     if (tok_base >= tok_end) return;
