@@ -862,11 +862,11 @@ __device__ __forceinline__ rein_v4i rein_mmq_act_operand(const MmqLds<TM>& lds, 
 // order that keeps every wait off the freshest requests).
 // `ck` and `sm` are private copies; they are rotated so the loop indexes entries
 // 0 and 1.
-template <int FMT, int TM, class Refill>
+template <int FMT, int TM, class Refill, class Prefetch>
 __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds, MmqWLds<FMT>& wl, unsigned wsel,
                                                            MmqChunk<FMT> ck, typename MmqChunk<FMT>::Small sm,
                                                            rein_v16f (&acc)[TM / 32], unsigned j, unsigned h,
-                                                           bool more, const Refill& refill)
+                                                           bool more, const Refill& refill, const Prefetch& prefetch)
 {
     using C = MmqChunk<FMT>;
     constexpr int NT = TM / 32;
@@ -895,6 +895,10 @@ __device__ __forceinline__ void rein_mmq_chunk_math_rolled(const MmqLds<TM>& lds
         if (p == 2) {
             // slot 1 of this chunk: only the refill of slot 0 (if any) is younger
             if (more) REIN_WAIT_VMCNT(kDma); else REIN_WAIT_VMCNT(0);
+            // the next activation blocks are requested here, behind the wait, so that it
+            // does not wait for them: they have until the end of the chunk
+            __builtin_amdgcn_sched_barrier(0);
+            if (more) prefetch();
         }
         const uint4* slot = wl.q[wsel][p >> 1];
         const unsigned s4 = 2u * (p & 1u);
@@ -1037,9 +1041,11 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     // only ever count ring requests, never the compiler's (whose number of instructions
     // is its own business):
     //   top of c        small words of c+1                                  (registers)
-    //   after pair 1    activation image of c+1 -> LDS (blocks fetched during c-1),
-    //                   activation blocks of c+2 (registers), then ring slot 0 <- c+1
-    //   before pair 2   wait until only the slot 0 refill is in flight (slot 1 of c is in)
+    //   after pair 1    activation image of c+1 -> LDS (blocks fetched during c-1), then ring
+    //                   slot 0 <- c+1
+    //   before pair 2   wait until only the slot 0 refill is in flight (slot 1 of c is in);
+    //                   behind the wait, activation blocks of c+2 (registers): they have until
+    //                   the end of the chunk and the wait does not include them
     //   after pair 3    ring slot 1 <- c+1
     //   end of c        wait until only the slot 1 refill is in flight (slot 0 of c+1 is
     //                   in), barrier
@@ -1065,14 +1071,14 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
         rein_mmq_chunk_math_rolled<FMT, TM>(lds[buf], wl, wsel, ck, cur, acc, j, h, more, [&](unsigned half) {
             if (half == 0) {
                 rein_mmq_xstore<TM, C::kSplitK>(nxt, xr, n_sub, tok_base, tok_end, sb0 + 8);
-                // The loads below land in the registers the stores above have just read.  Without
-                // the fence the compiler issues them first, into other registers, and copies them
-                // over after the stores -- a wait for the loads in the middle of the chunk.
+                // the next fetch (behind the wait of pair 2) lands in the registers these stores
+                // have read; the fence keeps the compiler from issuing it up here into others
                 __builtin_amdgcn_sched_barrier(0);
-                // past the last chunk the fetch repeats on clamped addresses and is never stored
-                rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, more2 ? sb0 + 16 : sb0 + 8);
             }
             rein_mmq_wload<FMT>(wsrc, half, fmt, sb0 + 8 + 4 * half, n_sub);
+        }, [&]() {
+            // past the last chunk the fetch repeats on clamped addresses and is never stored
+            rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, more2 ? sb0 + 16 : sb0 + 8);
         });
         if (more) REIN_WAIT_VMCNT(kDma);             // slot 0 of the next chunk has landed
         __syncthreads();
