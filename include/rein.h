@@ -276,12 +276,34 @@ int rein_matvec_q8_0_splitk(const void *w, const void *xq, float *y_partials, un
  * Y[p_rows][out_dim] = Xq . W^T on the int8 MFMA path. */
 int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                  unsigned out_dim, unsigned p_rows, rein_stream_t s);
+/* The same product with a caller-provided workspace of rein_mmq_workspace_bytes(fmt, in_dim,
+ * p_rows) bytes (16-byte aligned; 0 = the format or row count has no use for one, and NULL
+ * falls back to rein_mmq_xq8).  With it Q4_K above 16 rows runs on the block-scaled fp6
+ * matrix instruction: the activations are first brought into operand form in the workspace
+ * (one extra launch), then the GEMM streams them from there.  The reference keeps such
+ * scratch in its PrefillGemm object (src/runtime/prefill.rs:479-495); here the caller owns
+ * it, so nothing allocates and the call can be captured into a graph.  Calls that share a
+ * workspace must be ordered on one stream. */
+size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows);
+int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
+                    unsigned out_dim, unsigned p_rows, void *workspace, size_t workspace_bytes,
+                    rein_stream_t s);
+/* How rein_mmq_xq8_ws cuts the tokens of a 128-row block: n4 groups of four 32-token tiles,
+ * n2 groups of two, single tiles for the rest.  No counterpart in the reference. */
+int rein_mmq_tile_plan_ws(int fmt, unsigned out_dim, unsigned p_rows, unsigned *n4, unsigned *n2);
 /* PrefillGemm::matmul_into_raw (src/runtime/prefill.rs:343-384): quantize x
  * [n_rows][in_dim] into the caller's `xq_scratch` (n_rows*in_dim/32*40 bytes),
  * then dispatch by row count: 1 -> matvec, 2..8 -> batched matvec (the reference
  * switches to its narrow MMQ at 5), above -> MMQ. */
 int rein_matmul(int fmt, const void *w, const float *x, float *y, unsigned in_dim,
                 unsigned out_dim, unsigned n_rows, void *xq_scratch, rein_stream_t s);
+/* rein_matmul with one scratch buffer of rein_matmul_scratch_bytes(fmt, in_dim, n_rows) bytes
+ * (16-byte aligned) that holds the quantized activations and, for the MMQ path, the workspace
+ * of rein_mmq_xq8_ws.  A scratch that only holds the activations runs rein_matmul. */
+size_t rein_matmul_scratch_bytes(int fmt, unsigned in_dim, unsigned n_rows);
+int rein_matmul_ws(int fmt, const void *w, const float *x, float *y, unsigned in_dim,
+                   unsigned out_dim, unsigned n_rows, void *scratch, size_t scratch_bytes,
+                   rein_stream_t s);
 /* Which path rein_matmul takes: 0 matvec, 1 batched matvec, 2 MMQ; <0 on error. */
 int rein_matmul_path(int fmt, unsigned n_rows);
 /* How rein_mmq_xq8 tiles the tokens of a P-row GEMM above 16 rows: the number of 64-token
@@ -298,6 +320,13 @@ int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows);
 int rein_block_dot_parts(int fmt);
 int rein_block_dots(int fmt, const void *w, const void *xq, int32_t *out, unsigned in_dim,
                     unsigned out_dim, unsigned n_rows, int via_mfma, rein_stream_t s);
+
+/* The per-block dots of the workspace launch of rein_mmq_xq8_ws (Q4_K): out [n_rows][out_dim]
+ * [in_dim/32] int32, converted from the fp32 results of the fp6 matrix instruction, which are
+ * exact integers.  workspace as for rein_mmq_xq8_ws (any n_rows). */
+int rein_mmq_block_dots_ws(int fmt, const void *w, const void *xq, int32_t *out, unsigned in_dim,
+                           unsigned out_dim, unsigned n_rows, void *workspace,
+                           size_t workspace_bytes, rein_stream_t s);
 
 /* ------------------------------------------------------------------- MoE */
 /* moe_topk_f32 (kernels/moe_topk.cpp:17-108; launcher qwen35.rs:2873-2886) */

@@ -82,6 +82,12 @@ SIGNATURES = {
     "rein_matvec_batched_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_mmq_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_matmul": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _vp]),
+    "rein_mmq_workspace_bytes": (_sz, [_i, _u, _u]),
+    "rein_mmq_xq8_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
+    "rein_mmq_tile_plan_ws": (_i, [_i, _u, _u, _vp, _vp]),
+    "rein_mmq_block_dots_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
+    "rein_matmul_scratch_bytes": (_sz, [_i, _u, _u]),
+    "rein_matmul_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
     "rein_matmul_path": (_i, [_i, _u]),
     "rein_mmq_tile_plan": (_i, [_i, _u, _u]),
     "rein_block_dot_parts": (_i, [_i]),

@@ -633,6 +633,140 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_t32", (unsigned)grid, 1, 1, 256, 0, s, args);
 }
 
+// ---- Q4_K on the block-scaled fp6 matrix instruction (kernels/mmq_fp6.h)
+namespace {
+constexpr unsigned kX6Rec = 4352;          // REIN_X6_REC: bytes per (sub-block pair, 32-token tile) record
+size_t x6_image_bytes(unsigned n_sub, unsigned p_rows)
+{
+    return (size_t)((n_sub + 1) / 2) * ((p_rows + 31) / 32) * kX6Rec + 1024;      // rein_x6_bytes
+}
+bool mmq6_format(int fmt) { return fmt == REIN_TYPE_Q4_K && env_u("REIN_MMQ6", 1) != 0; }
+unsigned mmq6_lds_bytes(unsigned nt)       // rein_mmq6_lds_bytes<NT>()
+{
+    return 3 * ((nt * kX6Rec + 1023u) & ~1023u) + 4 * 4096 + 4 * 1280;
+}
+// Token groups per 128-row block: n4 groups of four 32-token tiles, n2 of two, the rest single.
+// Relative cost of a workgroup per 32-token tile, fitted to a sweep of the splits of 512 x 5120
+// x 17408: 1.00 in a group of four, 1.15 in a group of two, 1.8 alone (the weight unpack is
+// shared by fewer tiles, and a narrow workgroup still holds a wide one's LDS).  Workgroups are
+// handed to CUs in launch order, widest first; a CU's finish time is the sum of what it was
+// handed, and the split with the earliest last finish wins (ties: the least total work).
+void mmq6_pick(unsigned out_dim, unsigned p_rows, unsigned* n4_out, unsigned* n2_out)
+{
+    const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + 31) / 32;
+    const unsigned f4 = env_u("REIN_MMQ6_N4", 0xFFFFFFFFu), f2 = env_u("REIN_MMQ6_N2", 0xFFFFFFFFu);
+    if (f4 != 0xFFFFFFFFu || f2 != 0xFFFFFFFFu) {
+        unsigned n4 = f4 == 0xFFFFFFFFu ? 0 : std::min(f4, n_tt / 4);
+        unsigned n2 = f2 == 0xFFFFFFFFu ? 0 : std::min(f2, (n_tt - 4 * n4) / 2);
+        *n4_out = n4; *n2_out = n2;
+        return;
+    }
+    const unsigned a4 = n_tt / 4, rest = n_tt - 4 * a4;
+    *n4_out = a4; *n2_out = rest / 2;                          // very large grids: granularity no longer matters
+    if ((unsigned long long)n_rb * n_tt > 64ull * kCUs) return;
+    static std::mutex mu;
+    static std::unordered_map<unsigned long long, unsigned> memo;
+    const unsigned long long key = ((unsigned long long)out_dim << 32) | p_rows;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = memo.find(key);
+        if (it != memo.end()) { *n4_out = it->second >> 16; *n2_out = it->second & 0xFFFFu; return; }
+    }
+    const double c4 = 4.0, c2 = 2.3, c1 = 1.8;
+    double best = 1e30;
+    unsigned b4 = 0, b2 = 0;
+    std::vector<double> load(kCUs);
+    for (unsigned n4 = a4 > 3 ? a4 - 3 : 0; n4 <= a4; n4++) {
+        const unsigned left = n_tt - 4 * n4;
+        for (unsigned n2 = 0; 2 * n2 <= left && n2 <= 8; n2++) {
+            const unsigned n1 = left - 2 * n2;
+            std::fill(load.begin(), load.end(), 0.0);
+            std::make_heap(load.begin(), load.end());          // max-heap of negated loads: top = least loaded CU
+            const unsigned long long cnt[3] = {(unsigned long long)n_rb * n4, (unsigned long long)n_rb * n2, (unsigned long long)n_rb * n1};
+            const double cost[3] = {c4, c2, c1};
+            for (int kind = 0; kind < 3; kind++)
+                for (unsigned long long i = 0; i < cnt[kind]; i++) {
+                    std::pop_heap(load.begin(), load.end());
+                    load.back() -= cost[kind];
+                    std::push_heap(load.begin(), load.end());
+                }
+            const double total = (cnt[0] * c4 + cnt[1] * c2 + cnt[2] * c1) / kCUs;
+            const double finish = -*std::min_element(load.begin(), load.end()) + 1e-3 * total;
+            if (finish < best - 1e-9) { best = finish; b4 = n4; b2 = n2; }
+        }
+    }
+    *n4_out = b4; *n2_out = b2;
+    std::lock_guard<std::mutex> lock(mu);
+    if (memo.size() > 4096) memo.clear();
+    memo[key] = (b4 << 16) | b2;
+}
+int mmq6_prep(const void* xq, void* img, unsigned n_sub, unsigned p_rows, rein_stream_t s)
+{
+    void* a[] = {(void*)&xq, (void*)&img, (void*)&n_sub, (void*)&p_rows};
+    return launch("rein_mmq6_prep", (p_rows + 31) / 32, (n_sub + 7) / 8, 1, 256, 0, s, a);
+}
+}  // namespace
+
+size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows)
+{
+    // below ~300 rows the int8 launch (more, smaller workgroups in flight) is the faster one:
+    // 128 rows 61 vs 93 us, 256 rows 112 vs 122 us, 512 rows 185 vs 177 us at 5120 x 17408
+    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < env_u("REIN_MMQ6_FROM", 320)) return 0;
+    return x6_image_bytes(in_dim / 32, p_rows);
+}
+
+int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                    unsigned p_rows, void* workspace, size_t workspace_bytes, rein_stream_t s)
+{
+    const char* who = "rein_mmq_xq8_ws";
+    const size_t need = rein_mmq_workspace_bytes(fmt, in_dim, p_rows);
+    if (!workspace || need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
+    if (int rc = check_ptr(who, w, 16, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    if (int rc = check_ptr(who, workspace, 16, "workspace")) return rc;
+    if (workspace_bytes < need)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace of " + std::to_string(workspace_bytes) + " bytes, rein_mmq_workspace_bytes asks for " + std::to_string(need));
+    unsigned n4, n2;
+    mmq6_pick(out_dim, p_rows, &n4, &n2);
+    const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + 31) / 32, n1 = n_tt - 4 * n4 - 2 * n2;
+    const unsigned long long grid = 8ull * ((n_rb + 7) / 8) * (n4 + n2 + n1);
+    if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, std::string(who) + ": too many tiles for one launch");
+    if (int rc = mmq6_prep(xq, workspace, in_dim / 32, p_rows, s)) return rc;
+    void* a[] = {(void*)&w, (void*)&workspace, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&n4, (void*)&n2};
+    return launch("rein_mmq6_q4k_mix", (unsigned)grid, 1, 1, 256, mmq6_lds_bytes(n4 ? 4 : n2 ? 2 : 1), s, a);
+}
+
+int rein_mmq_tile_plan_ws(int fmt, unsigned out_dim, unsigned p_rows, unsigned* n4, unsigned* n2)
+{
+    if (!n4 || !n2) return fail(REIN_E_BAD_POINTER, "rein_mmq_tile_plan_ws: NULL output");
+    if (!mmq6_format(fmt)) return fail(REIN_E_BAD_FORMAT, "rein_mmq_tile_plan_ws: the format has no workspace launch");
+    if (out_dim == 0 || p_rows == 0) return fail(REIN_E_BAD_SHAPE, "rein_mmq_tile_plan_ws: empty shape");
+    mmq6_pick(out_dim, p_rows, n4, n2);
+    return 0;
+}
+
+int rein_mmq_block_dots_ws(int fmt, const void* w, const void* xq, int32_t* out, unsigned in_dim, unsigned out_dim,
+                           unsigned n_rows, void* workspace, size_t workspace_bytes, rein_stream_t s)
+{
+    const char* who = "rein_mmq_block_dots_ws";
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_rows)) return rc;
+    if (!mmq6_format(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": the format has no workspace launch");
+    if (int rc = check_ptr(who, w, 16, "w")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, out, 4, "out")) return rc;
+    if (int rc = check_ptr(who, workspace, 16, "workspace")) return rc;
+    if (workspace_bytes < x6_image_bytes(in_dim / 32, n_rows))
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace too small");
+    const unsigned n_rb = (out_dim + 127) / 128, n_tt = (n_rows + 31) / 32;
+    const unsigned long long grid = 8ull * ((n_rb + 7) / 8) * n_tt;
+    if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, std::string(who) + ": too many tiles for one launch");
+    if (int rc = mmq6_prep(xq, workspace, in_dim / 32, n_rows, s)) return rc;
+    void* a[] = {(void*)&w, (void*)&workspace, (void*)&out, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+    return launch("rein_mmq6_q4k_dots", (unsigned)grid, 1, 1, 256, mmq6_lds_bytes(1), s, a);
+}
+
 int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows)
 {
     if (!rein_block_size(fmt)) return fail(REIN_E_BAD_FORMAT, "rein_mmq_tile_plan: unknown format " + std::to_string(fmt));
@@ -659,6 +793,28 @@ int rein_matmul(int fmt, const void* w, const float* x, float* y, unsigned in_di
     case 1:  return rein_matvec_batched_xq8(fmt, w, xq_scratch, y, in_dim, out_dim, n_rows, s);
     default: return rein_mmq_xq8(fmt, w, xq_scratch, y, in_dim, out_dim, n_rows, s);
     }
+}
+
+size_t rein_matmul_scratch_bytes(int fmt, unsigned in_dim, unsigned n_rows)
+{
+    if (!rein_block_size(fmt) || in_dim == 0 || in_dim % 32 != 0 || n_rows == 0) return 0;
+    const size_t xq = ((size_t)n_rows * (in_dim / 32) * 40 + 255) & ~(size_t)255;
+    return xq + (rein_matmul_path(fmt, n_rows) == 2 ? rein_mmq_workspace_bytes(fmt, in_dim, n_rows) : 0);
+}
+
+int rein_matmul_ws(int fmt, const void* w, const float* x, float* y, unsigned in_dim, unsigned out_dim,
+                   unsigned n_rows, void* scratch, size_t scratch_bytes, rein_stream_t s)
+{
+    if (int rc = check_shape("rein_matmul_ws", fmt, in_dim, out_dim, n_rows)) return rc;
+    if (int rc = check_dense_fmt("rein_matmul_ws", fmt)) return rc;
+    if (int rc = check_ptr("rein_matmul_ws", scratch, 16, "scratch")) return rc;
+    const size_t xq = ((size_t)n_rows * (in_dim / 32) * 40 + 255) & ~(size_t)255;
+    if (scratch_bytes < (size_t)n_rows * (in_dim / 32) * 40)
+        return fail(REIN_E_BAD_SHAPE, "rein_matmul_ws: scratch smaller than the quantized activations");
+    if (rein_matmul_path(fmt, n_rows) != 2 || scratch_bytes < rein_matmul_scratch_bytes(fmt, in_dim, n_rows))
+        return rein_matmul(fmt, w, x, y, in_dim, out_dim, n_rows, scratch, s);
+    if (int rc = rein_quantize_q8(x, scratch, in_dim, n_rows, s)) return rc;
+    return rein_mmq_xq8_ws(fmt, w, scratch, y, in_dim, out_dim, n_rows, static_cast<char*>(scratch) + xq, scratch_bytes - xq, s);
 }
 
 int rein_block_dot_parts(int fmt) { return fmt == REIN_TYPE_Q6_K ? 2 : (rein_block_size(fmt) ? 1 : 0); }

@@ -76,6 +76,38 @@ def mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, stream=None):
     check(lib.rein_mmq_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _s(stream)))
 
 
+def mmq_workspace_bytes(fmt, in_dim, p_rows):
+    """bytes of workspace mmq_xq8_ws wants for this shape (0: none)"""
+    return int(lib.rein_mmq_workspace_bytes(fmt, in_dim, p_rows))
+
+
+def mmq_xq8_ws(fmt, w, xq, y, in_dim, out_dim, p_rows, workspace, workspace_bytes, stream=None):
+    """mmq_xq8 with the caller's workspace (the scratch PrefillGemm keeps, prefill.rs:479-495)"""
+    check(lib.rein_mmq_xq8_ws(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _p(workspace), workspace_bytes,
+                              _s(stream)))
+
+
+def mmq_tile_plan_ws(fmt, out_dim, p_rows):
+    """(n4, n2): token groups of four and of two 32-token tiles per 128-row block in mmq_xq8_ws"""
+    n4, n2 = C.c_uint(0), C.c_uint(0)
+    check(lib.rein_mmq_tile_plan_ws(fmt, out_dim, p_rows, C.byref(n4), C.byref(n2)))
+    return n4.value, n2.value
+
+
+def mmq_block_dots_ws(fmt, w, xq, out, in_dim, out_dim, n_rows, workspace, workspace_bytes, stream=None):
+    check(lib.rein_mmq_block_dots_ws(fmt, _p(w), _p(xq), _p(out), in_dim, out_dim, n_rows, _p(workspace),
+                                     workspace_bytes, _s(stream)))
+
+
+def matmul_scratch_bytes(fmt, in_dim, n_rows):
+    return int(lib.rein_matmul_scratch_bytes(fmt, in_dim, n_rows))
+
+
+def matmul_ws(fmt, w, x, y, in_dim, out_dim, n_rows, scratch, scratch_bytes, stream=None):
+    """matmul with one scratch buffer for the quantized activations and the MMQ workspace"""
+    check(lib.rein_matmul_ws(fmt, _p(w), _p(x), _p(y), in_dim, out_dim, n_rows, _p(scratch), scratch_bytes, _s(stream)))
+
+
 def matmul(fmt, w, x, y, in_dim, out_dim, n_rows, xq_scratch, stream=None):
     """PrefillGemm::matmul_into_raw (src/runtime/prefill.rs:343-384)"""
     check(lib.rein_matmul(fmt, _p(w), _p(x), _p(y), in_dim, out_dim, n_rows, _p(xq_scratch), _s(stream)))
