@@ -118,248 +118,6 @@ __device__ __forceinline__ void rein_matvec_body(const uint8_t* __restrict__ w,
     }
 }
 
-// LDS image of the activation blocks of one iteration (64*U sub-blocks x B rows),
-// split so that a lane's reads are conflict-free: header (d, xsum), quants 0-15,
-// quants 16-31.
-template <int B, int U>
-struct XStage {
-    uint2 hdr[B][64 * U];
-    uint4 lo[B][64 * U];
-    uint4 hi[B][64 * U];
-};
-
-// Tuned decode matvec: the same math as rein_matvec_body, for a fixed workgroup of
-// WPB wavefronts.  The activation blocks are 40 bytes at 8-byte alignment, so a
-// per-lane read of one block is three misaligned vector loads that every
-// wavefront repeats; here the workgroup fetches each iteration's blocks once
-// with fully coalesced 8-byte loads, stages them in LDS (double-buffered, one
-// barrier per iteration) and every lane reads its block with aligned ds_read.
-// The weight loads of the iteration are issued before the staging, so their HBM
-// latency overlaps it.  One row group per wavefront: grid = ceil(groups / WPB).
-template <int FMT, int R, int B, int U, int WPB>
-__device__ __forceinline__ void rein_matvec_lds_body(const uint8_t* __restrict__ w,
-                                                     const BlockQ8* __restrict__ xq,
-                                                     float* __restrict__ y,
-                                                     unsigned in_dim, unsigned out_dim, unsigned n_rows)
-{
-    using F = Fmt<FMT>;
-    __shared__ XStage<B, U> stage[2];
-    const unsigned lane  = threadIdx.x & 63u;
-    const unsigned wave  = threadIdx.x >> 6;
-    const unsigned n_sub = in_dim >> 5;
-    const F fmt(w, n_sub, out_dim);
-    const unsigned rmax = out_dim - 1;
-    const unsigned row0 = (blockIdx.x * WPB + wave) * R;     // may lie past the end: clamped, not stored
-
-    float acc[R][B];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < B; b++) acc[r][b] = 0.0f;
-
-    const uint2* xw = reinterpret_cast<const uint2*>(xq);    // 5 words of 8 bytes per block
-    unsigned buf = 0;
-    for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 64 * U, buf ^= 1u) {
-        bool     live[U];
-        unsigned sb[U];
-        typename F::Raw raw[U][R];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            live[u] = sb0 + 64 * u + lane < n_sub;
-            sb[u]   = live[u] ? sb0 + 64 * u + lane : n_sub - 1;
-#pragma unroll
-            for (int r = 0; r < R; r++) raw[u][r] = fmt.load(min(row0 + r, rmax), sb[u]);
-        }
-
-        // stage this iteration's activation blocks: word i of the chunk of row b
-        const unsigned chunk_sbs = min(64u * U, n_sub - sb0);
-        XStage<B, U>& st = stage[buf];
-        for (unsigned b = 0; b < n_rows; b++) {
-            const uint2* src = xw + ((size_t)b * n_sub + sb0) * 5;
-            for (unsigned i = threadIdx.x; i < chunk_sbs * 5; i += WPB * 64) {
-                const uint2 v = src[i];
-                const unsigned blk = i / 5, part = i - blk * 5;
-                if (part == 0) st.hdr[b][blk] = v;
-                else if (part < 3) reinterpret_cast<uint2*>(&st.lo[b][blk])[part - 1] = v;
-                else reinterpret_cast<uint2*>(&st.hi[b][blk])[part - 3] = v;
-            }
-        }
-        __syncthreads();
-
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const unsigned ls = live[u] ? 64 * u + lane : 0;         // slot inside the chunk
-            XBlocks<B> xb;
-#pragma unroll
-            for (int b = 0; b < B; b++) {
-                const unsigned bb = min((unsigned)b, n_rows - 1);
-                const uint2 h = st.hdr[bb][ls];
-                const uint4 lo = st.lo[bb][ls], hi = st.hi[bb][ls];
-                xb.dx[b]   = live[u] ? __builtin_bit_cast(float, h.x) : 0.0f;
-                xb.xsum[b] = live[u] ? __builtin_bit_cast(float, h.y) : 0.0f;
-                xb.q[b][0] = (int)lo.x; xb.q[b][1] = (int)lo.y; xb.q[b][2] = (int)lo.z; xb.q[b][3] = (int)lo.w;
-                xb.q[b][4] = (int)hi.x; xb.q[b][5] = (int)hi.y; xb.q[b][6] = (int)hi.z; xb.q[b][7] = (int)hi.w;
-            }
-            XSums xs[B];
-#pragma unroll
-            for (int b = 0; b < B; b++) {
-                if (F::kNeedsXSums) xs[b] = rein_xsums(xb.q[b]);
-                else { xs[b].lo = 0; xs[b].hi = 0; }
-            }
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                SubW sw;
-                F::unpack(raw[u][r], sw);
-#pragma unroll
-                for (int b = 0; b < B; b++) {
-                    int i0 = 0, i1 = 0;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        i0 = rein_dot4(sw.w[j], xb.q[b][j], i0);
-                        i1 = rein_dot4(sw.w[j + 4], xb.q[b][j + 4], i1);
-                    }
-                    acc[r][b] += F::term(sw, i0, i1, xb.dx[b], xb.xsum[b], xs[b]);
-                }
-            }
-        }
-    }
-
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < B; b++) {
-            const float s = rein_wave_sum(acc[r][b]);
-            if (lane == 0 && row0 + r < out_dim && (unsigned)b < n_rows)
-                y[(size_t)b * out_dim + row0 + r] = s;
-        }
-}
-
-// Persistent decode matvec.  The grid is sized to what is resident at once
-// (a few wavefronts per SIMD on every CU) and wavefront i walks row groups
-// i, i+W, i+2W, ... so all wavefronts retire together and there is no ragged
-// last round.  The activation rows (B x n_sub blocks) are staged once per
-// workgroup in dynamic LDS, split into header / low quants / high quants planes
-// so per-lane reads are aligned and conflict-free.  The unit of work is one trip
-// (64 sub-blocks of R rows); the next unit's weight loads are issued before the
-// current unit's dots, so HBM requests stay in flight across the math.
-// Dynamic shared memory: B * n_sub * 40 bytes.
-template <int FMT, int R, int B, int WPB>
-__device__ __forceinline__ void rein_matvec_persist_body(const uint8_t* __restrict__ w,
-                                                         const BlockQ8* __restrict__ xq,
-                                                         float* __restrict__ y,
-                                                         unsigned in_dim, unsigned out_dim, unsigned n_rows)
-{
-    using F = Fmt<FMT>;
-    extern __shared__ uint4 rein_dyn_lds[];
-    const unsigned lane  = threadIdx.x & 63u;
-    const unsigned wave  = threadIdx.x >> 6;
-    const unsigned n_sub = in_dim >> 5;
-    const F fmt(w, n_sub, out_dim);
-    const unsigned rmax = out_dim - 1;
-
-    uint4* s_lo  = rein_dyn_lds;                                   // [B][n_sub]
-    uint4* s_hi  = s_lo + (size_t)B * n_sub;                       // [B][n_sub]
-    uint2* s_hdr = reinterpret_cast<uint2*>(s_hi + (size_t)B * n_sub);   // [B][n_sub]
-
-    const unsigned n_groups = (out_dim + R - 1) / R;
-    const unsigned n_waves  = gridDim.x * WPB;
-    const unsigned wid      = blockIdx.x * WPB + wave;
-    const unsigned trips    = (n_sub + 63u) >> 6;
-    const unsigned my_groups = wid < n_groups ? (n_groups - wid + n_waves - 1) / n_waves : 0;
-    const unsigned n_units  = my_groups * trips;
-
-    // first unit's weights go out before the activation staging
-    typename F::Raw cur[R];
-    {
-        const unsigned sb = min(lane, n_sub - 1);
-#pragma unroll
-        for (int r = 0; r < R; r++) cur[r] = fmt.load(min(wid * R + r, rmax), sb);
-    }
-
-    const uint2* xw = reinterpret_cast<const uint2*>(xq);
-    for (unsigned b = 0; b < n_rows; b++) {
-        const uint2* src = xw + (size_t)b * n_sub * 5;
-        for (unsigned i = threadIdx.x; i < n_sub * 5; i += WPB * 64) {
-            const uint2 v = src[i];
-            const unsigned blk = i / 5, part = i - blk * 5;
-            if (part == 0) s_hdr[b * n_sub + blk] = v;
-            else if (part < 3) reinterpret_cast<uint2*>(&s_lo[b * n_sub + blk])[part - 1] = v;
-            else reinterpret_cast<uint2*>(&s_hi[b * n_sub + blk])[part - 3] = v;
-        }
-    }
-    __syncthreads();
-
-    float acc[R][B];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < B; b++) acc[r][b] = 0.0f;
-
-    unsigned g = wid, trip = 0;
-    for (unsigned unit = 0; unit < n_units; unit++) {
-        // next unit (same group next trip, or next group first trip)
-        unsigned ng = g, ntrip = trip + 1;
-        if (ntrip == trips) { ntrip = 0; ng = g + n_waves; }
-        typename F::Raw nxt[R];
-        if (unit + 1 < n_units) {
-            const unsigned nsb = min(ntrip * 64 + lane, n_sub - 1);
-#pragma unroll
-            for (int r = 0; r < R; r++) nxt[r] = fmt.load(min(ng * R + r, rmax), nsb);
-        }
-
-        const bool     live = trip * 64 + lane < n_sub;
-        const unsigned sb   = live ? trip * 64 + lane : n_sub - 1;
-        XBlocks<B> xb;
-#pragma unroll
-        for (int b = 0; b < B; b++) {
-            const unsigned o = min((unsigned)b, n_rows - 1) * n_sub + sb;
-            const uint2 h = s_hdr[o];
-            const uint4 lo = s_lo[o], hi = s_hi[o];
-            xb.dx[b]   = live ? __builtin_bit_cast(float, h.x) : 0.0f;
-            xb.xsum[b] = live ? __builtin_bit_cast(float, h.y) : 0.0f;
-            xb.q[b][0] = (int)lo.x; xb.q[b][1] = (int)lo.y; xb.q[b][2] = (int)lo.z; xb.q[b][3] = (int)lo.w;
-            xb.q[b][4] = (int)hi.x; xb.q[b][5] = (int)hi.y; xb.q[b][6] = (int)hi.z; xb.q[b][7] = (int)hi.w;
-        }
-        XSums xs[B];
-#pragma unroll
-        for (int b = 0; b < B; b++) {
-            if (F::kNeedsXSums) xs[b] = rein_xsums(xb.q[b]);
-            else { xs[b].lo = 0; xs[b].hi = 0; }
-        }
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            SubW sw;
-            F::unpack(cur[r], sw);
-#pragma unroll
-            for (int b = 0; b < B; b++) {
-                int i0 = 0, i1 = 0;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    i0 = rein_dot4(sw.w[j], xb.q[b][j], i0);
-                    i1 = rein_dot4(sw.w[j + 4], xb.q[b][j + 4], i1);
-                }
-                acc[r][b] += F::term(sw, i0, i1, xb.dx[b], xb.xsum[b], xs[b]);
-            }
-        }
-
-        if (trip + 1 == trips) {
-#pragma unroll
-            for (int r = 0; r < R; r++)
-#pragma unroll
-                for (int b = 0; b < B; b++) {
-                    const float s = rein_wave_sum(acc[r][b]);
-                    if (lane == 0 && g * R + r < out_dim && (unsigned)b < n_rows)
-                        y[(size_t)b * out_dim + g * R + r] = s;
-                    acc[r][b] = 0.0f;
-                }
-        }
-#pragma unroll
-        for (int r = 0; r < R; r++) cur[r] = nxt[r];
-        g = ng;
-        trip = ntrip;
-    }
-}
-
 // Per-block integer dots exactly as the matvec forms them, for the bit-exact
 // parity check: out[((t*out_dim + row)*n_sub + sb)*parts + p].  One lane per
 // (row, sub-block); grid-stride over rows; blockIdx.y = activation row t.
@@ -411,22 +169,6 @@ __device__ __forceinline__ void rein_block_dots_body(const uint8_t* __restrict__
     extern "C" __global__ __launch_bounds__(256) void name(REIN_MATVEC_ARGS, unsigned int n_rows) \
     {                                                                                             \
         rein_matvec_body<FMT, R, B>(w, xq, y, in_dim, out_dim, n_rows);                           \
-    }
-
-// tuned variant: LDS-staged activations, fixed workgroup of WPB wavefronts
-#define REIN_DEFINE_MATVEC_LDS(name, FMT, R, B, U, WPB)                                           \
-    extern "C" __global__ __launch_bounds__(WPB * 64) void name(REIN_MATVEC_ARGS,                 \
-                                                                unsigned int n_rows)              \
-    {                                                                                             \
-        rein_matvec_lds_body<FMT, R, B, U, WPB>(w, xq, y, in_dim, out_dim, n_rows);               \
-    }
-
-// tuned variant: persistent wavefronts, activations resident in dynamic LDS
-#define REIN_DEFINE_MATVEC_PERSIST(name, FMT, R, B, WPB)                                          \
-    extern "C" __global__ __launch_bounds__(WPB * 64) void name(REIN_MATVEC_ARGS,                 \
-                                                                unsigned int n_rows)              \
-    {                                                                                             \
-        rein_matvec_persist_body<FMT, R, B, WPB>(w, xq, y, in_dim, out_dim, n_rows);              \
     }
 
 // tuned variant with U trips of loads in flight per iteration

@@ -9,11 +9,13 @@
 //   * activations: the TM x 8 BlockQ8 of the chunk are staged in LDS, split into
 //     the two 16-quant halves (so an MFMA operand is one conflict-free
 //     ds_read_b128) plus planes of dx and of the bf16 splits of xsum;
-//   * weights: lane (j = lane%32, h = lane/32) streams row j's eight sub-blocks
-//     straight from HBM/L2 (8 x 16 B contiguous = one cache line, scales as one
-//     16 B load), expands half h of each to int8 in registers, and keeps them
-//     for all TM/32 token tiles.  Weights have no reuse across wavefronts in
-//     this mapping, so they never touch LDS;
+//   * weights: lane (j = lane%32, h = lane/32) owns row j's eight sub-blocks, expands
+//     half h of each to int8 in registers and keeps them for all TM/32 token tiles.
+//     Weights have no reuse across wavefronts in this mapping.  The plain kernels
+//     (rein_mmq_tile) load them straight into registers (8 x 16 B contiguous = one
+//     cache line, scales as one 16 B load); the tuned kernel (rein_mmq_pipelined_tile)
+//     moves the 16-byte plane HBM -> LDS asynchronously into a per-wavefront ring and
+//     reads it back as it is consumed;
 //   * per sub-block and tile one v_mfma_i32_32x32x32_i8 (tokens = rows of the
 //     tile, weights = columns) yields the exact int32 block dots; MFMA K = 32
 //     is exactly one sub-block, lane half h carries quants 16h..16h+15 on both

@@ -10,3 +10,16 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(autouse=True)
+def _release_device_uploads(request):
+    """GPU tests: wait for the test's launches, then free what helpers.dev() uploaded."""
+    yield
+    if request.node.get_closest_marker("gpu") is None:
+        return
+    import helpers
+    if helpers._uploads:
+        from reinstinct_amd import hip
+        hip.synchronize()
+        helpers.release_uploads()

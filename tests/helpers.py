@@ -5,6 +5,23 @@ from oracle import orc
 
 MASK64 = (1 << 64) - 1
 
+# Device uploads of the GPU tests.  Launches are asynchronous: a buffer passed straight into a
+# launch as `dev(array)` would otherwise be freed when the call returns, while the kernel may
+# still read it.  They are kept here and released by conftest's fixture after each test has
+# synchronized.
+_uploads = []
+
+
+def dev(a):
+    from reinstinct_amd import hip
+    buf = hip.DeviceBuf.from_host(np.ascontiguousarray(a))
+    _uploads.append(buf)
+    return buf
+
+
+def release_uploads():
+    _uploads.clear()
+
 
 class Lcg:
     """The reference tests' generator (src/runtime/kernels.rs:3030-3048):

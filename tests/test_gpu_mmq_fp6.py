@@ -30,8 +30,7 @@ def gpu():
     os.environ.pop("REIN_MMQ6_FROM", None)
 
 
-def dev(a):
-    return hip.DeviceBuf.from_host(a)
+from helpers import dev  # noqa: E402  (uploads that stay alive until the test's last launch has finished)
 
 
 def weights(in_dim, out_dim, seed, gaussian):

@@ -28,12 +28,12 @@ def gpu():
     hip.synchronize()
 
 
-def dev(a):
-    return hip.DeviceBuf.from_host(np.ascontiguousarray(a))
+from helpers import dev  # noqa: E402  (uploads that stay alive until the test's last launch has finished)
 
 
-def expert_slabs(fmt, in_dim, out_dim, n_expert, seed, gaussian=True):
-    # out_dim a multiple of 8 keeps every expert's slab 16-byte aligned (the library checks it)
+def expert_slabs(fmt, in_dim, out_dim, n_expert, seed, gaussian=True, pad16=False):
+    # out_dim a multiple of 8 keeps every expert's slab 16-byte aligned (the library checks it);
+    # pad16 pads each slab to a multiple of 16 bytes instead (bytes_per_expert is a stride)
     slabs = []
     for e in range(n_expert):
         if gaussian and fmt != rein.Q5_1:               # no synthetic quantizer for Q5_1
@@ -42,6 +42,8 @@ def expert_slabs(fmt, in_dim, out_dim, n_expert, seed, gaussian=True):
         else:
             raw = random_raw_weights(fmt, in_dim, out_dim, seed + e)
         slabs.append(quant.repack_for_matvec(fmt, raw, in_dim, out_dim))
+        if pad16 and slabs[-1].nbytes % 16:
+            slabs[-1] = np.concatenate([slabs[-1], np.zeros(16 - slabs[-1].nbytes % 16, np.uint8)])
     return np.concatenate(slabs), slabs[0].nbytes
 
 
@@ -53,7 +55,7 @@ def oracle_expert_matvec(fmt, slab, bpe, ids, xq_rows, in_dim, out_dim, slot_row
         for s in range(n_used):
             e = int(ids[t, s])
             row = xq_rows[t, s if slot_rows else 0]
-            y[t, s] = orc.matvec_q8(fmt, slab[e * bpe:(e + 1) * bpe], in_dim, out_dim, row, 1)[0]
+            y[t, s] = orc.matvec_q8(fmt, slab[e * bpe:e * bpe + orc.repacked_len(fmt, in_dim, out_dim)], in_dim, out_dim, row, 1)[0]
     return y
 
 
@@ -227,17 +229,16 @@ def test_gate_up_swiglu_q8_equals_the_two_launches(in_dim, out_dim, n_tok):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("in_dim,out_dim,n_tok", [(768, 2048, 1), (768, 56, 2), (256, 43, 1), (2048, 64, 1)])
+@pytest.mark.parametrize("in_dim,out_dim,n_tok", [(768, 2048, 1), (768, 56, 2), (768, 43, 1), (2048, 64, 1), (1280, 37, 2)])
 def test_down_combine_equals_the_two_launches(fmt, in_dim, out_dim, n_tok):
     # down projection + weighted combine in one launch: bit for bit the two-launch result
-    # (both team widths: up to 32 sub-blocks half-wavefronts, 2048 the full wavefront)
-    if out_dim % 8 and fmt != rein.Q8_0:
-        out_dim += 8 - out_dim % 8          # slabs must stay 16-byte aligned
+    # (both team widths: up to 32 sub-blocks half-wavefronts, 2048 the full wavefront; the odd
+    # row counts end on a workgroup that owns a single row -- their slabs are padded to the
+    # 16-byte stride the library asks for)
     n_expert, n_used = 12, 8
     rng = np.random.default_rng(in_dim * 5 + out_dim + fmt)
-    slab, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=fmt * 100 + 77)
-    if bpe % 16:
-        pytest.skip("expert slab not 16-byte aligned at this shape")
+    slab, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=fmt * 100 + 77, pad16=True)
+    assert bpe % 16 == 0
     ids = np.stack([rng.permutation(n_expert)[:n_used] for _ in range(n_tok)]).astype(np.int32)
     wts = rng.random((n_tok, n_used)).astype(np.float32)
     scales = (0.5 + rng.random(n_expert)).astype(np.float32)

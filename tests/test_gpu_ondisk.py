@@ -29,8 +29,7 @@ def gpu():
     hip.synchronize()
 
 
-def dev(a):
-    return hip.DeviceBuf.from_host(np.ascontiguousarray(a))
+from helpers import dev  # noqa: E402  (uploads that stay alive until the test's last launch has finished)
 
 
 def gpu_quantize(x):

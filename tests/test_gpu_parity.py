@@ -34,8 +34,7 @@ def gpu():
     hip.synchronize()
 
 
-def dev(a):
-    return hip.DeviceBuf.from_host(a)
+from helpers import dev  # noqa: E402  (uploads that stay alive until the test's last launch has finished)
 
 
 def make_weights(fmt, in_dim, out_dim, seed, gaussian=False):

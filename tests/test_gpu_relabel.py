@@ -22,8 +22,7 @@ def gpu():
     hip.synchronize()
 
 
-def dev(a):
-    return hip.DeviceBuf.from_host(np.ascontiguousarray(a))
+from helpers import dev  # noqa: E402  (uploads that stay alive until the test's last launch has finished)
 
 
 def slabs(fmt, in_dim, out_dim, n_expert, seed):
