@@ -288,6 +288,16 @@ size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                     unsigned out_dim, unsigned p_rows, void *workspace, size_t workspace_bytes,
                     rein_stream_t s);
+/* rein_mmq_xq8_ws without the workspace argument and without any allocation, for callers that
+ * cannot allocate device memory: code under graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  The workspace is a fixed array of
+ * 8 MiB in device memory that every GPU the process uses holds until the process ends
+ * (librein_scratch.so, loaded from the directory of librein.so on the first call).  Shapes whose
+ * rein_mmq_workspace_bytes exceeds 8 MiB are refused with REIN_E_TOO_LARGE (at in_dim 5120
+ * that is above 768 rows); shapes that need no workspace run rein_mmq_xq8.  All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+int rein_mmq_xq8_noalloc(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
+                         unsigned out_dim, unsigned p_rows, rein_stream_t s);
 /* How rein_mmq_xq8_ws cuts the tokens of a 128-row block: n4 groups of four 32-token tiles,
  * n2 groups of two, single tiles for the rest.  No counterpart in the reference. */
 int rein_mmq_tile_plan_ws(int fmt, unsigned out_dim, unsigned p_rows, unsigned *n4, unsigned *n2);

@@ -738,6 +738,51 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
     return launch("rein_mmq6_q4k_mix", (unsigned)grid, 1, 1, 256, mmq6_lds_bytes(n4 ? 4 : n2 ? 2 : 1), s, a);
 }
 
+// ---- the entry point that allocates nothing
+namespace {
+typedef int (*static_scratch_fn)(void**, size_t*);
+std::mutex g_scratch_mu;
+static_scratch_fn g_scratch_fn = nullptr;
+
+// librein_scratch.so (host/static_scratch.hip) next to this library: loaded on first use
+int static_scratch(void** ptr, size_t* bytes)
+{
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        if (!g_scratch_fn) {
+            std::string path = default_hsaco_path();
+            const size_t slash = path.find_last_of('/');
+            path = (slash == std::string::npos ? std::string(".") : path.substr(0, slash)) + "/librein_scratch.so";
+            void* h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
+            if (!h) {
+                const char* err = dlerror();
+                return fail(REIN_E_NOT_LOADED, "rein_mmq_xq8_noalloc: cannot load " + path + ": " + (err ? err : "unknown error"));
+            }
+            g_scratch_fn = reinterpret_cast<static_scratch_fn>(dlsym(h, "rein_static_scratch"));
+            if (!g_scratch_fn) return fail(REIN_E_NOT_LOADED, "rein_mmq_xq8_noalloc: " + path + " does not export rein_static_scratch");
+        }
+    }
+    const int e = g_scratch_fn(ptr, bytes);
+    if (e != 0) return check_hip(g_rt.api, (hipError_t)e, "hipGetSymbolAddress(scratch)");
+    return 0;
+}
+}  // namespace
+
+int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                         unsigned p_rows, rein_stream_t s)
+{
+    if (int rc = need_runtime()) return rc;
+    const size_t need = rein_mmq_workspace_bytes(fmt, in_dim, p_rows);
+    if (need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);      // that launch has no scratch
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    if (int rc = static_scratch(&ptr, &bytes)) return rc;
+    if (need > bytes)
+        return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8_noalloc: this shape needs " + std::to_string(need) + " bytes of scratch, the fixed array holds " +
+                                          std::to_string(bytes) + "; use rein_mmq_xq8_ws with a workspace of your own");
+    return rein_mmq_xq8_ws(fmt, w, xq, y, in_dim, out_dim, p_rows, ptr, bytes, s);
+}
+
 int rein_mmq_tile_plan_ws(int fmt, unsigned out_dim, unsigned p_rows, unsigned* n4, unsigned* n2)
 {
     if (!n4 || !n2) return fail(REIN_E_BAD_POINTER, "rein_mmq_tile_plan_ws: NULL output");

@@ -87,6 +87,11 @@ def mmq_xq8_ws(fmt, w, xq, y, in_dim, out_dim, p_rows, workspace, workspace_byte
                               _s(stream)))
 
 
+def mmq_xq8_noalloc(fmt, w, xq, y, in_dim, out_dim, p_rows, stream=None):
+    """mmq_xq8_ws on the library's fixed 8 MiB device array: allocates nothing"""
+    check(lib.rein_mmq_xq8_noalloc(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _s(stream)))
+
+
 def mmq_tile_plan_ws(fmt, out_dim, p_rows):
     """(n4, n2): token groups of four and of two 32-token tiles per 128-row block in mmq_xq8_ws"""
     n4, n2 = C.c_uint(0), C.c_uint(0)
