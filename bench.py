@@ -15,9 +15,12 @@ ONE JSON line.
 
 The same line carries the per-shape figures, the roofline object of the dominant
 kernel (the gate+up launch), the MMQ prefill GEMM (Q4_K, 512 x 5120 x 17408) in
-"mmq" and the CPU baseline (the oracle's restatement of the reference CPU path:
-dequantize once, then the f32 matvec of src/cpu/ops.rs:108-140 over the host
-cores) timed on a bounded sample.
+"mmq", one compact object per remaining BASELINE configuration in "configs"
+(configs[2]: Q4_K / Q6_K / Q8_0 x M 128 / 512 / 2048; configs[3]: the MoE expert FFN;
+configs[4]: the 64-layer decode weight stream under one hipGraph) and the CPU baseline
+(the oracle's restatement of the reference CPU path: dequantize once, then the f32
+matvec of src/cpu/ops.rs:108-140 over the host cores, plus the int8 restatement of
+the kernel formulas on one and on all cores) timed on a bounded sample.
 """
 import argparse
 import json
@@ -137,43 +140,71 @@ class MmqCase:
         runtime.quantize_q8(self.dx, self.dq, in_dim, p_rows, stream)
         stream.synchronize()
         self.ops = 2.0 * p_rows * in_dim * out_dim      # reference convention, kernels.rs:2917
+        # the workspace launch (activation operand image + GEMM) where the format has one
+        self.ws_bytes = runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
+        self.ws = hip.DeviceBuf(self.ws_bytes) if self.ws_bytes else None
+
+    def launch(self, i):
+        runtime.mmq_xq8_ws(self.fmt, self.weights[i % self.n_buf], self.dq, self.dy, self.in_dim, self.out_dim,
+                           self.p, self.ws, self.ws_bytes, self.stream)
 
     def time(self, launches, warmup):
         for i in range(warmup):
-            runtime.mmq_xq8(self.fmt, self.weights[i % self.n_buf], self.dq, self.dy, self.in_dim, self.out_dim,
-                            self.p, self.stream)
+            self.launch(i)
         self.stream.synchronize()
         e0, e1 = hip.Event(), hip.Event()
         e0.record(self.stream)
         for i in range(launches):
-            runtime.mmq_xq8(self.fmt, self.weights[i % self.n_buf], self.dq, self.dy, self.in_dim, self.out_dim,
-                            self.p, self.stream)
+            self.launch(i)
         e1.record(self.stream)
         e1.synchronize()
         return e0.elapsed_ms(e1) * 1e-3 / launches
 
 
-def cpu_baseline(fmt, in_dim, out_dim, seed, budget_s=12.0):
-    """The reference CPU path (dequantize once, untimed; then f32 matvec over all
-    cores) on the headline shape, repeated for about `budget_s` seconds."""
-    from oracle import orc          # the checker, used here only as the timed CPU baseline
+def cpu_threads():
+    """Threads for the CPU legs: the CPU share the box grants this job (OMP_NUM_THREADS where it
+    is set -- 16 on a one-GPU box, whatever the host's core count), else every core."""
+    host = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    return (max(1, min(int(env), host)) if env and env.isdigit() else host), host
 
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else int(os.environ["OMP_NUM_THREADS"])
-    raw, _ = synth_weights(fmt, in_dim, out_dim, seed)
-    w = orc.dequantize_to_f32(fmt, raw, in_dim * out_dim).reshape(out_dim, in_dim)
-    x = np.random.default_rng(seed + 1).standard_normal(in_dim).astype(np.float32)
-    orc.matvec_f32(x, w, n_threads=cores)
+
+def best_of(fn, budget_s, max_reps=2000):
+    fn()
     best, reps, t_start = 1e30, 0, time.perf_counter()
-    while time.perf_counter() - t_start < budget_s and reps < 2000:
+    while time.perf_counter() - t_start < budget_s and reps < max_reps:
         t0 = time.perf_counter()
-        orc.matvec_f32(x, w, n_threads=cores)
+        fn()
         best = min(best, time.perf_counter() - t0)
         reps += 1
-    return {"value": round(matvec_bytes(fmt, in_dim, out_dim, 1) / best / 1e9, 3), "unit": "GB/s",
-            "cores": cores, "kind": "port",
-            "sample": f"dequantize_to_f32 once (untimed) + f32 matvec {in_dim}->{out_dim}, best of {reps} runs, "
-                      f"algorithmic (repacked) bytes / time; {round(in_dim * out_dim * 4 / best / 1e9, 2)} GB/s of f32 traffic"}
+    return best, reps
+
+
+def cpu_baseline(fmt, in_dim, out_dim, seed, budget_s=10.0):
+    """The reference CPU path (dequantize once, untimed; then the f32 matvec of
+    src/cpu/ops.rs:108-140 over the granted cores) on the headline shape, and beside it the
+    int8 restatement of the kernel formulas (quantized activations against the repacked
+    weights) on one thread and on all of them; each leg repeats for a bounded time."""
+    from oracle import orc          # the checker, used here only as the timed CPU baseline
+
+    cores, host = cpu_threads()
+    raw, packed = synth_weights(fmt, in_dim, out_dim, seed)
+    w = orc.dequantize_to_f32(fmt, raw, in_dim * out_dim).reshape(out_dim, in_dim)
+    x = np.random.default_rng(seed + 1).standard_normal(in_dim).astype(np.float32)
+    nbytes = matvec_bytes(fmt, in_dim, out_dim, 1)
+    best, reps = best_of(lambda: orc.matvec_f32(x, w, n_threads=cores), budget_s * 0.5)
+    xq = orc.quantize_q8(x[None, :])
+    i1, r1 = best_of(lambda: orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, 1, n_threads=1), budget_s * 0.25, 200)
+    ia, ra = best_of(lambda: orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, 1, n_threads=cores), budget_s * 0.25)
+    return {"value": round(nbytes / best / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "host_hardware_concurrency": host,
+            "sample": f"dequantize_to_f32 once (untimed) + f32 matvec {in_dim}->{out_dim} on {cores} threads (the CPU share "
+                      f"of this job; the host reports {host}), best of {reps} runs, algorithmic (repacked) bytes / time; "
+                      f"{round(in_dim * out_dim * 4 / best / 1e9, 2)} GB/s of f32 traffic",
+            "int8_restatement": {"unit": "GB/s", "threads_1": round(nbytes / i1 / 1e9, 3), "runs_1": r1,
+                                 f"threads_{cores}": round(nbytes / ia / 1e9, 3), "runs_all": ra,
+                                 "sample": f"oracle int8 matvec (BlockQ8 x repacked {FMT_NAME[fmt]}) {in_dim}->{out_dim}, "
+                                           "best run, same algorithmic bytes"}}
 
 
 def tiled_weights(fmt, in_dim, out_dim, seed, base_rows=512):
@@ -205,10 +236,13 @@ def time_graph(stream, launch_all, n_launches, steps=5):
     return e0.elapsed_ms(e1) * 1e-3 / (steps * n_launches)
 
 
-def mmq_kernel_name(fmt, out_dim, p_rows):
-    """the kernel mmq_xq8 launches for this shape (64-token tiles per row block, the rest in 32-token tiles)"""
-    n64 = runtime.mmq_tile_plan(fmt, out_dim, p_rows)
+def mmq_kernel_name(fmt, in_dim, out_dim, p_rows):
+    """the kernels the MMQ launch of this shape runs"""
     tag = {rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k"}.get(fmt, FMT_NAME[fmt])
+    if runtime.mmq_workspace_bytes(fmt, in_dim, p_rows):
+        n4, n2 = runtime.mmq_tile_plan_ws(fmt, out_dim, p_rows)
+        return f"rein_mmq6_prep + rein_mmq6_{tag}_mix (n4 = {n4}, n2 = {n2})"
+    n64 = runtime.mmq_tile_plan(fmt, out_dim, p_rows)
     return f"rein_mmq_{tag}_mix (n64 = {n64})" if n64 else f"rein_mmq_{tag}_t32"
 
 
@@ -223,12 +257,14 @@ def extras_mmq(stream):
             x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
             dx, dq, dy = hip.DeviceBuf.from_host(x), hip.DeviceBuf(m * (k // 32) * 40), hip.DeviceBuf(m * n * 4)
             runtime.quantize_q8(dx, dq, k, m, stream)
-            sec = time_graph(stream, lambda: [runtime.mmq_xq8(f, w_, dq, dy, k, n, m, stream) for w_ in ws], len(ws))
+            wsb = runtime.mmq_workspace_bytes(f, k, m)
+            wsp = hip.DeviceBuf(wsb) if wsb else None
+            sec = time_graph(stream, lambda: [runtime.mmq_xq8_ws(f, w_, dq, dy, k, n, m, wsp, wsb, stream) for w_ in ws], len(ws))
             tops = 2.0 * m * k * n / sec / 1e12
             out.append({"fmt": FMT_NAME[f], "M": m, "us": round(sec * 1e6, 1), "TOPS": round(tops, 1),
                         "frac_int8_peak": round(tops / INT8_PEAK_TOPS, 4)})
             log("mmq", out[-1])
-            del dx, dq, dy
+            del dx, dq, dy, wsp
         del ws
     return out
 
@@ -259,7 +295,7 @@ def extras_moe(stream):
     res = {"workload": "MoE expert FFN, 512 tok x 128 experts top-8, hidden 2048, ff 768 (Q4_K gate/up, Q6_K down)",
            "us": round(sec * 1e6, 1), "weight_GBs": round(weight_bytes / sec / 1e9, 0),
            "frac_hbm_peak": round(weight_bytes / sec / 1e9 / HBM_PEAK_GBS, 4), "TOPS": round(ops / sec / 1e12, 1),
-           "weight_bytes": weight_bytes,
+           "frac_int8_peak": round(ops / sec / 1e12 / INT8_PEAK_TOPS, 4), "weight_bytes": weight_bytes,
            "note": "the 401 MB of expert weights are re-read from the 256 MB Infinity Cache + HBM on every repetition"}
     log("moe", res)
     return res
@@ -503,8 +539,10 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="also time the format x shape x batch sweep of configs[1]")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mmq", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the objects of BASELINE configs[2..4] (MMQ formats x M, MoE expert FFN, decode weight stream)")
     ap.add_argument("--extras", action="store_true",
-                    help="also time BASELINE configs[2..4]: MMQ formats x M, the MoE expert FFN, the decode weight stream")
+                    help="also time the fused producers, the MoE decode path, the remaining matvec sites and the decode FFN chain")
     ap.add_argument("--fmt", default="q4_k")
     ap.add_argument("--batch", type=int, default=1)
     args = ap.parse_args()
@@ -562,6 +600,8 @@ def main():
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2), "shapes": shapes},
         "roofline": {"bound": "hbm", "achieved": dom["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": dom["frac_of_hbm_peak"], "traffic": DOMINANT_TRAFFIC_BYTES if is_headline else None,
+                     "traffic_source": "recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file "
+                                       "(profiles/rein_mv_q4k_b1_decode_shapes.txt), not read in this run" if is_headline else None,
                      "kernel": "rein_mv_q4k_r4_b1 (K=5120 -> N=34816)", "us_per_launch": dom["us_per_launch"],
                      "algorithmic_bytes_per_launch": dom["bytes_per_launch"]},
     }
@@ -593,8 +633,12 @@ def main():
                       "us_per_launch": round(sec * 1e6, 2), "value": round(tops, 2), "unit": "int8 TOPS",
                       "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                    "frac": round(tops / INT8_PEAK_TOPS, 4),
-                                   "kernel": mmq_kernel_name(rein.Q4_K, 17408, 512)}}
+                                   "kernel": mmq_kernel_name(rein.Q4_K, 5120, 17408, 512)}}
         del mm
+
+    if not args.no_configs:
+        out["configs"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
+                          "decode_stream_configs4": extras_decode_stream(stream)}
 
     if args.sweep:
         sweep = []
@@ -612,8 +656,7 @@ def main():
         out["sweep"] = sweep
 
     if args.extras:
-        out["extras"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
-                         "decode_stream_configs4": extras_decode_stream(stream), "fused_producers": extras_fused(stream),
+        out["extras"] = {"fused_producers": extras_fused(stream),
                          "moe_decode": extras_moe_decode(stream), "other_matvec_sites": extras_ondisk(stream),
                          "decode_ffn_chain": extras_decode_ffn(stream)}
 
