@@ -274,9 +274,9 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
 }
 
 // Grouped GEMM launch.  The tile count lives on the device; the grid covers its upper bound
-// (qwen35.rs:3051).  One tile per workgroup (rein_mmq_<fmt>_grouped_t32, grid.z = 2 when a
-// second slab / output pair is given) as long as that bound fits grid.y; beyond it the
-// reference-named kernel, which strides over tiles, once per slab.
+// (qwen35.rs:3051).  One tile per workgroup (rein_mmq_<fmt>_grouped_t32, both slabs in one
+// launch when a second slab / output pair is given) as long as that bound fits a 1-D grid;
+// beyond it the reference-named kernel, which strides over tiles, once per slab.
 int launch_grouped(int fmt, const void* slab0, const void* slab1, unsigned bytes_per_expert, const int32_t* expert_off,
                    const int32_t* tile_off, unsigned n_expert, const void* xq, float* y0, float* y1, unsigned in_dim,
                    unsigned out_dim, unsigned n_entries, rein_stream_t s)
@@ -284,12 +284,14 @@ int launch_grouped(int fmt, const void* slab0, const void* slab1, unsigned bytes
     const unsigned bn = rein_moe_gemm_bn();
     const unsigned tile_ub = (n_entries + bn - 1) / bn + n_expert;
     const unsigned gx = (out_dim + 127) / 128;
-    if (tile_ub <= 65535 && env_u("REIN_GROUPED_STRIDED", 0) == 0) {
+    const unsigned n_slab = slab1 ? 2 : 1;
+    const unsigned long long grid = 8ull * ((tile_ub + 7) / 8) * n_slab * gx;
+    if (grid <= 0x7FFFFFFFull && env_u("REIN_GROUPED_STRIDED", 0) == 0) {
         const void* s1 = slab1 ? slab1 : slab0;
         float* o1 = y1 ? y1 : y0;
         void* a[] = {(void*)&slab0, (void*)&s1, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off,
-                     (void*)&n_expert, (void*)&xq, (void*)&y0, (void*)&o1, (void*)&in_dim, (void*)&out_dim};
-        return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_grouped_t32", gx, tile_ub, slab1 ? 2 : 1, 256, 0, s, a);
+                     (void*)&n_expert, (void*)&xq, (void*)&y0, (void*)&o1, (void*)&in_dim, (void*)&out_dim, (void*)&n_slab};
+        return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_grouped_t32", (unsigned)grid, 1, 1, 256, 0, s, a);
     }
     const std::string name = std::string("mmq_gemm_") + fmt_tag(fmt) + "_grouped_f32";
     for (int z = 0; z < (slab1 ? 2 : 1); z++) {
@@ -641,10 +643,13 @@ size_t x6_image_bytes(unsigned n_sub, unsigned p_rows)
     return (size_t)((n_sub + 1) / 2) * ((p_rows + 31) / 32) * kX6Rec + 1024;      // rein_x6_bytes
 }
 bool mmq6_format(int fmt) { return fmt == REIN_TYPE_Q4_K && env_u("REIN_MMQ6", 1) != 0; }
-unsigned mmq6_lds_bytes(unsigned nt)       // rein_mmq6_lds_bytes<NT>()
+unsigned mmq6_lds_bytes(unsigned nt)       // rein_mmq6_lds_bytes<NT>(), depths of Mmq6Cfg<NT>
 {
-    return 3 * ((nt * kX6Rec + 1023u) & ~1023u) + 4 * 4096 + 4 * 1280;
+    const unsigned r = nt == 4 ? 2 : nt == 2 ? 4 : 3, d = nt == 4 ? 3 : 4, sm = nt == 2 ? 2 : 1;
+    return d * ((nt * kX6Rec + 1023u) & ~1023u) + 4 * r * 2048 + 4 * sm * 1280;
 }
+// a launch whose workgroups run tiles of several widths holds the largest layout
+unsigned mmq6_lds_max() { return std::max(mmq6_lds_bytes(4), std::max(mmq6_lds_bytes(2), mmq6_lds_bytes(1))); }
 // Token groups per 128-row block: n4 groups of four 32-token tiles, n2 of two, the rest single.
 // Relative cost of a workgroup per 32-token tile, fitted to a sweep of the splits of 512 x 5120
 // x 17408: 1.00 in a group of four, 1.15 in a group of two, 1.8 alone (the weight unpack is
@@ -662,8 +667,10 @@ void mmq6_pick(unsigned out_dim, unsigned p_rows, unsigned* n4_out, unsigned* n2
         return;
     }
     const unsigned a4 = n_tt / 4, rest = n_tt - 4 * a4;
-    *n4_out = a4; *n2_out = rest / 2;                          // very large grids: granularity no longer matters
-    if ((unsigned long long)n_rb * n_tt > 64ull * kCUs) return;
+    *n4_out = a4; *n2_out = rest / 2;
+    // from about three rounds of wide workgroups the grain no longer matters (2048 x 17408: all
+    // wide 591 us, the split the walk below prefers 611 us)
+    if ((unsigned long long)n_rb * a4 > 6ull * kCUs) return;
     static std::mutex mu;
     static std::unordered_map<unsigned long long, unsigned> memo;
     const unsigned long long key = ((unsigned long long)out_dim << 32) | p_rows;
@@ -735,7 +742,7 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
     if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, std::string(who) + ": too many tiles for one launch");
     if (int rc = mmq6_prep(xq, workspace, in_dim / 32, p_rows, s)) return rc;
     void* a[] = {(void*)&w, (void*)&workspace, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&n4, (void*)&n2};
-    return launch("rein_mmq6_q4k_mix", (unsigned)grid, 1, 1, 256, mmq6_lds_bytes(n4 ? 4 : n2 ? 2 : 1), s, a);
+    return launch("rein_mmq6_q4k_mix", (unsigned)grid, 1, 1, 256, mmq6_lds_max(), s, a);
 }
 
 // ---- the entry point that allocates nothing
@@ -1254,7 +1261,7 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     }
     // the expert-sorted BlockQ8 rows straight from x (quantize_q8 + moe_gather_xq in one launch)
     if (int rc = rein_moe_quantize_scatter(x, inv, base + w.g_in, sh.hidden, sh.n_used, sh.n_tok, s)) return rc;
-    // gate and up projections in one launch (grid.z = 2)
+    // gate and up projections in one launch (two slabs)
     if (int rc = launch_grouped(sh.gate_up_fmt, gate_exps, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert, base + w.g_in,
                                 (float*)(base + w.e_gate), (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;
     // SwiGLU straight into the down projection's BlockQ8 rows (rows are expert_ff long,

@@ -81,18 +81,12 @@ __host__ __device__ constexpr size_t rein_x6_bytes(unsigned n_sub, unsigned p_ro
     return (size_t)((n_sub + 1u) / 2u) * ((p_rows + 31u) / 32u) * REIN_X6_REC + 1024u;   // + slack, see issue_acts
 }
 
-// xq [p_rows][n_sub] BlockQ8 -> X6 image.  One lane per (token, sub-block): the eight lanes
-// of a token read eight consecutive blocks (320 contiguous bytes); blockIdx.x = token tile,
-// blockIdx.y = group of 8 sub-blocks (4 pairs), 256 threads.
-__device__ __forceinline__ void rein_mmq6_prep_body(const BlockQ8* __restrict__ xq, uint8_t* __restrict__ img,
-                                                    unsigned n_sub, unsigned p_rows)
+// One lane's share of the image: BlockQ8 block `sb` of row `tok` of xq (ok: the row and the
+// block exist) goes into token slot j of record `rec`; n_rec = records per sub-block pair.
+__device__ __forceinline__ void rein_mmq6_prep_lane(const BlockQ8* __restrict__ xq, uint8_t* __restrict__ img,
+                                                    unsigned n_sub, unsigned n_rec, unsigned rec, unsigned j,
+                                                    unsigned sb, unsigned tok, bool ok)
 {
-    const unsigned n_tt = (p_rows + 31u) / 32u;
-    const unsigned tt = blockIdx.x;
-    const unsigned j = threadIdx.x >> 3, s8 = threadIdx.x & 7u;
-    const unsigned sb = blockIdx.y * 8u + s8, tok = tt * 32u + j;
-    if (tt >= n_tt || sb >= ((n_sub + 1u) & ~1u)) return;
-    const bool ok = tok < p_rows && sb < n_sub;
     float d = 0.0f, xs = 0.0f;
     int q[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (ok) {
@@ -112,17 +106,31 @@ __device__ __forceinline__ void rein_mmq6_prep_body(const BlockQ8* __restrict__ 
         hi[wd] |= ch << sh; lo[wd] |= cl << sh;
         if (sh > 26) { hi[wd + 1] |= ch >> (32 - sh); lo[wd + 1] |= cl >> (32 - sh); }
     }
-    uint8_t* rec = img + ((size_t)(sb >> 1) * n_tt + tt) * REIN_X6_REC;
-    uint8_t* a = rec + (sb & 1u) * 1536u;
+    uint8_t* r = img + ((size_t)(sb >> 1) * n_rec + rec) * REIN_X6_REC;
+    uint8_t* a = r + (sb & 1u) * 1536u;
     *reinterpret_cast<uint4*>(a + j * 16u)          = make_uint4(hi[0], hi[1], hi[2], hi[3]);
     *reinterpret_cast<uint4*>(a + 512u + j * 16u)   = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     *reinterpret_cast<uint2*>(a + 1024u + j * 8u)   = make_uint2(hi[4], hi[5]);
     *reinterpret_cast<uint2*>(a + 1280u + j * 8u)   = make_uint2(lo[4], lo[5]);
-    *reinterpret_cast<float*>(rec + 3072u + (sb & 1u) * 128u + j * 4u) = ok ? d : 0.0f;
+    *reinterpret_cast<float*>(r + 3072u + (sb & 1u) * 128u + j * 4u) = ok ? d : 0.0f;
     uint16_t sp[3];
     rein_mmq_split_xsum(ok ? xs : 0.0f, sp);
     const uint32_t x0 = sp[0], x1 = sp[1], x2 = sp[2];
-    *reinterpret_cast<uint4*>(rec + 3328u + (sb & 1u) * 512u + j * 16u) = make_uint4(x0 | (x0 << 16), x1 | (x0 << 16), x1 | (x2 << 16), 0u);
+    *reinterpret_cast<uint4*>(r + 3328u + (sb & 1u) * 512u + j * 16u) = make_uint4(x0 | (x0 << 16), x1 | (x0 << 16), x1 | (x2 << 16), 0u);
+}
+
+// xq [p_rows][n_sub] BlockQ8 -> X6 image.  One lane per (token, sub-block): the eight lanes
+// of a token read eight consecutive blocks (320 contiguous bytes); blockIdx.x = token tile,
+// blockIdx.y = group of 8 sub-blocks (4 pairs), 256 threads.
+__device__ __forceinline__ void rein_mmq6_prep_body(const BlockQ8* __restrict__ xq, uint8_t* __restrict__ img,
+                                                    unsigned n_sub, unsigned p_rows)
+{
+    const unsigned n_tt = (p_rows + 31u) / 32u;
+    const unsigned tt = blockIdx.x;
+    const unsigned j = threadIdx.x >> 3, s8 = threadIdx.x & 7u;
+    const unsigned sb = blockIdx.y * 8u + s8, tok = tt * 32u + j;
+    if (tt >= n_tt || sb >= ((n_sub + 1u) & ~1u)) return;
+    rein_mmq6_prep_lane(xq, img, n_sub, n_tt, tt, j, sb, tok, tok < p_rows && sb < n_sub);
 }
 
 // ---- DMA helpers ----------------------------------------------------------------------
@@ -139,60 +147,110 @@ __device__ __forceinline__ void rein_lds_dma_u32(const void* gptr, unsigned lds_
 
 // ---- the tile -------------------------------------------------------------------------
 // LDS of one workgroup (4 wavefronts, 128 weight rows x 32 NT tokens):
-//   acts   3 x NT x 4352   activation records of three consecutive sub-block pairs
-//   ring   4 x 2 x 2048    per wavefront: two slots of 4 sub-blocks x 32 rows x 16 B (MmqWLds)
-//   small  4 x 1280        per wavefront: (sc, m) of the superblock [row][8] as dwords, then
-//                          (d, dmin) [row]
+//   acts   D x NT x 4352       activation records of D consecutive sub-block pairs
+//   ring   4 x R x 2048        per wavefront: R slots of 4 sub-blocks x 32 rows x 16 B
+//   small  4 x S x 1280        per wavefront: S buffers of (sc, m) of a superblock [row][8] as
+//                              dwords, then (d, dmin) [row]
+// The depths set how far ahead of their use the transfers are requested: D - 1 pair-steps for
+// the records, R - 1 ring stages (2 pair-steps each) for the weights, 4 S - 2 pair-steps for
+// the small words.  A pair-step of a 4-tile group computes for about a microsecond, which covers
+// the memory latency at the shallowest depths; the narrow groups (and the short contractions
+// of expert FFNs, whose weights come from HBM once) need the weights several stages ahead.
+template <int NT> struct Mmq6Cfg;
+template <> struct Mmq6Cfg<4> { static constexpr int R = 2, D = 3, S = 1; };
+template <> struct Mmq6Cfg<2> { static constexpr int R = 4, D = 4, S = 2; };
+template <> struct Mmq6Cfg<1> { static constexpr int R = 3, D = 4, S = 1; };
+
 template <int NT>
 constexpr unsigned rein_mmq6_act_stride() { return (NT * REIN_X6_REC + 1023u) & ~1023u; }   // whole 1 KiB transfers
 template <int NT>
-constexpr int rein_mmq6_lds_bytes() { return 3 * (int)rein_mmq6_act_stride<NT>() + 4 * (int)sizeof(MmqWLds<REIN_Q4_K>) + 4 * 1280; }
+constexpr int rein_mmq6_lds_bytes()
+{
+    return Mmq6Cfg<NT>::D * (int)rein_mmq6_act_stride<NT>() + 4 * Mmq6Cfg<NT>::R * 2048 + 4 * Mmq6Cfg<NT>::S * 1280;
+}
 
 // All global -> LDS traffic of the loop is DMA that the compiler cannot see; the waits are
 // placed by hand and count exactly the transfers below.  Per pair-step i (one pair of
 // sub-blocks), every wavefront issues, in this order:
-//   acts(i + 2)                     kActDma transfers   into buffer (i + 2) % 3
-//   i % 2 == 0: ring(i / 2 + 1)     2 transfers         into slot (i / 2 + 1) & 1
-//   i % 4 == 2: small(i / 4 + 1)    5 transfers         into the small buffer (read at i % 4 == 0 only)
-// and at the top of step i everything issued in step i - 2 must have landed, i.e. at most
-// the transfers of step i - 1 may be in flight.  Past the end of the contraction the same
-// transfers are issued on clamped addresses into buffers nobody reads again, which keeps
+//   acts(i + D - 1)                     K transfers   into record buffer (i + D - 1) % D
+//   i % 2 == 0: ring(i / 2 + R - 1)     2 transfers   into slot (i / 2 + R - 1) % R
+//   i % 4 == 2: small(i / 4 + S)        5 transfers   into small buffer (i / 4) % S (last read in this step)
+// Transfers complete in order, so "X has landed" is "at most as many transfers are in flight as
+// were issued after X".  At the top of step i the step needs acts(i), at even i the ring stage
+// i / 2, at i % 4 == 0 the small words of chunk i / 4; Mmq6Waits counts what was issued after the
+// oldest of those, per i % 4.  The prologue issues everything the first steps need and drains
+// it, so the counts of the steady state hold from step 0.  Past the end of the contraction the
+// same transfers are issued on clamped addresses into buffers nobody reads again, which keeps
 // the counts uniform; the kernel drains them before it ends.
+template <int K, int R, int D, int S>
+struct Mmq6Waits {
+    static constexpr int ring(int s) { return s % 2 == 0 ? 2 : 0; }
+    static constexpr int small(int s) { return s % 4 == 2 ? 5 : 0; }
+    static constexpr int cnt(int s) { return K + ring(s) + small(s); }
+    static constexpr int sum(int a, int b) { int t = 0; for (int s = a; s <= b; s++) t += cnt(s); return t; }
+    static constexpr int at(int r)                 // r = i % 4; the step is taken as r + 64 (period 4)
+    {
+        const int i = r + 64;
+        int n = ring(i - D + 1) + small(i - D + 1) + sum(i - D + 2, i - 1);                    // after acts(i)
+        if (r % 2 == 0) {
+            const int m = small(i - 2 * R + 2) + sum(i - 2 * R + 3, i - 1);                    // after ring(i / 2)
+            n = m < n ? m : n;
+        }
+        if (r == 0) {
+            const int m = sum(i - 4 * S + 3, i - 1);                                           // after small(i / 4)
+            n = m < n ? m : n;
+        }
+        return n;
+    }
+};
+
+// The records and the rows of xq / y that one workgroup covers.
+struct Mmq6Span {
+    unsigned n_rec;      // records per sub-block pair in the image
+    unsigned rec0;       // first record of this workgroup
+    unsigned rec_cnt;    // records that exist from rec0 on (>= 1); min(NT, rec_cnt) are computed
+    unsigned tok_base;   // row of y of token 0 of record rec0; record rec0 + t starts 32 t rows on
+    unsigned tok_end;    // one past the last row of this span
+};
+
 template <int NT, int DOTS>
 __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, const uint8_t* __restrict__ img,
                                                float* __restrict__ y, int* __restrict__ dots, unsigned in_dim,
-                                               unsigned out_dim, unsigned p_rows, unsigned rb, unsigned tt0)
+                                               unsigned out_dim, unsigned rb, const Mmq6Span span)
 {
     constexpr int FMT = REIN_Q4_K;
     using F = Fmt<FMT>;
     constexpr unsigned kActBytes = rein_mmq6_act_stride<NT>();           // LDS buffer of one pair (records + pad)
     constexpr unsigned kActDma = (kActBytes + 4095u) / 4096u;          // transfers per wavefront and pair-step
+    constexpr unsigned R = Mmq6Cfg<NT>::R, D = Mmq6Cfg<NT>::D, S = Mmq6Cfg<NT>::S;
+    using Waits = Mmq6Waits<(int)kActDma, (int)R, (int)D, (int)S>;
+    static_assert(Waits::at(0) < 64 && Waits::at(1) < 64 && Waits::at(2) < 64 && Waits::at(3) < 64, "vmcnt holds 6 bits");
     extern __shared__ __attribute__((aligned(16))) unsigned char rein_mmq6_lds[];
     unsigned char* const raw = rein_mmq6_lds;
     typedef __attribute__((address_space(3))) const void* lptr_t;
 
     const unsigned lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned j = lane & 31u, h = lane >> 5;
-    const unsigned n_sub = in_dim >> 5, n_pair = n_sub >> 1, n_tt = (p_rows + 31u) / 32u;
+    const unsigned n_sub = in_dim >> 5, n_pair = n_sub >> 1, n_tt = span.n_rec, tt0 = span.rec0;
     const F fmt(w, n_sub, out_dim);
     const unsigned row_base = rb * 128u + wave * 32u;
     const unsigned row = row_base + j;
     const unsigned rowc = min(row, out_dim - 1u);
 
-    MmqWLds<FMT>& wl = reinterpret_cast<MmqWLds<FMT>*>(raw + 3 * kActBytes)[wave];
-    const uint32_t* const small = reinterpret_cast<const uint32_t*>(raw + 3 * kActBytes + 4 * sizeof(MmqWLds<FMT>) + wave * 1280u);
+    const uint4* const ring = reinterpret_cast<const uint4*>(raw + D * kActBytes + wave * (R * 2048u));
+    const uint32_t* const small0 = reinterpret_cast<const uint32_t*>(raw + D * kActBytes + 4u * R * 2048u + wave * (S * 1280u));
     const unsigned lds_acts = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)raw);
-    const unsigned lds_small = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)small);
-    MmqWSrc<FMT> wsrc;
-    wsrc.init(wl, fmt, row_base, out_dim, lane);
+    const unsigned lds_small = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)small0);
+    MmqWSrc<FMT> wsrc;                               // slot s of the ring is 2048 s bytes on, as rein_mmq_wload addresses it
+    wsrc.init(*reinterpret_cast<const MmqWLds<FMT>*>(ring), fmt, row_base, out_dim, lane);
 
     // activation source: this workgroup's NT records of a pair are contiguous
-    const unsigned tt_cnt = min((unsigned)NT, n_tt - tt0);                 // records that exist (>= 1)
+    const unsigned tt_cnt = min((unsigned)NT, span.rec_cnt);              // records that exist (>= 1)
     const size_t pair_stride = (size_t)n_tt * REIN_X6_REC;
     auto issue_acts = [&](unsigned pair) {
         const unsigned p = min(pair, n_pair - 1u);
         const uint8_t* src = img + (size_t)p * pair_stride + (size_t)tt0 * REIN_X6_REC;
-        const unsigned buf = lds_acts + (pair % 3u) * kActBytes;
+        const unsigned buf = lds_acts + (pair % D) * kActBytes;
 #pragma unroll
         for (unsigned k = 0; k < kActDma; k++) {
             // transfer k of this wavefront covers bytes [off, off + 1024) of the records; one
@@ -206,16 +264,17 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
     };
     auto issue_ring = [&](unsigned stage) {
         const unsigned sb_first = min(stage * 4u, n_sub - 4u);
-        rein_mmq_wload<FMT>(wsrc, stage & 1u, fmt, sb_first, n_sub);
+        rein_mmq_wload<FMT>(wsrc, stage % R, fmt, sb_first, n_sub);
     };
     auto issue_small = [&](unsigned chunk) {
         const unsigned sup = min(chunk, (n_sub >> 3) - 1u);
+        const unsigned dst = lds_small + (chunk % S) * 1280u;
 #pragma unroll
         for (unsigned k = 0; k < 4; k++) {
             const unsigned r = min(row_base + 8u * k + (lane >> 3), out_dim - 1u);
-            rein_lds_dma_u16(fmt.smp + (size_t)r * fmt.nsp + sup * 8u + (lane & 7u), lds_small + k * 256u);
+            rein_lds_dma_u16(fmt.smp + (size_t)r * fmt.nsp + sup * 8u + (lane & 7u), dst + k * 256u);
         }
-        rein_lds_dma_u32(fmt.ddp + (size_t)rowc * fmt.n_super + sup, lds_small + 1024u);
+        rein_lds_dma_u32(fmt.ddp + (size_t)rowc * fmt.n_super + sup, dst + 1024u);
     };
 
     rein_v16f acc[NT];
@@ -231,9 +290,14 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
     for (int v = 0; v < 32; v++) z32[v] = 0.0f;
     const int scale_a = h ? 130 : 134, scale_b = 130;                   // 2^3, 2^7 | 2^3 (E8M0)
 
-    // prologue = steps -2 and -1 of the schedule above
-    issue_acts(0); issue_ring(0); issue_small(0);
-    issue_acts(1);
+    // prologue: everything the steps before the first in-loop requests land need
+#pragma unroll
+    for (unsigned k = 0; k + 1u < D; k++) issue_acts(k);
+#pragma unroll
+    for (unsigned k = 0; k + 1u < R; k++) issue_ring(k);
+#pragma unroll
+    for (unsigned k = 0; k < S; k++) issue_small(k);
+    REIN_WAIT_VMCNT(0);
 
     // Words 4, 5 of the second operand of a pair are addressed through an offset the compiler
     // cannot see through: with a common base it pairs that read with the first operand's in
@@ -246,15 +310,17 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
     const unsigned rot = j >> 1;
 
     for (unsigned i = 0; i < n_pair; i++) {
-        if ((i & 1u) == 0u) REIN_WAIT_VMCNT(kActDma);
-        else if ((i & 3u) == 1u) REIN_WAIT_VMCNT(kActDma + 2);
-        else REIN_WAIT_VMCNT(kActDma + 7);
+        if ((i & 3u) == 0u) REIN_WAIT_VMCNT(Waits::at(0));
+        else if ((i & 3u) == 1u) REIN_WAIT_VMCNT(Waits::at(1));
+        else if ((i & 3u) == 2u) REIN_WAIT_VMCNT(Waits::at(2));
+        else REIN_WAIT_VMCNT(Waits::at(3));
         __syncthreads();
-        issue_acts(i + 2u);
+        issue_acts(i + D - 1u);
         if ((i & 1u) == 0u) {
-            issue_ring((i >> 1) + 1u);
+            issue_ring((i >> 1) + R - 1u);
             // scales of this stage's four sub-blocks from the small buffer
             const unsigned half = (i >> 1) & 1u;                         // which half of the superblock
+            const uint32_t* const small = small0 + ((i >> 2) % S) * 320u;
             const uint32_t dd = small[256 + lane];
             const float d = rein_h2f((uint16_t)(dd & 0xFFFFu)), ndmin = -rein_h2f((uint16_t)(dd >> 16));
 #pragma unroll
@@ -273,12 +339,12 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
             }
             if ((i & 3u) == 2u) {
                 __builtin_amdgcn_s_waitcnt(0xC07F);                      // the small buffer has been read
-                issue_small((i >> 2) + 1u);
+                issue_small((i >> 2) + S);
             }
         }
-        const unsigned char* const act = raw + (i % 3u) * kActBytes;
+        const unsigned char* const act = raw + (i % D) * kActBytes;
         const unsigned q = i & 1u;
-        const uint4* slot = wl.q[0][(i >> 1) & 1u];
+        const uint4* slot = ring + ((i >> 1) % R) * 128u;
         const rein_v8i b0 = rein_fp6_weights(slot[4u * j + ((2u * q + rot) & 3u)]);
         const rein_v8i b1 = rein_fp6_weights(slot[4u * j + ((2u * q + 1u + rot) & 3u)]);
         const float sc = q ? scq[1] : scq[0];
@@ -300,8 +366,8 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
             if constexpr (DOTS != 0) {
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    const unsigned tok = (tt0 + t) * 32u + 8 * (v / 4) + 4 * h + (v % 4);
-                    if (tok < p_rows && row < out_dim) {
+                    const unsigned tok = span.tok_base + t * 32u + 8 * (v / 4) + 4 * h + (v % 4);
+                    if (tok < span.tok_end && row < out_dim) {
                         int* o = dots + ((size_t)tok * out_dim + row) * n_sub + 2u * i;
                         o[0] = (int)d0[v];
                         o[1] = (int)d1[v];
@@ -326,8 +392,8 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
         for (int t = 0; t < NT; t++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const unsigned tok = (tt0 + t) * 32u + 8 * (v / 4) + 4 * h + (v % 4);
-                if (tok < p_rows && row < out_dim) y[(size_t)tok * out_dim + row] = acc[t][v];
+                const unsigned tok = span.tok_base + t * 32u + 8 * (v / 4) + 4 * h + (v % 4);
+                if (tok < span.tok_end && row < out_dim) y[(size_t)tok * out_dim + row] = acc[t][v];
             }
     }
 }
@@ -341,6 +407,12 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
 // with the narrow ones behind them as fillers, the machine drains evenly.  The host picks
 // n4 and n2 (n4 * 4 + n2 * 2 <= token tiles).
 // Grid: 8 * ceil(n_row_blocks / 8) * (n4 + n2 + n1) workgroups of 256 threads, n1 = the rest.
+__device__ __forceinline__ Mmq6Span rein_mmq6_dense_span(unsigned p_rows, unsigned tt0)
+{
+    const unsigned n_tt = (p_rows + 31u) / 32u;
+    return Mmq6Span{n_tt, tt0, n_tt - tt0, tt0 * 32u, p_rows};
+}
+
 __device__ __forceinline__ void rein_mmq6_mixed(const uint8_t* __restrict__ w, const uint8_t* __restrict__ img,
                                                 float* __restrict__ y, unsigned in_dim, unsigned out_dim,
                                                 unsigned p_rows, unsigned n4, unsigned n2)
@@ -352,19 +424,19 @@ __device__ __forceinline__ void rein_mmq6_mixed(const uint8_t* __restrict__ w, c
     unsigned k = blockIdx.x >> 3;
     if (k < n_rbg * n4) {
         const unsigned rb = (k / n4) * 8u + xcd;
-        if (rb < n_rb) rein_mmq6_tile<4, 0>(w, img, y, nullptr, in_dim, out_dim, p_rows, rb, (k % n4) * 4u);
+        if (rb < n_rb) rein_mmq6_tile<4, 0>(w, img, y, nullptr, in_dim, out_dim, rb, rein_mmq6_dense_span(p_rows, (k % n4) * 4u));
         return;
     }
     k -= n_rbg * n4;
     if (k < n_rbg * n2) {
         const unsigned rb = (k / n2) * 8u + xcd;
-        if (rb < n_rb) rein_mmq6_tile<2, 0>(w, img, y, nullptr, in_dim, out_dim, p_rows, rb, 4u * n4 + (k % n2) * 2u);
+        if (rb < n_rb) rein_mmq6_tile<2, 0>(w, img, y, nullptr, in_dim, out_dim, rb, rein_mmq6_dense_span(p_rows, 4u * n4 + (k % n2) * 2u));
         return;
     }
     k -= n_rbg * n2;
     if (n1 == 0u) return;
     const unsigned rb = (k / n1) * 8u + xcd;
-    if (rb < n_rb) rein_mmq6_tile<1, 0>(w, img, y, nullptr, in_dim, out_dim, p_rows, rb, 4u * n4 + 2u * n2 + k % n1);
+    if (rb < n_rb) rein_mmq6_tile<1, 0>(w, img, y, nullptr, in_dim, out_dim, rb, rein_mmq6_dense_span(p_rows, 4u * n4 + 2u * n2 + k % n1));
 }
 
 template <int NT, int DOTS>
@@ -377,7 +449,7 @@ __device__ __forceinline__ void rein_mmq6_dense(const uint8_t* __restrict__ w, c
     const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
     const unsigned rb = (k / n_tg) * 8u + xcd, tg = k % n_tg;
     if (rb >= n_rb) return;
-    rein_mmq6_tile<NT, DOTS>(w, img, y, dots, in_dim, out_dim, p_rows, rb, tg * NT);
+    rein_mmq6_tile<NT, DOTS>(w, img, y, dots, in_dim, out_dim, rb, rein_mmq6_dense_span(p_rows, tg * NT));
 }
 
 #define REIN_DEFINE_MMQ6_PREP(name)                                                                 \

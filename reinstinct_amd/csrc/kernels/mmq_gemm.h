@@ -1197,31 +1197,35 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
     }
 }
 
-// The library's own launch of the grouped GEMM: exactly one tile per workgroup --
-// blockIdx.x = 128-row block, blockIdx.y = token tile (the host launches an upper bound of
-// the tile count; surplus workgroups leave at once), blockIdx.z selects one of two slabs
-// with its output, so that the gate and the up projection of an expert FFN run in one
-// launch (twice the workgroups fill the machine better than two launches of half the
-// size, and the second launch's fill / drain disappears).  Without the grid-stride loops
+// The library's own launch of the grouped GEMM: exactly one (token tile, 128-row block, slab)
+// per workgroup of a 1-D grid of 8 * ceil(tile_ub / 8) * n_slab * ceil(out_dim / 128)
+// workgroups (tile_ub = the host's upper bound of the tile count; surplus workgroups leave
+// at once).  Workgroup i runs on XCD i % 8, and all row blocks and slabs of a token tile are
+// dealt to the same XCD, so the tile's activation blocks are pulled into one L2 and re-read
+// there by the others.  Two slabs with their outputs let the gate and the up projection of
+// an expert FFN run in one launch (twice the workgroups fill the machine better than two
+// launches of half the size, and the second launch's fill / drain disappears).  Without the grid-stride loops
 // of rein_mmq_grouped around it the tile keeps to the register budget of three
 // wavefronts per SIMD, which is what hides the pipeline fill of the short contractions
-// of expert FFNs (24 to 64 sub-blocks).  Requires gridDim.x >= ceil(out_dim / 128) and
-// gridDim.y >= tile_off[n_expert].
+// of expert FFNs (24 to 64 sub-blocks).
 template <int FMT>
 __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__ slab0, const uint8_t* __restrict__ slab1,
                                                      unsigned bytes_per_expert, const int* __restrict__ expert_off,
                                                      const int* __restrict__ tile_off, unsigned n_expert,
                                                      const BlockQ8* __restrict__ xq, float* __restrict__ y0,
-                                                     float* __restrict__ y1, unsigned in_dim, unsigned out_dim)
+                                                     float* __restrict__ y1, unsigned in_dim, unsigned out_dim,
+                                                     unsigned n_slab)
 {
-    const unsigned tile = blockIdx.y, rb = blockIdx.x;
-    if (blockDim.x != 256u || rb * 128u >= out_dim || tile >= (unsigned)tile_off[n_expert]) return;
+    const unsigned n_rb = (out_dim + 127u) / 128u, per = n_slab * n_rb;
+    const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
+    const unsigned tile = (k / per) * 8u + xcd, rb = (k % per) % n_rb, z = (k % per) / n_rb;
+    if (blockDim.x != 256u || tile >= (unsigned)tile_off[n_expert]) return;
     const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
     const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
     const unsigned tok_end = (unsigned)expert_off[lo + 1];
     if (tok_base >= tok_end) return;
-    const uint8_t* slab = blockIdx.z ? slab1 : slab0;
-    rein_mmq_pipelined_tile<FMT, 32>(slab + (size_t)lo * bytes_per_expert, xq, blockIdx.z ? y1 : y0, in_dim, out_dim, rb,
+    const uint8_t* slab = z ? slab1 : slab0;
+    rein_mmq_pipelined_tile<FMT, 32>(slab + (size_t)lo * bytes_per_expert, xq, z ? y1 : y0, in_dim, out_dim, rb,
                                      tok_base, min(tok_end, tok_base + 32u));
 }
 
@@ -1276,8 +1280,9 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
         const unsigned char* __restrict__ slab0, const unsigned char* __restrict__ slab1,        \
         unsigned int bytes_per_expert, const int* __restrict__ expert_off,                       \
         const int* __restrict__ tile_off, unsigned int n_expert, const BlockQ8* __restrict__ xq, \
-        float* __restrict__ y0, float* __restrict__ y1, unsigned int in_dim, unsigned int out_dim) \
+        float* __restrict__ y0, float* __restrict__ y1, unsigned int in_dim, unsigned int out_dim, \
+        unsigned int n_slab)                                                                     \
     {                                                                                            \
         rein_mmq_grouped_one<FMT>(slab0, slab1, bytes_per_expert, expert_off, tile_off,          \
-                                  n_expert, xq, y0, y1, in_dim, out_dim);                        \
+                                  n_expert, xq, y0, y1, in_dim, out_dim, n_slab);                \
     }

@@ -5,7 +5,7 @@
 #include "mmq_gemm.h"
 
 REIN_DEFINE_MMQ_GROUPED(mmq_gemm_q5k_grouped_f32, REIN_Q5_K)
-// the library's launch: one tile per workgroup; grid.z = 2 runs gate and up of an expert FFN at once
+// the library's launch: one tile per workgroup; two slabs run gate and up of an expert FFN at once
 REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q5k_grouped_t32, REIN_Q5_K)
 
 // Q5_1 experts: the reference compiles this file a second time with Q5_1_SCALES
