@@ -239,7 +239,11 @@ def time_graph(stream, launch_all, n_launches, steps=5):
 def mmq_kernel_name(fmt, in_dim, out_dim, p_rows):
     """the kernels the MMQ launch of this shape runs"""
     tag = {rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k"}.get(fmt, FMT_NAME[fmt])
-    if runtime.mmq_workspace_bytes(fmt, in_dim, p_rows):
+    ws_bytes = runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
+    form = runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, ws_bytes)
+    if form == 2:
+        return f"rein_mmq6_prep + rein_mmq6_{tag}_sk (split-tail launch) + rein_mmq6_tail_sum"
+    if form == 1:
         n4, n2 = runtime.mmq_tile_plan_ws(fmt, out_dim, p_rows)
         return f"rein_mmq6_prep + rein_mmq6_{tag}_mix (n4 = {n4}, n2 = {n2})"
     n64 = runtime.mmq_tile_plan(fmt, out_dim, p_rows)

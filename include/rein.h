@@ -283,8 +283,21 @@ int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_d
  * (one extra launch), then the GEMM streams them from there.  The reference keeps such
  * scratch in its PrefillGemm object (src/runtime/prefill.rs:479-495); here the caller owns
  * it, so nothing allocates and the call can be captured into a graph.  Calls that share a
- * workspace must be ordered on one stream. */
+ * workspace must be ordered on one stream.
+ * Two sizes: rein_mmq_workspace_min_bytes holds the activation image alone; with
+ * rein_mmq_workspace_bytes (the image and one partial tile per resident workgroup, 32 MiB
+ * more) the GEMM may run as a split-tail launch -- one workgroup per resident slot, whole tiles
+ * in rounds, the tiles left over after the last whole round split along the contraction and
+ * their partial tiles summed in a fixed order by a second launch -- which is what evens out shapes
+ * such as 512 x 17408 whose tiles do not divide over the CUs.  Any size from the minimum on is
+ * accepted; below the full size the GEMM runs its one-tile-group-per-workgroup launch.  Results
+ * of the two launches can differ in the order of fp32 additions across superblocks (both within
+ * the parity bar); each is reproducible from run to run. */
 size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows);
+size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
+/* Which launch rein_mmq_xq8_ws takes for this shape and workspace size: 0 = the int8 launch of
+ * rein_mmq_xq8, 1 = fp6 with one token group per workgroup, 2 = fp6 split-tail. */
+int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes);
 int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                     unsigned out_dim, unsigned p_rows, void *workspace, size_t workspace_bytes,
                     rein_stream_t s);
@@ -293,7 +306,7 @@ int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned i
  * forbid hipMalloc.  It has no counterpart in the reference.  The workspace is a fixed array of
  * 8 MiB in device memory that every GPU the process uses holds until the process ends
  * (librein_scratch.so, loaded from the directory of librein.so on the first call).  Shapes whose
- * rein_mmq_workspace_bytes exceeds 8 MiB are refused with REIN_E_TOO_LARGE (at in_dim 5120
+ * rein_mmq_workspace_min_bytes exceeds 8 MiB are refused with REIN_E_TOO_LARGE (at in_dim 5120
  * that is above 768 rows); shapes that need no workspace run rein_mmq_xq8.  All calls on one
  * GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
 int rein_mmq_xq8_noalloc(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,

@@ -83,6 +83,8 @@ SIGNATURES = {
     "rein_mmq_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_matmul": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _vp]),
     "rein_mmq_workspace_bytes": (_sz, [_i, _u, _u]),
+    "rein_mmq_workspace_min_bytes": (_sz, [_i, _u, _u]),
+    "rein_mmq_form_ws": (_i, [_i, _u, _u, _u, _sz]),
     "rein_mmq_xq8_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
     "rein_mmq_xq8_noalloc": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_mmq_tile_plan_ws": (_i, [_i, _u, _u, _vp, _vp]),

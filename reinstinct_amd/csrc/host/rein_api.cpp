@@ -712,21 +712,75 @@ int mmq6_prep(const void* xq, void* img, unsigned n_sub, unsigned p_rows, rein_s
     void* a[] = {(void*)&xq, (void*)&img, (void*)&n_sub, (void*)&p_rows};
     return launch("rein_mmq6_prep", (p_rows + 31) / 32, (n_sub + 7) / 8, 1, 256, 0, s, a);
 }
+
+// Split-tail launch (rein_mmq6_split_tail): one workgroup per resident slot, two per CU; whole
+// 4-tile units in rounds, the units left over split along the contraction.  Behind the activation
+// image the workspace then holds one partial tile per workgroup.
+constexpr unsigned kSkGrid = 2 * kCUs;
+constexpr size_t kSkPartBytes = (size_t)4 * 16 * 256 * 4;                 // one partial tile: 4 x 32 tokens x 128 rows fp32
+size_t sk_image_bytes(unsigned in_dim, unsigned p_rows) { return (x6_image_bytes(in_dim / 32, p_rows) + 255) & ~(size_t)255; }
+size_t sk_workspace_bytes(unsigned in_dim, unsigned p_rows)
+{
+    return sk_image_bytes(in_dim, p_rows) + (size_t)kSkGrid * kSkPartBytes;
+}
+unsigned sk_grid()                 // REIN_MMQ6_SK_GRID: fewer workgroups (a multiple of 8), for tests of several rounds
+{
+    const unsigned g = env_u("REIN_MMQ6_SK_GRID", kSkGrid) & ~7u;
+    return g >= 8 && g <= kSkGrid ? g : kSkGrid;
+}
+// Workgroups per tail unit: at most 8 (every range pays a pipeline fill and a partial tile), at most one per
+// chunk; behind whole rounds as many as fill one workgroup per CU, without them both slots.  Measured at
+// 5120 x 17408 (us at split 1 / 2 / 4 / 8): 128 tokens 97 / 77 / 63 / 63 (3 in effect), 512 tokens 216 / 181 /
+// 169 / 167, 2048 tokens 570 / 575 / 586 / 595.
+unsigned sk_split(unsigned in_dim, unsigned out_dim, unsigned p_rows)
+{
+    const unsigned g = sk_grid(), n_unit = ((out_dim + 127) / 128) * (((p_rows + 31) / 32 + 3) / 4), n_tail = n_unit % g;
+    if (n_tail == 0) return 1;
+    const unsigned forced = env_u("REIN_MMQ6_SK_SPLIT", 0);
+    const unsigned room = (n_unit >= g ? g / 2 : g) / n_tail;
+    const unsigned most = std::min(g / n_tail, in_dim / 256);
+    return std::max(1u, std::min(forced ? forced : std::min(8u, room), most));
+}
+// The launch wants whole 4-tile token groups (a ragged last group computes its missing tiles all the same).
+// It pays where the tail is what decides: no whole round and a tail that splits at least two ways (small
+// grids that would leave CUs idle), or one whole round and a tail that splits at least four ways (512 x 17408:
+// 167-172 us against 189-204 for the mixed launch).  With more rounds the workgroups of the mixed launch
+// drift apart and overlap their fills and stores, which this launch's lock-step rounds do not (2048 tokens:
+// 575-690 us against 586-617), and an unsplit tail is the mixed launch's all-wide plan.  REIN_MMQ6_SK = 2
+// forces the launch wherever it is valid.
+bool mmq6_split_tail(unsigned in_dim, unsigned out_dim, unsigned p_rows)
+{
+    const unsigned mode = env_u("REIN_MMQ6_SK", 1);
+    if (mode == 0) return false;
+    if (std::getenv("REIN_MMQ6_N4") || std::getenv("REIN_MMQ6_N2")) return false;      // a forced token-group split
+    const unsigned n_tt = (p_rows + 31) / 32, n_tg = (n_tt + 3) / 4;
+    if (8 * (4 * n_tg - n_tt) > n_tt) return false;                       // more than an eighth of the tiles empty
+    if (mode == 2 || std::getenv("REIN_MMQ6_SK_GRID")) return true;
+    const unsigned rounds = ((out_dim + 127) / 128) * n_tg / sk_grid(), split = sk_split(in_dim, out_dim, p_rows);
+    return (rounds == 0 && split >= 2) || (rounds == 1 && split >= 4);
+}
+
 }  // namespace
+
+size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows)
+{
+    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < env_u("REIN_MMQ6_FROM", 320)) return 0;
+    return x6_image_bytes(in_dim / 32, p_rows);
+}
 
 size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
     // below ~300 rows the int8 launch (more, smaller workgroups in flight) is the faster one:
     // 128 rows 61 vs 93 us, 256 rows 112 vs 122 us, 512 rows 185 vs 177 us at 5120 x 17408
-    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < env_u("REIN_MMQ6_FROM", 320)) return 0;
-    return x6_image_bytes(in_dim / 32, p_rows);
+    if (rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows) == 0) return 0;
+    return env_u("REIN_MMQ6_SK", 1) != 0 ? sk_workspace_bytes(in_dim, p_rows) : x6_image_bytes(in_dim / 32, p_rows);
 }
 
 int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
                     unsigned p_rows, void* workspace, size_t workspace_bytes, rein_stream_t s)
 {
     const char* who = "rein_mmq_xq8_ws";
-    const size_t need = rein_mmq_workspace_bytes(fmt, in_dim, p_rows);
+    const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
     if (!workspace || need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
@@ -734,7 +788,19 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     if (int rc = check_ptr(who, workspace, 16, "workspace")) return rc;
     if (workspace_bytes < need)
-        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace of " + std::to_string(workspace_bytes) + " bytes, rein_mmq_workspace_bytes asks for " + std::to_string(need));
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace of " + std::to_string(workspace_bytes) + " bytes, rein_mmq_workspace_min_bytes asks for " + std::to_string(need));
+    if (workspace_bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows)) {
+        char* base = static_cast<char*>(workspace);
+        float* part = reinterpret_cast<float*>(base + sk_image_bytes(in_dim, p_rows));
+        const unsigned split = sk_split(in_dim, out_dim, p_rows), g = sk_grid();
+        const unsigned n_unit = ((out_dim + 127) / 128) * (((p_rows + 31) / 32 + 3) / 4), n_tail = n_unit % g, first = n_unit - n_tail;
+        if (int rc = mmq6_prep(xq, workspace, in_dim / 32, p_rows, s)) return rc;
+        void* a[] = {(void*)&w, (void*)&workspace, (void*)&y, (void*)&part, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&split};
+        if (int rc = launch("rein_mmq6_q4k_sk", g, 1, 1, 256, mmq6_lds_bytes(4), s, a)) return rc;
+        if (n_tail == 0 || split == 1) return 0;
+        void* b[] = {(void*)&part, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&first, (void*)&split};
+        return launch("rein_mmq6_tail_sum", n_tail, 4, 1, 256, 0, s, b);
+    }
     unsigned n4, n2;
     mmq6_pick(out_dim, p_rows, &n4, &n2);
     const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + 31) / 32, n1 = n_tt - 4 * n4 - 2 * n2;
@@ -779,7 +845,8 @@ int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsig
                          unsigned p_rows, rein_stream_t s)
 {
     if (int rc = need_runtime()) return rc;
-    const size_t need = rein_mmq_workspace_bytes(fmt, in_dim, p_rows);
+    // the smallest workspace form: the activation image alone (the 8 MiB array has no room for partial tiles)
+    const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
     if (need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);      // that launch has no scratch
     void* ptr = nullptr;
     size_t bytes = 0;
@@ -788,6 +855,13 @@ int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsig
         return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8_noalloc: this shape needs " + std::to_string(need) + " bytes of scratch, the fixed array holds " +
                                           std::to_string(bytes) + "; use rein_mmq_xq8_ws with a workspace of your own");
     return rein_mmq_xq8_ws(fmt, w, xq, y, in_dim, out_dim, p_rows, ptr, bytes, s);
+}
+
+int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes)
+{
+    const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
+    if (need == 0 || workspace_bytes < need) return 0;
+    return workspace_bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows) ? 2 : 1;
 }
 
 int rein_mmq_tile_plan_ws(int fmt, unsigned out_dim, unsigned p_rows, unsigned* n4, unsigned* n2)
@@ -863,7 +937,8 @@ int rein_matmul_ws(int fmt, const void* w, const float* x, float* y, unsigned in
     const size_t xq = ((size_t)n_rows * (in_dim / 32) * 40 + 255) & ~(size_t)255;
     if (scratch_bytes < (size_t)n_rows * (in_dim / 32) * 40)
         return fail(REIN_E_BAD_SHAPE, "rein_matmul_ws: scratch smaller than the quantized activations");
-    if (rein_matmul_path(fmt, n_rows) != 2 || scratch_bytes < rein_matmul_scratch_bytes(fmt, in_dim, n_rows))
+    if (rein_matmul_path(fmt, n_rows) != 2 || rein_mmq_workspace_min_bytes(fmt, in_dim, n_rows) == 0 ||
+        scratch_bytes < xq + rein_mmq_workspace_min_bytes(fmt, in_dim, n_rows))
         return rein_matmul(fmt, w, x, y, in_dim, out_dim, n_rows, scratch, s);
     if (int rc = rein_quantize_q8(x, scratch, in_dim, n_rows, s)) return rc;
     return rein_mmq_xq8_ws(fmt, w, scratch, y, in_dim, out_dim, n_rows, static_cast<char*>(scratch) + xq, scratch_bytes - xq, s);

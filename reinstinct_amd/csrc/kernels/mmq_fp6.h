@@ -211,6 +211,10 @@ struct Mmq6Span {
     unsigned rec_cnt;    // records that exist from rec0 on (>= 1); min(NT, rec_cnt) are computed
     unsigned tok_base;   // row of y of token 0 of record rec0; record rec0 + t starts 32 t rows on
     unsigned tok_end;    // one past the last row of this span
+    unsigned pair_begin; // the sub-block pairs [pair_begin, pair_end) of the contraction are summed,
+    unsigned pair_end;   // both multiples of 4 (whole superblocks); pair_end = 0 stands for the whole contraction
+    float* part;         // nullptr: the sums are the result, stored to y; else: a partial tile, stored
+                         // here as [tile][register][thread] (NT * 16 * 256 floats) for rein_mmq6_tail_sum
 };
 
 template <int NT, int DOTS>
@@ -290,13 +294,17 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
     for (int v = 0; v < 32; v++) z32[v] = 0.0f;
     const int scale_a = h ? 130 : 134, scale_b = 130;                   // 2^3, 2^7 | 2^3 (E8M0)
 
-    // prologue: everything the steps before the first in-loop requests land need
+    // prologue: everything the steps before the first in-loop requests land need.  A workgroup
+    // may run several tiles in a row: the barrier keeps the first transfers off buffers that a
+    // slower wavefront still reads for the previous tile.
+    const unsigned pb = span.pair_begin, pe = span.pair_end ? span.pair_end : n_pair;     // 0: the whole contraction
+    __syncthreads();
 #pragma unroll
-    for (unsigned k = 0; k + 1u < D; k++) issue_acts(k);
+    for (unsigned k = 0; k + 1u < D; k++) issue_acts(pb + k);
 #pragma unroll
-    for (unsigned k = 0; k + 1u < R; k++) issue_ring(k);
+    for (unsigned k = 0; k + 1u < R; k++) issue_ring((pb >> 1) + k);
 #pragma unroll
-    for (unsigned k = 0; k < S; k++) issue_small(k);
+    for (unsigned k = 0; k < S; k++) issue_small((pb >> 2) + k);
     REIN_WAIT_VMCNT(0);
 
     // Words 4, 5 of the second operand of a pair are addressed through an offset the compiler
@@ -309,7 +317,7 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
     rein_v8bf pmin[2];               // bf16 pieces of -dmin * m of that sub-block, in slot order
     const unsigned rot = j >> 1;
 
-    for (unsigned i = 0; i < n_pair; i++) {
+    for (unsigned i = pb; i < pe; i++) {
         if ((i & 3u) == 0u) REIN_WAIT_VMCNT(Waits::at(0));
         else if ((i & 3u) == 1u) REIN_WAIT_VMCNT(Waits::at(1));
         else if ((i & 3u) == 2u) REIN_WAIT_VMCNT(Waits::at(2));
@@ -388,6 +396,13 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
     REIN_WAIT_VMCNT(0);
 
     if constexpr (DOTS == 0) {
+        if (span.part) {
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) span.part[(t * 16 + v) * 256 + threadIdx.x] = acc[t][v];
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -410,7 +425,7 @@ __device__ __forceinline__ void rein_mmq6_tile(const uint8_t* __restrict__ w, co
 __device__ __forceinline__ Mmq6Span rein_mmq6_dense_span(unsigned p_rows, unsigned tt0)
 {
     const unsigned n_tt = (p_rows + 31u) / 32u;
-    return Mmq6Span{n_tt, tt0, n_tt - tt0, tt0 * 32u, p_rows};
+    return Mmq6Span{n_tt, tt0, n_tt - tt0, tt0 * 32u, p_rows, 0u, 0u, nullptr};
 }
 
 __device__ __forceinline__ void rein_mmq6_mixed(const uint8_t* __restrict__ w, const uint8_t* __restrict__ img,
@@ -452,6 +467,77 @@ __device__ __forceinline__ void rein_mmq6_dense(const uint8_t* __restrict__ w, c
     rein_mmq6_tile<NT, DOTS>(w, img, y, dots, in_dim, out_dim, rb, rein_mmq6_dense_span(p_rows, tg * NT));
 }
 
+// ---- split-tail launch ----------------------------------------------------------------
+// 17408 rows are 136 row blocks, 512 tokens four 4-tile groups: 544 workgroup tiles on 512
+// resident slots is 1.06 rounds, and no tiling by powers of two changes that 17/16.  Here the
+// launch is exactly the resident slots (gridDim.x = G workgroups, a multiple of 8), and the
+// units -- unit u = (row block u / n_tg, 4-tile token group u % n_tg) -- are dealt in rounds:
+// in round r workgroup `pos` computes unit r G + pos whole.  What is left after the whole
+// rounds (U mod G units, the tail) is split along the contraction: `split` workgroups per
+// unit, each a contiguous range of superblock chunks, all at the same time; the workgroup of
+// range k of tail unit t stores its partial tile to slot t * split + k of `part`, and
+// rein_mmq6_tail_sum, launched behind this kernel, adds the partial tiles of every tail unit
+// in range order.
+// pos = (blockIdx.x % 8) * G / 8 + blockIdx.x / 8: the workgroups of one XCD hold neighbouring
+// units, so the token groups of a row block -- and the ranges of a tail unit -- meet in one
+// L2 at the same time.
+__device__ __forceinline__ void rein_mmq6_split_tail(const uint8_t* __restrict__ w, const uint8_t* __restrict__ img,
+                                                     float* __restrict__ y, float* __restrict__ part,
+                                                     unsigned in_dim, unsigned out_dim, unsigned p_rows, unsigned split)
+{
+    constexpr unsigned kPart = 4u * 16u * 256u;                          // floats per partial tile
+    const unsigned n_rb = (out_dim + 127u) / 128u, n_tt = (p_rows + 31u) / 32u, n_tg = (n_tt + 3u) / 4u;
+    const unsigned n_chunk = in_dim >> 8, g = gridDim.x, n_unit = n_rb * n_tg;
+    const unsigned pos = (blockIdx.x & 7u) * (g >> 3) + (blockIdx.x >> 3);
+    const unsigned rounds = n_unit / g, n_tail = n_unit - rounds * g;
+
+    for (unsigned r = 0; r < rounds; r++) {
+        const unsigned u = r * g + pos, rb = u / n_tg, tg = u % n_tg;
+        const Mmq6Span span{n_tt, tg * 4u, n_tt - tg * 4u, tg * 128u, p_rows, 0u, 0u, nullptr};
+        rein_mmq6_tile<4, 0>(w, img, y, nullptr, in_dim, out_dim, rb, span);
+    }
+    // the tail's ranges are dealt evenly over the XCDs, each XCD a contiguous run of them
+    const unsigned n_seg = n_tail * split, per_xcd = (n_seg + 7u) >> 3;
+    const unsigned seg = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if ((blockIdx.x >> 3) >= per_xcd || seg >= n_seg) return;
+
+    const unsigned tu = seg / split, k = seg - tu * split;               // tail unit, range within it
+    const unsigned u = rounds * g + tu, rb = u / n_tg, tg = u % n_tg;
+    const unsigned c0 = n_chunk * k / split, c1 = n_chunk * (k + 1u) / split;
+    if (c0 == c1) return;                                                // more ranges than chunks: nothing to add
+    const Mmq6Span span{n_tt, tg * 4u, n_tt - tg * 4u, tg * 128u, p_rows, 4u * c0, 4u * c1,
+                        split > 1u ? part + (size_t)seg * kPart : nullptr};
+    rein_mmq6_tile<4, 0>(w, img, y, nullptr, in_dim, out_dim, rb, span);
+}
+
+// y of the tail units = their partial tiles added in range order.  blockIdx.x = tail unit,
+// blockIdx.y = 32-token tile of the unit's four, 256 threads as in the GEMM (thread -> weight
+// row, register -> token).  `first_unit` = the whole rounds' unit count.
+__device__ __forceinline__ void rein_mmq6_tail_sum_body(const float* __restrict__ part, float* __restrict__ y,
+                                                        unsigned in_dim, unsigned out_dim, unsigned p_rows,
+                                                        unsigned first_unit, unsigned split)
+{
+    constexpr unsigned kPart = 4u * 16u * 256u;
+    const unsigned n_tt = (p_rows + 31u) / 32u, n_tg = (n_tt + 3u) / 4u, n_chunk = in_dim >> 8;
+    const unsigned tu = blockIdx.x, t = blockIdx.y, u = first_unit + tu, rb = u / n_tg, tg = u % n_tg;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, j = lane & 31u, h = lane >> 5;
+    const unsigned row = rb * 128u + wave * 32u + j;
+    float sum[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) sum[v] = 0.0f;
+    for (unsigned q = 0; q < split; q++) {
+        if (n_chunk * q / split == n_chunk * (q + 1u) / split) continue;           // an empty range stored nothing
+        const float* src = part + (size_t)(tu * split + q) * kPart;
+#pragma unroll
+        for (int v = 0; v < 16; v++) sum[v] += src[(t * 16 + v) * 256 + threadIdx.x];
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const unsigned tok = tg * 128u + t * 32u + 8 * (v / 4) + 4 * h + (v % 4);
+        if (tok < p_rows && row < out_dim) y[(size_t)tok * out_dim + row] = sum[v];
+    }
+}
+
 #define REIN_DEFINE_MMQ6_PREP(name)                                                                 \
     extern "C" __global__ __launch_bounds__(256) void name(const BlockQ8* __restrict__ xq,          \
                                                            unsigned char* __restrict__ img,         \
@@ -475,6 +561,23 @@ __device__ __forceinline__ void rein_mmq6_dense(const uint8_t* __restrict__ w, c
         unsigned int n4, unsigned int n2)                                                           \
     {                                                                                               \
         rein_mmq6_mixed(w, img, y, in_dim, out_dim, p_rows, n4, n2);                                \
+    }
+
+#define REIN_DEFINE_MMQ6_SPLIT_TAIL(name)                                                           \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                            \
+        const unsigned char* __restrict__ w, const unsigned char* __restrict__ img,                 \
+        float* __restrict__ y, float* __restrict__ part, unsigned int in_dim,                       \
+        unsigned int out_dim, unsigned int p_rows, unsigned int split)                              \
+    {                                                                                               \
+        rein_mmq6_split_tail(w, img, y, part, in_dim, out_dim, p_rows, split);                      \
+    }
+
+#define REIN_DEFINE_MMQ6_TAIL_SUM(name)                                                             \
+    extern "C" __global__ __launch_bounds__(256) void name(                                         \
+        const float* __restrict__ part, float* __restrict__ y, unsigned int in_dim,                 \
+        unsigned int out_dim, unsigned int p_rows, unsigned int first_unit, unsigned int split)     \
+    {                                                                                               \
+        rein_mmq6_tail_sum_body(part, y, in_dim, out_dim, p_rows, first_unit, split);               \
     }
 
 #define REIN_DEFINE_MMQ6_DOTS(name)                                                                 \

@@ -81,6 +81,16 @@ def mmq_workspace_bytes(fmt, in_dim, p_rows):
     return int(lib.rein_mmq_workspace_bytes(fmt, in_dim, p_rows))
 
 
+def mmq_form_ws(fmt, in_dim, out_dim, p_rows, workspace_bytes):
+    """0: int8 launch, 1: fp6 with one token group per workgroup, 2: fp6 stream-K"""
+    return int(lib.rein_mmq_form_ws(fmt, in_dim, out_dim, p_rows, workspace_bytes))
+
+
+def mmq_workspace_min_bytes(fmt, in_dim, p_rows):
+    """the smallest workspace rein_mmq_xq8_ws accepts: the activation image alone (no stream-K launch)"""
+    return int(lib.rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows))
+
+
 def mmq_xq8_ws(fmt, w, xq, y, in_dim, out_dim, p_rows, workspace, workspace_bytes, stream=None):
     """mmq_xq8 with the caller's workspace (the scratch PrefillGemm keeps, prefill.rs:479-495)"""
     check(lib.rein_mmq_xq8_ws(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _p(workspace), workspace_bytes,

@@ -117,8 +117,8 @@ def test_workspace_contract():
     packed = weights(in_dim, out_dim, seed=1, gaussian=True)
     x = np.random.default_rng(2).standard_normal((p_rows, in_dim)).astype(np.float32)
     dw, dq = dev(packed), quantized(x)
-    need = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows)
-    assert need > 0
+    need = runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, p_rows)
+    assert 0 < need <= runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows)
     # formats and row counts without a workspace launch ask for none
     assert runtime.mmq_workspace_bytes(rein.Q6_K, in_dim, p_rows) == 0
     assert runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, 16) == 0
@@ -160,3 +160,91 @@ def test_two_launches_and_a_reused_workspace_agree():
         hip.synchronize()
         want = orc.matvec_q8(rein.Q4_K, packed, in_dim, out_dim, dq.to_host(np.uint8), p_rows)
         assert_close_f32(dy.to_host(np.float32).reshape(p_rows, out_dim), want, what=f"reused workspace P {p_rows}")
+
+
+# ---- split-tail launch: whole tiles in rounds over the resident workgroups, the tiles left over split along the
+# contraction, their partial tiles summed in range order by whichever workgroup completes the tile
+def run_split_tail(dw, dq, in_dim, out_dim, p_rows, grid):
+    ws_bytes = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows)
+    os.environ["REIN_MMQ6_SK_GRID"] = str(grid)
+    try:
+        assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, p_rows, ws_bytes) == 2, "shape does not take the split-tail launch"
+        ws = hip.DeviceBuf(ws_bytes)
+        dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+        outs = []
+        for _ in range(2):                               # the second launch finds the first one's counters and partial tiles
+            runtime.mmq_xq8_ws(rein.Q4_K, dw, dq, dy, in_dim, out_dim, p_rows, ws, ws_bytes)
+            hip.synchronize()
+            outs.append(dy.to_host(np.float32).reshape(p_rows, out_dim).copy())
+    finally:
+        os.environ.pop("REIN_MMQ6_SK_GRID", None)
+    return outs
+
+
+# (tokens, K, N, workgroups): 128 units on 512 workgroups (no whole round, four ranges per tile); 18 units on 64
+# (three ranges over four chunks: uneven, ragged rows); 20 units on 8 (two whole rounds, then four tiles in two
+# ranges each; ragged last token group and last tile); 8 units on 16; 15 units on 32 (two ranges over five chunks)
+@pytest.mark.parametrize("p_rows,in_dim,out_dim,grid,gaussian", [
+    (512, 2048, 4096, 512, True), (256, 1024, 1100, 64, False), (470, 768, 640, 8, True), (128, 2048, 1024, 16, True),
+    (384, 1280, 520, 32, False)])
+def test_split_tail_matches_oracle_and_repeats(p_rows, in_dim, out_dim, grid, gaussian):
+    print(f"mmq6 split-tail P {p_rows} K {in_dim} N {out_dim} grid {grid}", flush=True)
+    packed = weights(in_dim, out_dim, seed=p_rows + grid, gaussian=gaussian)
+    x = np.random.default_rng(grid).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dw, dq = dev(packed), quantized(x)
+    first, second = run_split_tail(dw, dq, in_dim, out_dim, p_rows, grid)
+    want = orc.matvec_q8(rein.Q4_K, packed, in_dim, out_dim, dq.to_host(np.uint8), p_rows)
+    assert_close_f32(first, want, what=f"split-tail {p_rows}x{in_dim}x{out_dim} grid {grid}")
+    assert np.array_equal(first.view(np.uint32), second.view(np.uint32)), "split-tail result is not reproducible"
+
+
+def test_split_tail_needs_the_full_workspace():
+    p_rows, in_dim, out_dim = 512, 2048, 4096
+    full, least = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows), runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, p_rows)
+    assert 0 < least < full
+    assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, p_rows, full) == 2
+    assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, p_rows, full - 1) == 1
+    assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, p_rows, least - 1) == 0
+    assert runtime.mmq_form_ws(rein.Q6_K, in_dim, out_dim, p_rows, full) == 0
+    # the two fp6 launches agree within the bar (different order of the fp32 additions across superblocks)
+    packed = weights(in_dim, out_dim, seed=21, gaussian=True)
+    x = np.random.default_rng(22).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dw, dq = dev(packed), quantized(x)
+    outs = []
+    for nbytes in (full, least):
+        ws = hip.DeviceBuf(nbytes)
+        dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+        runtime.mmq_xq8_ws(rein.Q4_K, dw, dq, dy, in_dim, out_dim, p_rows, ws, nbytes)
+        hip.synchronize()
+        outs.append(dy.to_host(np.float32).reshape(p_rows, out_dim))
+    assert_close_f32(outs[0], outs[1], what="split-tail vs one group per workgroup")
+
+
+def test_workspace_launches_at_the_benchmark_shape():
+    # 5120 x 17408 at 512 tokens (one whole round + 32 tiles split eight ways) and 2048 tokens (mixed launch):
+    # every element against the int8 launch, sampled tokens against the oracle; the default row threshold applies
+    os.environ.pop("REIN_MMQ6_FROM", None)
+    try:
+        in_dim, out_dim = 5120, 17408
+        w = (np.random.default_rng(31).standard_normal((512, in_dim)) * 0.02).astype(np.float32)
+        raw = np.tile(quant.quantize_weights(rein.Q4_K, w), out_dim // 512)
+        packed = quant.repack_for_matvec(rein.Q4_K, raw, in_dim, out_dim)
+        x = np.random.default_rng(32).standard_normal((2048, in_dim)).astype(np.float32)
+        dw, dq = dev(packed), quantized(x)
+        xq = dq.to_host(np.uint8).reshape(2048, -1)
+        for m, form in ((512, 2), (2048, 1)):
+            print(f"mmq6 benchmark shape M {m}", flush=True)
+            ws_bytes = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, m)
+            assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, m, ws_bytes) == form
+            ws = hip.DeviceBuf(ws_bytes)
+            dy, dy8 = dev(np.full(m * out_dim, np.nan, np.float32)), dev(np.full(m * out_dim, np.nan, np.float32))
+            runtime.mmq_xq8_ws(rein.Q4_K, dw, dq, dy, in_dim, out_dim, m, ws, ws_bytes)
+            runtime.mmq_xq8(rein.Q4_K, dw, dq, dy8, in_dim, out_dim, m)
+            hip.synchronize()
+            got = dy.to_host(np.float32).reshape(m, out_dim)
+            assert_close_f32(got, dy8.to_host(np.float32).reshape(m, out_dim), what=f"workspace launch vs int8 launch, M {m}")
+            toks = np.unique(np.r_[0, 127, 128, m - 129, m - 1, np.random.default_rng(m).integers(0, m, 8)])
+            want = orc.matvec_q8(rein.Q4_K, packed, in_dim, out_dim, np.ascontiguousarray(xq[toks]).reshape(-1), len(toks))
+            assert_close_f32(got[toks], want, what=f"workspace launch vs oracle, M {m}")
+    finally:
+        os.environ["REIN_MMQ6_FROM"] = "17"

@@ -1,6 +1,7 @@
 """The entry point that allocates nothing (rein_mmq_xq8_noalloc) against the entry point it is a
-variant of (rein_mmq_xq8_ws with a caller's workspace): the same bits, on two calls in a row,
-the second with a smaller input; shapes beyond the fixed array are refused."""
+variant of (rein_mmq_xq8_ws with a caller's workspace of the size the fixed array is used at: the
+activation image, rein_mmq_workspace_min_bytes): the same bits, on two calls in a row, the second
+with a smaller input; shapes beyond the fixed array are refused."""
 import numpy as np
 import pytest
 
@@ -19,7 +20,7 @@ def run_pair(fmt, p_rows, in_dim, out_dim, seed):
     x = np.random.default_rng(seed).standard_normal((p_rows, in_dim)).astype(np.float32)
     d_x, dq = dev(x), hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
     runtime.quantize_q8(d_x, dq, in_dim, p_rows)
-    need = runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
+    need = runtime.mmq_workspace_min_bytes(fmt, in_dim, p_rows)
     ws = hip.DeviceBuf(max(need, 16))
     d_ref = dev(np.full(p_rows * out_dim, np.nan, np.float32))
     runtime.mmq_xq8_ws(fmt, dw, dq, d_ref, in_dim, out_dim, p_rows, ws if need else None, need)
@@ -49,7 +50,7 @@ def test_no_alloc_entry_refuses_what_the_fixed_array_cannot_hold():
     init()
     hip.set_device(0)
     p_rows, in_dim, out_dim = 1024, 5120, 128
-    assert runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows) > (8 << 20)
+    assert runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, p_rows) > (8 << 20)
     raw = random_raw_weights(rein.Q4_K, in_dim, out_dim, 6)
     dw = dev(quant.repack_for_matvec(rein.Q4_K, raw, in_dim, out_dim))
     dq = hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
