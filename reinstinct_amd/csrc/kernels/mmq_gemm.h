@@ -1051,15 +1051,20 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     //   after pair 3    ring slot 1 <- c+1
     //   end of c        wait until only the slot 1 refill is in flight (slot 0 of c+1 is
     //                   in), barrier
+    // Fill: the ring requests go first, so that one memory latency covers them and the first
+    // activation blocks together: the store of those blocks waits for them, and by then the
+    // older ring requests have landed too (requests complete in order); the explicit wait
+    // behind the store costs nothing in that case and holds if the compiler moved a load.
     typename C::Small small;
     MmqXRegs<TM> xr;
+    rein_mmq_wload<FMT>(wsrc, 0, fmt, 0, n_sub);
+    rein_mmq_wload<FMT>(wsrc, 1, fmt, 4, n_sub);
     C::fetch_small(small, fmt, rowc, 0, n_sub, h);
     rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 0);
     rein_mmq_xstore<TM, C::kSplitK>(lds[0], xr, n_sub, tok_base, tok_end, 0);
+    REIN_WAIT_VMCNT(0);                              // both slots of chunk 0 have landed
+    __builtin_amdgcn_sched_barrier(0);               // the next fetch reuses the registers just stored
     rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 8 < n_sub ? 8 : 0);
-    rein_mmq_wload<FMT>(wsrc, 0, fmt, 0, n_sub);
-    rein_mmq_wload<FMT>(wsrc, 1, fmt, 4, n_sub);
-    REIN_WAIT_VMCNT(kDma);                           // slot 0 of chunk 0 has landed
     __syncthreads();
 
     unsigned buf = 0;
