@@ -1207,7 +1207,8 @@ __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ sla
 // workgroups (tile_ub = the host's upper bound of the tile count; surplus workgroups leave
 // at once).  Workgroup i runs on XCD i % 8, and all row blocks and slabs of a token tile are
 // dealt to the same XCD, so the tile's activation blocks are pulled into one L2 and re-read
-// there by the others.  Two slabs with their outputs let the gate and the up projection of
+// there by the others; XCD x takes the x-th eighth of the tiles, so the tiles of an expert
+// meet in one L2 too.  Two slabs with their outputs let the gate and the up projection of
 // an expert FFN run in one launch (twice the workgroups fill the machine better than two
 // launches of half the size, and the second launch's fill / drain disappears).  Without the grid-stride loops
 // of rein_mmq_grouped around it the tile keeps to the register budget of three
@@ -1221,10 +1222,13 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
                                                      float* __restrict__ y1, unsigned in_dim, unsigned out_dim,
                                                      unsigned n_slab)
 {
+    // XCD x takes the x-th eighth of the tiles that exist: neighbouring tiles -- the tiles of one
+    // expert -- run on one XCD at the same time and share the expert's weights in its L2
     const unsigned n_rb = (out_dim + 127u) / 128u, per = n_slab * n_rb;
     const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
-    const unsigned tile = (k / per) * 8u + xcd, rb = (k % per) % n_rb, z = (k % per) / n_rb;
-    if (blockDim.x != 256u || tile >= (unsigned)tile_off[n_expert]) return;
+    const unsigned n_tile = (unsigned)tile_off[n_expert], per_xcd = (n_tile + 7u) >> 3;
+    const unsigned tile = xcd * per_xcd + k / per, rb = (k % per) % n_rb, z = (k % per) / n_rb;
+    if (blockDim.x != 256u || k / per >= per_xcd || tile >= n_tile) return;
     const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
     const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
     const unsigned tok_end = (unsigned)expert_off[lo + 1];
