@@ -154,8 +154,8 @@ __device__ __forceinline__ void rein_lds_dma_u32(const void* gptr, unsigned lds_
 // The depths set how far ahead of their use the transfers are requested: D - 1 pair-steps for
 // the records, R - 1 ring stages (2 pair-steps each) for the weights, 4 S - 2 pair-steps for
 // the small words.  A pair-step of a 4-tile group computes for about a microsecond, which covers
-// the memory latency at the shallowest depths; the narrow groups (and the short contractions
-// of expert FFNs, whose weights come from HBM once) need the weights several stages ahead.
+// the memory latency at the shallowest depths; the narrow groups, whose pair-steps are a
+// quarter as long, are given the weights several stages ahead.
 template <int NT> struct Mmq6Cfg;
 template <> struct Mmq6Cfg<4> { static constexpr int R = 2, D = 3, S = 1; };
 template <> struct Mmq6Cfg<2> { static constexpr int R = 4, D = 4, S = 2; };
@@ -179,9 +179,10 @@ constexpr int rein_mmq6_lds_bytes()
 // were issued after X".  At the top of step i the step needs acts(i), at even i the ring stage
 // i / 2, at i % 4 == 0 the small words of chunk i / 4; Mmq6Waits counts what was issued after the
 // oldest of those, per i % 4.  The prologue issues everything the first steps need and drains
-// it, so the counts of the steady state hold from step 0.  Past the end of the contraction the
-// same transfers are issued on clamped addresses into buffers nobody reads again, which keeps
-// the counts uniform; the kernel drains them before it ends.
+// it, so the counts of the steady state hold from the first step.  Past the end of the pair
+// range the same transfers are issued (into buffers nobody reads again; past the end of the
+// contraction on clamped addresses), which keeps the counts uniform; the tile drains them
+// before it ends.
 template <int K, int R, int D, int S>
 struct Mmq6Waits {
     static constexpr int ring(int s) { return s % 2 == 0 ? 2 : 0; }
@@ -544,14 +545,6 @@ __device__ __forceinline__ void rein_mmq6_tail_sum_body(const float* __restrict_
                                                            unsigned int n_sub, unsigned int p_rows) \
     {                                                                                               \
         rein_mmq6_prep_body(xq, img, n_sub, p_rows);                                                \
-    }
-
-#define REIN_DEFINE_MMQ6(name, NT)                                                                  \
-    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                            \
-        const unsigned char* __restrict__ w, const unsigned char* __restrict__ img,                 \
-        float* __restrict__ y, unsigned int in_dim, unsigned int out_dim, unsigned int p_rows)      \
-    {                                                                                               \
-        rein_mmq6_dense<NT, 0>(w, img, y, nullptr, in_dim, out_dim, p_rows);                        \
     }
 
 #define REIN_DEFINE_MMQ6_MIXED(name)                                                                \

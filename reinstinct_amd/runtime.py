@@ -82,12 +82,12 @@ def mmq_workspace_bytes(fmt, in_dim, p_rows):
 
 
 def mmq_form_ws(fmt, in_dim, out_dim, p_rows, workspace_bytes):
-    """0: int8 launch, 1: fp6 with one token group per workgroup, 2: fp6 stream-K"""
+    """0: int8 launch, 1: fp6 with one token group per workgroup, 2: fp6 split-tail"""
     return int(lib.rein_mmq_form_ws(fmt, in_dim, out_dim, p_rows, workspace_bytes))
 
 
 def mmq_workspace_min_bytes(fmt, in_dim, p_rows):
-    """the smallest workspace rein_mmq_xq8_ws accepts: the activation image alone (no stream-K launch)"""
+    """the smallest workspace rein_mmq_xq8_ws accepts: the activation image alone (no split-tail launch)"""
     return int(lib.rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows))
 
 
