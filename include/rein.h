@@ -382,6 +382,16 @@ int rein_moe_grouped_gemm(int fmt, const void *slab, unsigned bytes_per_expert,
                           const int32_t *expert_off, const int32_t *tile_off, unsigned n_expert,
                           const void *xq, float *y, unsigned in_dim, unsigned out_dim,
                           unsigned n_entries, rein_stream_t s);
+/* Gate and up projection of an expert FFN with SwiGLU and the BlockQ8 quantizer in the GEMM's
+ * epilogue: xq_out [n_entries][out_dim/32] blocks = the bytes that rein_moe_grouped_gemm on
+ * gate_slab and on up_slab followed by rein_swiglu_q8 (swiglu_q8_f32,
+ * kernels/qwen35_fused.cpp:132-146) produce, without the two fp32 matrices between them.
+ * out_dim (the expert's ff width) a multiple of 32.  Formats: Q4_K, Q5_K, Q6_K, Q8_0. */
+int rein_moe_grouped_swiglu_q8(int fmt, const void *gate_slab, const void *up_slab,
+                               unsigned bytes_per_expert, const int32_t *expert_off,
+                               const int32_t *tile_off, unsigned n_expert, const void *xq,
+                               void *xq_out, unsigned in_dim, unsigned out_dim,
+                               unsigned n_entries, rein_stream_t s);
 /* ---- MoE decode: expert matvecs, the expert id is read on the device.
  * launch_moe_expert_matvec (qwen35.rs:3071-3100; kernels/moe_matvec_*_repacked.cpp):
  * y[tok][slot][out_dim] = W[ids[tok*n_used+slot]] . xq row at

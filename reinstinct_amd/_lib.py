@@ -101,6 +101,7 @@ SIGNATURES = {
     "rein_moe_quantize_scatter": (_i, [_vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_moe_scatter_rows": (_i, [_vp, _vp, _vp, _u, _u, _vp]),
     "rein_moe_grouped_gemm": (_i, [_i, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
+    "rein_moe_grouped_swiglu_q8": (_i, [_i, _vp, _vp, _u, _vp, _vp, _u, _vp, _vp, _u, _u, _u, _vp]),
     "rein_swiglu_mul": (_i, [_vp, _vp, _vp, _u, _vp]),
     "rein_ingest_format": (_i, [_i]),
     "rein_ingest_expert_format": (_i, [_i]),

@@ -1088,6 +1088,34 @@ int rein_moe_grouped_gemm(int fmt, const void* slab, unsigned bytes_per_expert, 
                           out_dim, n_entries, s);
 }
 
+// Gate + up + SwiGLU + BlockQ8 in one launch (rein_mmq_<fmt>_grouped_swiglu_q8): the grid is
+// 8 * ceil(tile_ub / 8) * ceil(out_dim / 64) workgroups, tile_ub as in launch_grouped.
+int rein_moe_grouped_swiglu_q8(int fmt, const void* gate_slab, const void* up_slab, unsigned bytes_per_expert,
+                               const int32_t* expert_off, const int32_t* tile_off, unsigned n_expert, const void* xq,
+                               void* xq_out, unsigned in_dim, unsigned out_dim, unsigned n_entries, rein_stream_t s)
+{
+    const char* who = "rein_moe_grouped_swiglu_q8";
+    if (fmt != REIN_TYPE_Q4_K && fmt != REIN_TYPE_Q5_K && fmt != REIN_TYPE_Q6_K && fmt != REIN_TYPE_Q8_0)
+        return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0");
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_entries)) return rc;
+    if (n_expert == 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": n_expert is zero");
+    if (out_dim % 32 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": out_dim must be a multiple of 32 (whole BlockQ8 blocks)");
+    if (bytes_per_expert % 16 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": bytes_per_expert must be a multiple of 16");
+    if (int rc = check_ptr(who, gate_slab, 16, "gate_slab")) return rc;
+    if (int rc = check_ptr(who, up_slab, 16, "up_slab")) return rc;
+    if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+    if (int rc = check_ptr(who, xq_out, 8, "xq_out")) return rc;
+    if (int rc = check_ptr(who, expert_off, 4, "expert_off")) return rc;
+    if (int rc = check_ptr(who, tile_off, 4, "tile_off")) return rc;
+    const unsigned bn = rein_moe_gemm_bn();
+    const unsigned tile_ub = (n_entries + bn - 1) / bn + n_expert;
+    const unsigned long long grid = 8ull * ((tile_ub + 7) / 8) * ((out_dim + 63) / 64);
+    if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, std::string(who) + ": more than 2^31 workgroup tiles");
+    void* a[] = {(void*)&gate_slab, (void*)&up_slab, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off,
+                 (void*)&n_expert, (void*)&xq, (void*)&xq_out, (void*)&in_dim, (void*)&out_dim};
+    return launch(std::string("rein_mmq_") + fmt_tag(fmt) + "_grouped_swiglu_q8", (unsigned)grid, 1, 1, 256, 0, s, a);
+}
+
 namespace {
 int moe_mv_launch(const char* who, const std::string& kernel, unsigned rows_per_block, int fmt, const void* slab0,
                   const void* slab1, const int32_t* ids, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
@@ -1336,6 +1364,13 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     }
     // the expert-sorted BlockQ8 rows straight from x (quantize_q8 + moe_gather_xq in one launch)
     if (int rc = rein_moe_quantize_scatter(x, inv, base + w.g_in, sh.hidden, sh.n_used, sh.n_tok, s)) return rc;
+    // gate and up projections, SwiGLU and the down projection's BlockQ8 rows in one launch;
+    // REIN_MOE_FUSED=0 takes the two-output GEMM and swiglu_q8_f32 instead (the same bytes)
+    const unsigned long long fused_grid = 8ull * (((ne + bn - 1) / bn + sh.n_expert + 7) / 8) * ((sh.expert_ff + 63) / 64);
+    if (sh.expert_ff % 32 == 0 && fused_grid <= 0x7FFFFFFFull && env_u("REIN_MOE_FUSED", 1) != 0) {
+        if (int rc = rein_moe_grouped_swiglu_q8(sh.gate_up_fmt, gate_exps, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
+                                                base + w.g_in, base + w.xq_exp, sh.hidden, sh.expert_ff, ne, s)) return rc;
+    } else {
     // gate and up projections in one launch (two slabs)
     if (int rc = launch_grouped(sh.gate_up_fmt, gate_exps, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert, base + w.g_in,
                                 (float*)(base + w.e_gate), (float*)(base + w.e_up), sh.hidden, sh.expert_ff, ne, s)) return rc;
@@ -1346,6 +1381,7 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
         const unsigned cnt = (unsigned)std::min(left, (size_t)1 << 30);
         if (int rc = rein_swiglu_q8((float*)(base + w.e_gate) + e0, (float*)(base + w.e_up) + e0, nullptr,
                                     base + w.xq_exp + e0 / 32 * 40, cnt, s)) return rc;
+    }
     }
     if (int rc = rein_moe_grouped_gemm(sh.down_fmt, down_exps, (unsigned)bpe_dn, eoff, toff, sh.n_expert,
                                        base + w.xq_exp, (float*)(base + w.g_out), sh.expert_ff, sh.hidden, ne, s)) return rc;

@@ -42,6 +42,7 @@
 #pragma once
 
 #include "rein_formats.h"
+#include "q8_block.h"
 
 typedef int   rein_v4i  __attribute__((ext_vector_type(4)));
 typedef int   rein_v16i __attribute__((ext_vector_type(16)));
@@ -1004,10 +1005,14 @@ __device__ __forceinline__ unsigned char* rein_mmq_tile_lds()
     return raw;
 }
 
+// The contraction of one workgroup tile: wavefront `wave` accumulates tokens tok_base ..
+// tok_end (at most TM) against the 32 weight rows from `row_base` of the matrix at `w`
+// (both may differ from wavefront to wavefront, but are uniform within one).  Ends on a
+// barrier: the tile's LDS is free again when it returns.
 template <int FMT, int TM, int LDSB = rein_mmq_tile_lds_bytes<FMT, TM>()>
-__device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
-                                                        float* __restrict__ y, unsigned in_dim, unsigned out_dim,
-                                                        unsigned rb, unsigned tok_base, unsigned tok_end)
+__device__ __forceinline__ void rein_mmq_pipelined_acc(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                       unsigned in_dim, unsigned out_dim, unsigned row_base,
+                                                       unsigned tok_base, unsigned tok_end, rein_v16f (&acc)[TM / 32])
 {
     using F = Fmt<FMT>;
     using C = MmqChunk<FMT>;
@@ -1023,7 +1028,6 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     const unsigned j = lane & 31u, h = lane >> 5;
     const unsigned n_sub = in_dim >> 5;
     const F fmt(w, n_sub, out_dim);
-    const unsigned row_base = rb * 128u + wave * 32u;
     const unsigned row = row_base + j;
     const unsigned rowc = row < out_dim ? row : out_dim - 1;
     const unsigned wsel = FMT == REIN_Q8_0 ? h : 0u;
@@ -1031,7 +1035,6 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
     MmqWSrc<FMT> wsrc;
     wsrc.init(wl, fmt, row_base, out_dim, lane);
 
-    rein_v16f acc[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -1090,7 +1093,19 @@ __device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restric
         if (more) REIN_WAIT_VMCNT(kDma);             // slot 0 of the next chunk has landed
         __syncthreads();
     }
+}
 
+template <int FMT, int TM, int LDSB = rein_mmq_tile_lds_bytes<FMT, TM>()>
+__device__ __forceinline__ void rein_mmq_pipelined_tile(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                        float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                        unsigned rb, unsigned tok_base, unsigned tok_end)
+{
+    constexpr int NT = TM / 32;
+    const unsigned lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned j = lane & 31u, h = lane >> 5;
+    const unsigned row = rb * 128u + wave * 32u + j;
+    rein_v16f acc[NT];
+    rein_mmq_pipelined_acc<FMT, TM, LDSB>(w, xq, in_dim, out_dim, rb * 128u + wave * 32u, tok_base, tok_end, acc);
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -1238,6 +1253,63 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
                                      tok_base, min(tok_end, tok_base + 32u));
 }
 
+// Gate and up projection of an expert FFN with SwiGLU and the BlockQ8 quantizer in the
+// epilogue: a workgroup owns one 32-token tile and 64 columns of the expert's ff dimension;
+// wavefronts 0, 1 run the gate rows of those columns, wavefronts 2, 3 the up rows (the same
+// contraction as rein_mmq_grouped_one, term for term, so gate and up carry the same bits as
+// the two-output launch).  The four 32 x 32 tiles then meet in LDS as [wavefront][token][column]
+// and the workgroup's sixteen 16-lane rows turn them into the 2 x 32 BlockQ8 blocks of
+// silu(gate) * up with the quantizer and the silu of swiglu_q8_f32 -- the same bytes as
+// rein_mmq_grouped_one + swiglu_q8_f32, without the two fp32 matrices between them.
+// Launch: 1-D, 8 * ceil(tile_ub / 8) * ceil(out_dim / 64) workgroups of 256 threads, tiles
+// dealt to XCDs as in rein_mmq_grouped_one.  out_dim a multiple of 32.
+template <int FMT>
+__device__ __forceinline__ void rein_mmq_grouped_swiglu(const uint8_t* __restrict__ gate_slab,
+                                                        const uint8_t* __restrict__ up_slab, unsigned bytes_per_expert,
+                                                        const int* __restrict__ expert_off, const int* __restrict__ tile_off,
+                                                        unsigned n_expert, const BlockQ8* __restrict__ xq,
+                                                        BlockQ8* __restrict__ out, unsigned in_dim, unsigned out_dim)
+{
+#pragma clang fp contract(off)
+    constexpr unsigned kPitch = 40;                   // floats per token row of a wavefront's tile: the two lane
+                                                      // halves (tokens 4 apart) land on different banks
+    static_assert(rein_mmq_tile_lds_bytes<FMT, 32>() >= 4 * 32 * (int)kPitch * 4, "epilogue image does not fit the tile LDS");
+    const unsigned n_cb = (out_dim + 63u) / 64u;
+    const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
+    const unsigned n_tile = (unsigned)tile_off[n_expert], per_xcd = (n_tile + 7u) >> 3;
+    const unsigned tile = xcd * per_xcd + k / n_cb, cb = k % n_cb;
+    if (blockDim.x != 256u || k / n_cb >= per_xcd || tile >= n_tile) return;
+    const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
+    const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
+    const unsigned tok_end = min((unsigned)expert_off[lo + 1], tok_base + 32u);
+    if (tok_base >= tok_end) return;
+
+    const unsigned lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint8_t* slab = (wave >> 1) ? up_slab : gate_slab;
+    rein_v16f acc[1];
+    rein_mmq_pipelined_acc<FMT, 32>(slab + (size_t)lo * bytes_per_expert, xq, in_dim, out_dim,
+                                    cb * 64u + (wave & 1u) * 32u, tok_base, tok_end, acc);
+
+    float* const img = reinterpret_cast<float*>(rein_mmq_tile_lds<rein_mmq_tile_lds_bytes<FMT, 32>()>());
+    const unsigned j = lane & 31u, h = lane >> 5;
+#pragma unroll
+    for (int v = 0; v < 16; v++) img[(wave * 32u + 8u * (v / 4) + 4u * h + (v % 4)) * kPitch + j] = acc[0][v];
+    __syncthreads();
+    const unsigned n_sub_out = out_dim >> 5;
+    const unsigned l = threadIdx.x & 15u, g = threadIdx.x >> 4;
+#pragma unroll
+    for (unsigned it = 0; it < 4u; it++) {
+        const unsigned idx = it * 16u + g, half = idx >> 5, tok = idx & 31u;
+        const unsigned blk = cb * 2u + half;
+        if (tok_base + tok < tok_end && blk < n_sub_out) {
+            const float* gt = img + (half * 32u + tok) * kPitch;
+            const float* ut = img + ((2u + half) * 32u + tok) * kPitch;
+            const float v0 = rein_silu_det(gt[l]) * ut[l], v1 = rein_silu_det(gt[l + 16]) * ut[l + 16];
+            rein_q8_store_sub(out + (size_t)(tok_base + tok) * n_sub_out + blk, l, v0, v1);
+        }
+    }
+}
+
 // Two wavefronts per SIMD: a 256-register budget, which makes the compiler keep
 // MFMA results in ordinary VGPRs (no AGPR round trips) without spilling.
 #define REIN_MMQ_OCC __attribute__((amdgpu_waves_per_eu(2)))
@@ -1294,4 +1366,15 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
     {                                                                                            \
         rein_mmq_grouped_one<FMT>(slab0, slab1, bytes_per_expert, expert_off, tile_off,          \
                                   n_expert, xq, y0, y1, in_dim, out_dim, n_slab);                \
+    }
+
+#define REIN_DEFINE_MMQ_GROUPED_SWIGLU(name, FMT)                                                \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                         \
+        const unsigned char* __restrict__ gate_slab, const unsigned char* __restrict__ up_slab,  \
+        unsigned int bytes_per_expert, const int* __restrict__ expert_off,                       \
+        const int* __restrict__ tile_off, unsigned int n_expert, const BlockQ8* __restrict__ xq, \
+        BlockQ8* __restrict__ out, unsigned int in_dim, unsigned int out_dim)                    \
+    {                                                                                            \
+        rein_mmq_grouped_swiglu<FMT>(gate_slab, up_slab, bytes_per_expert, expert_off, tile_off, \
+                                     n_expert, xq, out, in_dim, out_dim);                        \
     }

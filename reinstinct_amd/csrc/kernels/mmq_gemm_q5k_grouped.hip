@@ -12,3 +12,5 @@ REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q5k_grouped_t32, REIN_Q5_K)
 // (src/quant/q5_1.rs:58-60, qwen35.rs:3045) and looks up the same symbol in that module.
 REIN_DEFINE_MMQ_GROUPED(mmq_gemm_q5_1_grouped_f32, REIN_Q5_1)
 REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q5_1_grouped_t32, REIN_Q5_1)
+// gate + up + SwiGLU + BlockQ8 of an expert FFN in one launch
+REIN_DEFINE_MMQ_GROUPED_SWIGLU(rein_mmq_q5k_grouped_swiglu_q8, REIN_Q5_K)

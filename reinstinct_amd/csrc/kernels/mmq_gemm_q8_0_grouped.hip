@@ -7,3 +7,5 @@
 REIN_DEFINE_MMQ_GROUPED(mmq_gemm_q8_0_grouped_f32, REIN_Q8_0)
 // the library's launch: one tile per workgroup; two slabs run gate and up of an expert FFN at once
 REIN_DEFINE_MMQ_GROUPED_ONE(rein_mmq_q8_0_grouped_t32, REIN_Q8_0)
+// gate + up + SwiGLU + BlockQ8 of an expert FFN in one launch
+REIN_DEFINE_MMQ_GROUPED_SWIGLU(rein_mmq_q8_0_grouped_swiglu_q8, REIN_Q8_0)

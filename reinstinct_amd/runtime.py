@@ -175,6 +175,14 @@ def moe_grouped_gemm(fmt, slab, bytes_per_expert, expert_off, tile_off, n_expert
                                     _p(xq), _p(y), in_dim, out_dim, n_entries, _s(stream)))
 
 
+def moe_grouped_swiglu_q8(fmt, gate_slab, up_slab, bytes_per_expert, expert_off, tile_off, n_expert, xq, xq_out,
+                          in_dim, out_dim, n_entries, stream=None):
+    """gate + up grouped GEMM with SwiGLU and the BlockQ8 quantizer in the epilogue"""
+    check(lib.rein_moe_grouped_swiglu_q8(fmt, _p(gate_slab), _p(up_slab), bytes_per_expert, _p(expert_off),
+                                         _p(tile_off), n_expert, _p(xq), _p(xq_out), in_dim, out_dim, n_entries,
+                                         _s(stream)))
+
+
 def moe_expert_matvec(fmt, slab, ids, xq, y, in_dim, out_dim, bytes_per_expert, xq_tok_stride, xq_slot_stride,
                       n_used, n_tok=1, stream=None):
     """launch_moe_expert_matvec (src/runtime/qwen35.rs:3071-3100)"""

@@ -488,6 +488,42 @@ def test_grouped_gemm_parity(fmt, in_dim):
     assert_close_f32(dy.to_host(np.float32).reshape(n, out_dim), want, what=f"grouped fmt {fmt}")
 
 
+@pytest.mark.parametrize("fmt,in_dim,out_dim,n_tok,n_used", [
+    (rein.Q4_K, 512, 256, 40, 2), (rein.Q4_K, 256, 96, 75, 3), (rein.Q5_K, 512, 128, 40, 2),
+    (rein.Q6_K, 256, 160, 33, 2), (rein.Q8_0, 352, 64, 20, 4), (rein.Q4_K, 2048, 768, 64, 8)])
+def test_grouped_swiglu_q8_equals_the_three_launches(fmt, in_dim, out_dim, n_tok, n_used):
+    # gate + up + SwiGLU + BlockQ8 in the GEMM's epilogue: the bytes of two grouped GEMMs and
+    # swiglu_q8_f32 (whose own parity with the CPU restatement is tested in test_gpu_fused.py)
+    print(f"grouped swiglu fmt {fmt} K {in_dim} ff {out_dim} tokens {n_tok} x {n_used}", flush=True)
+    n_expert = 6
+    bpe = quant.repacked_len(fmt, in_dim, out_dim)
+    gate = np.concatenate([make_weights(fmt, in_dim, out_dim, seed=600 + e)[1] for e in range(n_expert)])
+    up = np.concatenate([make_weights(fmt, in_dim, out_dim, seed=700 + e)[1] for e in range(n_expert)])
+    rng = np.random.default_rng(in_dim + out_dim)
+    ids = rng.integers(0, n_expert, (n_tok, n_used)).astype(np.int32)
+    ids[ids == 2] = 3                                   # expert 2 gets no tokens
+    d_perm, d_eoff, d_toff = gpu_sort(ids, n_expert, runtime.moe_gemm_bn())
+    x = (rng.standard_normal((n_tok, in_dim)) * 3).astype(np.float32)
+    dq = gpu_quantize(x)
+    n = n_tok * n_used
+    d_gin = hip.DeviceBuf(n * (in_dim // 32) * 40)
+    runtime.moe_gather_xq(dq, d_perm, d_gin, in_dim // 32, n_used, n)
+    dg, du = dev(gate), dev(up)
+    d_eg, d_eu = hip.DeviceBuf(n * out_dim * 4), hip.DeviceBuf(n * out_dim * 4)
+    runtime.moe_grouped_gemm(fmt, dg, bpe, d_eoff, d_toff, n_expert, d_gin, d_eg, in_dim, out_dim, n)
+    runtime.moe_grouped_gemm(fmt, du, bpe, d_eoff, d_toff, n_expert, d_gin, d_eu, in_dim, out_dim, n)
+    nb = n * (out_dim // 32) * 40
+    d_want = hip.DeviceBuf(nb)
+    runtime.swiglu_q8(d_eg, d_eu, None, d_want, n * out_dim)
+    d_got = dev(np.full(nb, 0xA5, np.uint8))
+    runtime.moe_grouped_swiglu_q8(fmt, dg, du, bpe, d_eoff, d_toff, n_expert, d_gin, d_got, in_dim, out_dim, n)
+    hip.synchronize()
+    got, want = d_got.to_host(np.uint8).reshape(n, -1), d_want.to_host(np.uint8).reshape(n, -1)
+    assert n == int(d_eoff.to_host(np.int32)[n_expert]), "every routing entry belongs to an expert here"
+    bad = np.nonzero((got != want).any(axis=1))[0]
+    assert bad.size == 0, f"rows {bad[:8]} differ"
+
+
 def test_moe_ffn_end_to_end_small():
     # config 4 in miniature: top-k -> sort -> gather -> gate/up (Q4_K) -> SwiGLU ->
     # quantize -> down (Q6_K) -> scatter -> combine, against the same chain on the CPU

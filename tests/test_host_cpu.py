@@ -143,6 +143,8 @@ def test_compute_calls_fail_loudly_without_runtime():
     assert lib.rein_matvec_batched_xq8(rein.Q4_K, 16, 16, 16, 256, 8, 9, None) == -6
     assert lib.rein_quantize_q8(16, 16, 48, 1, None) == -3
     assert lib.rein_moe_grouped_gemm(rein.Q4_0, 16, 16, 16, 16, 1, 16, 16, 256, 8, 1, None) == -2
+    assert lib.rein_moe_grouped_swiglu_q8(rein.Q4_0, 16, 16, 16, 16, 16, 1, 16, 16, 256, 32, 1, None) == -2
+    assert lib.rein_moe_grouped_swiglu_q8(rein.Q8_0, 16, 16, 16, 16, 16, 1, 16, 16, 256, 40, 1, None) == -3   # ff not whole blocks
 
 
 def test_moe_workspace_layout():
