@@ -243,6 +243,8 @@ def mmq_kernel_name(fmt, in_dim, out_dim, p_rows):
     form = runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, ws_bytes)
     if form == 2:
         return f"rein_mmq6_prep + rein_mmq6_{tag}_sk (split-tail launch) + rein_mmq6_tail_sum"
+    if form == 3:
+        return f"rein_mmq_{tag}_sk / _sk32 (split-tail launch of the int8 tile) + rein_mmq_tail_sum_t64 / _t32"
     if form == 1:
         n4, n2 = runtime.mmq_tile_plan_ws(fmt, out_dim, p_rows)
         return f"rein_mmq6_prep + rein_mmq6_{tag}_mix (n4 = {n4}, n2 = {n2})"
@@ -270,6 +272,31 @@ def extras_mmq(stream):
             log("mmq", out[-1])
             del dx, dq, dy, wsp
         del ws
+    return out
+
+
+def extras_mmq_small(stream):
+    """Short prompts against the narrow projections (the decode shapes of BASELINE configs[1] as prefill
+    GEMMs): too few workgroup tiles for 256 CUs, which the split-tail launch of rein_mmq_xq8_ws repairs
+    when the caller provides the workspace; `us_no_workspace` is the plain launch of rein_mmq_xq8."""
+    out = []
+    for f in (rein.Q4_K, rein.Q6_K, rein.Q8_0):
+        for (k, n) in ((17408, 5120), (5120, 5120)):
+            packed = tiled_weights(f, k, n, seed=4)
+            ws = [hip.DeviceBuf.from_host(packed) for _ in range(max(4, (300 << 20) // packed.nbytes))]
+            for m in (32, 128):
+                x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+                dx, dq, dy = hip.DeviceBuf.from_host(x), hip.DeviceBuf(m * (k // 32) * 40), hip.DeviceBuf(m * n * 4)
+                runtime.quantize_q8(dx, dq, k, m, stream)
+                wsb = runtime.mmq_workspace_bytes(f, k, m)
+                wsp = hip.DeviceBuf(wsb) if wsb else None
+                sec = time_graph(stream, lambda: [runtime.mmq_xq8_ws(f, w_, dq, dy, k, n, m, wsp, wsb, stream) for w_ in ws], len(ws))
+                sec0 = time_graph(stream, lambda: [runtime.mmq_xq8(f, w_, dq, dy, k, n, m, stream) for w_ in ws], len(ws))
+                out.append({"fmt": FMT_NAME[f], "M": m, "K": k, "N": n, "us": round(sec * 1e6, 1),
+                            "us_no_workspace": round(sec0 * 1e6, 1), "launch": runtime.mmq_form_ws(f, k, n, m, wsb)})
+                log("mmq small", out[-1])
+                del dx, dq, dy, wsp
+            del ws
     return out
 
 
@@ -641,8 +668,8 @@ def main():
         del mm
 
     if not args.no_configs:
-        out["configs"] = {"mmq_configs2": extras_mmq(stream), "moe_configs3": extras_moe(stream),
-                          "decode_stream_configs4": extras_decode_stream(stream)}
+        out["configs"] = {"mmq_configs2": extras_mmq(stream), "mmq_short_prompts": extras_mmq_small(stream),
+                          "moe_configs3": extras_moe(stream), "decode_stream_configs4": extras_decode_stream(stream)}
 
     if args.sweep:
         sweep = []

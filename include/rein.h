@@ -277,7 +277,7 @@ int rein_matvec_q8_0_splitk(const void *w, const void *xq, float *y_partials, un
 int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                  unsigned out_dim, unsigned p_rows, rein_stream_t s);
 /* The same product with a caller-provided workspace of rein_mmq_workspace_bytes(fmt, in_dim,
- * p_rows) bytes (16-byte aligned; 0 = the format or row count has no use for one, and NULL
+ * p_rows) bytes (16-byte aligned; 0 = the row count has no use for one, and NULL
  * falls back to rein_mmq_xq8).  With it Q4_K above 16 rows runs on the block-scaled fp6
  * matrix instruction: the activations are first brought into operand form in the workspace
  * (one extra launch), then the GEMM streams them from there.  The reference keeps such
@@ -292,11 +292,19 @@ int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_d
  * such as 512 x 17408 whose tiles do not divide over the CUs.  Any size from the minimum on is
  * accepted; below the full size the GEMM runs its one-tile-group-per-workgroup launch.  Results
  * of the two launches can differ in the order of fp32 additions across superblocks (both within
- * the parity bar); each is reproducible from run to run. */
+ * the parity bar); each is reproducible from run to run.
+ * Every other dense format, and Q4_K below the fp6 launch's row count, needs no workspace
+ * (rein_mmq_workspace_min_bytes = 0) and can use one: rein_mmq_workspace_bytes is then 16 MiB,
+ * room for the partial tiles of the same split-tail scheme on the int8 tile (64-token units, or
+ * 32-token units where those would be half empty).  The library takes that launch where a GEMM
+ * has too few workgroup tiles for the machine or a tail that splits well -- 17408 -> 5120 at 64
+ * tokens is 40 workgroup tiles on 256 CUs -- and the plain launch of rein_mmq_xq8 everywhere
+ * else, and whenever the workspace is smaller. */
 size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 /* Which launch rein_mmq_xq8_ws takes for this shape and workspace size: 0 = the int8 launch of
- * rein_mmq_xq8, 1 = fp6 with one token group per workgroup, 2 = fp6 split-tail. */
+ * rein_mmq_xq8, 1 = fp6 with one token group per workgroup, 2 = fp6 split-tail, 3 = int8
+ * split-tail. */
 int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes);
 int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                     unsigned out_dim, unsigned p_rows, void *workspace, size_t workspace_bytes,

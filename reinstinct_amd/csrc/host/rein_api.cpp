@@ -760,6 +760,43 @@ bool mmq6_split_tail(unsigned in_dim, unsigned out_dim, unsigned p_rows)
     return (rounds == 0 && split >= 2) || (rounds == 1 && split >= 4);
 }
 
+// Split-tail launch of the int8 tile (rein_mmq_split_tail in mmq_gemm.h): the same scheme for every dense
+// format, with 64-token units, or 32-token units where a 64-token unit would be half empty (at most 32
+// tokens, or an odd number of 32-token tiles below nine).  The workspace holds one partial tile per
+// workgroup (32 KiB at 64 tokens).  Small GEMMs are what it is for: 17408 -> 5120 at 64 tokens is 40 units
+// on 256 CUs as whole tiles (126 us for Q8_0, 228 for Q6_K) and 480 ranges split twelve ways (46 and 83 us).
+constexpr size_t kSk8PartBytes = (size_t)2 * 16 * 256 * 4;
+struct Sk8Plan { unsigned tm, g, n_unit, n_tail, split; bool take; };
+Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
+{
+    Sk8Plan p{64, kSkGrid, 0, 0, 1, false};
+    const unsigned mode = env_u("REIN_MMQ_SK", 1);
+    if (mode == 0 || p_rows <= 16 || in_dim == 0 || out_dim == 0 || !fmt_tag(fmt) || fmt == REIN_TYPE_Q5_1) return p;
+    if (std::getenv("REIN_MMQ_TM") || std::getenv("REIN_MMQ_N64")) return p;           // a forced tiling
+    const unsigned gg = env_u("REIN_MMQ_SK_GRID", kSkGrid) & ~7u;        // fewer workgroups: tests of several rounds
+    p.g = gg >= 8 && gg <= kSkGrid ? gg : kSkGrid;
+    const unsigned n_tt = (p_rows + 31) / 32;
+    p.tm = 8 * (2 * ((n_tt + 1) / 2) - n_tt) > n_tt ? 32 : 64;           // more than an eighth of the 64-token units' tiles empty
+    if (unsigned forced_tm = env_u("REIN_MMQ_SK_TM", 0)) p.tm = forced_tm == 32 ? 32 : 64;
+    const unsigned n_chunk = (in_dim + 255) / 256;
+    p.n_unit = ((out_dim + 127) / 128) * ((p_rows + p.tm - 1) / p.tm);
+    p.n_tail = p.n_unit % p.g;
+    const unsigned rounds = p.n_unit / p.g;
+    if (p.n_tail) {
+        // behind whole rounds: ranges that fill one workgroup per CU, at most 8; without them both slots, ranges
+        // of two chunks and more, at most 12 (us at 4 / 8 / 10 / 12 ranges, Q8_0 17408 -> 5120 at 64 tokens:
+        // 62 / 54 / 48 / 46; 5120 -> 1024: 20 / 18 / 16 / 16 at 5 / 8 / 10 / 20)
+        const unsigned room = (rounds ? p.g / 2 : p.g) / p.n_tail, cap = rounds ? 8u : std::min(12u, std::max(1u, n_chunk / 2));
+        const unsigned forced = env_u("REIN_MMQ_SK_SPLIT", 0);
+        p.split = std::max(1u, std::min(std::min(forced ? forced : std::min(cap, room), p.g / p.n_tail), n_chunk));
+    }
+    // it pays where the tail decides: no whole round and a tail that splits, or up to three rounds and a tail that
+    // splits four ways (5120 x 17408 at 256 tokens: 117 -> 106 us Q8_0, 210 -> 184 Q6_K; at 512 tokens and more the
+    // mixed launch, whose workgroups drift apart, is level or ahead)
+    p.take = mode == 2 || std::getenv("REIN_MMQ_SK_GRID") || (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4);
+    return p;
+}
+
 }  // namespace
 
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows)
@@ -772,7 +809,11 @@ size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
     // below ~300 rows the int8 launch (more, smaller workgroups in flight) is the faster one:
     // 128 rows 61 vs 93 us, 256 rows 112 vs 122 us, 512 rows 185 vs 177 us at 5120 x 17408
-    if (rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows) == 0) return 0;
+    if (rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows) == 0) {
+        // the int8 launch needs none; with room for its partial tiles it may run as a split-tail launch
+        const bool dense = fmt_tag(fmt) && fmt != REIN_TYPE_Q5_1 && in_dim != 0 && p_rows > 16;
+        return dense && env_u("REIN_MMQ_SK", 1) != 0 ? (size_t)kSkGrid * kSk8PartBytes : 0;
+    }
     return env_u("REIN_MMQ6_SK", 1) != 0 ? sk_workspace_bytes(in_dim, p_rows) : x6_image_bytes(in_dim / 32, p_rows);
 }
 
@@ -781,6 +822,21 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
 {
     const char* who = "rein_mmq_xq8_ws";
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
+    const Sk8Plan sk8 = need == 0 ? sk8_plan(fmt, in_dim, out_dim, p_rows) : Sk8Plan{64, 0, 0, 0, 1, false};
+    if (workspace && sk8.take && workspace_bytes >= (size_t)kSkGrid * kSk8PartBytes) {
+        if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
+        if (int rc = check_dense_fmt(who, fmt)) return rc;
+        if (int rc = check_ptr(who, w, 16, "w")) return rc;
+        if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+        if (int rc = check_ptr(who, y, 4, "y")) return rc;
+        if (int rc = check_ptr(who, workspace, 16, "workspace")) return rc;
+        const unsigned first = sk8.n_unit - sk8.n_tail, n_chunk = (in_dim / 32 + 7) / 8, split = sk8.split;
+        void* a[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&workspace, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&split};
+        if (int rc = launch(std::string("rein_mmq_") + fmt_tag(fmt) + (sk8.tm == 32 ? "_sk32" : "_sk"), sk8.g, 1, 1, 256, 0, s, a)) return rc;
+        if (sk8.n_tail == 0 || split == 1) return 0;
+        void* b[] = {(void*)&workspace, (void*)&y, (void*)&n_chunk, (void*)&out_dim, (void*)&p_rows, (void*)&first, (void*)&split};
+        return launch(sk8.tm == 32 ? "rein_mmq_tail_sum_t32" : "rein_mmq_tail_sum_t64", sk8.n_tail, sk8.tm / 32, 1, 256, 0, s, b);
+    }
     if (!workspace || need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
@@ -860,7 +916,8 @@ int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsig
 int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes)
 {
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    if (need == 0 || workspace_bytes < need) return 0;
+    if (need == 0) return workspace_bytes >= (size_t)kSkGrid * kSk8PartBytes && sk8_plan(fmt, in_dim, out_dim, p_rows).take ? 3 : 0;
+    if (workspace_bytes < need) return 0;
     return workspace_bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows) ? 2 : 1;
 }
 

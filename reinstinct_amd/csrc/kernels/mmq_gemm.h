@@ -1008,11 +1008,13 @@ __device__ __forceinline__ unsigned char* rein_mmq_tile_lds()
 // The contraction of one workgroup tile: wavefront `wave` accumulates tokens tok_base ..
 // tok_end (at most TM) against the 32 weight rows from `row_base` of the matrix at `w`
 // (both may differ from wavefront to wavefront, but are uniform within one).  Ends on a
-// barrier: the tile's LDS is free again when it returns.
+// barrier: the tile's LDS is free again when it returns.  sb_begin / sb_stop (multiples of 8;
+// sb_stop = 0: the end) restrict the sum to the sub-blocks [sb_begin, sb_stop) of the contraction.
 template <int FMT, int TM, int LDSB = rein_mmq_tile_lds_bytes<FMT, TM>()>
 __device__ __forceinline__ void rein_mmq_pipelined_acc(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
                                                        unsigned in_dim, unsigned out_dim, unsigned row_base,
-                                                       unsigned tok_base, unsigned tok_end, rein_v16f (&acc)[TM / 32])
+                                                       unsigned tok_base, unsigned tok_end, rein_v16f (&acc)[TM / 32],
+                                                       unsigned sb_begin = 0u, unsigned sb_stop = 0u)
 {
     using F = Fmt<FMT>;
     using C = MmqChunk<FMT>;
@@ -1060,22 +1062,23 @@ __device__ __forceinline__ void rein_mmq_pipelined_acc(const uint8_t* __restrict
     // behind the store costs nothing in that case and holds if the compiler moved a load.
     typename C::Small small;
     MmqXRegs<TM> xr;
-    rein_mmq_wload<FMT>(wsrc, 0, fmt, 0, n_sub);
-    rein_mmq_wload<FMT>(wsrc, 1, fmt, 4, n_sub);
-    C::fetch_small(small, fmt, rowc, 0, n_sub, h);
-    rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 0);
-    rein_mmq_xstore<TM, C::kSplitK>(lds[0], xr, n_sub, tok_base, tok_end, 0);
-    REIN_WAIT_VMCNT(0);                              // both slots of chunk 0 have landed
+    const unsigned sb_end = sb_stop ? min(sb_stop, n_sub) : n_sub;
+    rein_mmq_wload<FMT>(wsrc, 0, fmt, sb_begin, n_sub);
+    rein_mmq_wload<FMT>(wsrc, 1, fmt, sb_begin + 4u, n_sub);
+    C::fetch_small(small, fmt, rowc, sb_begin, n_sub, h);
+    rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, sb_begin);
+    rein_mmq_xstore<TM, C::kSplitK>(lds[0], xr, n_sub, tok_base, tok_end, sb_begin);
+    REIN_WAIT_VMCNT(0);                              // both slots of the first chunk have landed
     __builtin_amdgcn_sched_barrier(0);               // the next fetch reuses the registers just stored
-    rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, 8 < n_sub ? 8 : 0);
+    rein_mmq_xfetch<TM>(xr, xq, n_sub, tok_base, tok_end, sb_begin + 8u < sb_end ? sb_begin + 8u : sb_begin);
     __syncthreads();
 
     unsigned buf = 0;
-    for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 8, buf ^= 1u) {
+    for (unsigned sb0 = sb_begin; sb0 < sb_end; sb0 += 8, buf ^= 1u) {
         C ck;
         ck.prepare_tuned(small, sb0, n_sub, h);
         const typename C::Small cur = small;
-        const bool more = sb0 + 8 < n_sub, more2 = sb0 + 16 < n_sub;
+        const bool more = sb0 + 8 < sb_end, more2 = sb0 + 16 < sb_end;
         if (more) C::fetch_small(small, fmt, rowc, sb0 + 8, n_sub, h);
         MmqLds<TM>& nxt = lds[buf ^ 1u];
         rein_mmq_chunk_math_rolled<FMT, TM>(lds[buf], wl, wsel, ck, cur, acc, j, h, more, [&](unsigned half) {
@@ -1158,6 +1161,93 @@ __device__ __forceinline__ void rein_mmq_pipelined_mixed(const uint8_t* __restri
     if (rb >= n_rb) return;
     const unsigned t0 = tok64 + tt * 32u;
     rein_mmq_pipelined_tile<FMT, 32, kLds>(w, xq, y, in_dim, out_dim, rb, t0, min(p_rows, t0 + 32u));
+}
+
+// Split-tail launch of the tuned tile: the grid IS the resident slots (gridDim.x = G
+// workgroups, a multiple of 8, two per CU).  Units -- unit u = (row block u / n_tg, TM-token
+// group u % n_tg) -- are dealt in rounds: in round r workgroup `pos` computes unit r G + pos
+// whole.  The U mod G units left after the whole rounds are split along the contraction, `split`
+// workgroups per unit, each a contiguous range of 256-weight chunks, all at the same time; range
+// k of tail unit t stores its partial tile to slot t * split + k of `part`
+// ([tile][register][thread], TM / 32 x 16 x 256 floats), and rein_mmq_tail_sum_body, launched behind
+// this kernel, adds the partial tiles of every tail unit in range order (a fixed order:
+// reproducible).  pos = (blockIdx.x % 8) * G / 8 + blockIdx.x / 8: the workgroups of one XCD
+// hold neighbouring units, so the token groups of a row block -- and the ranges of a tail unit
+// -- meet in one L2 at the same time.
+template <int FMT, int TM>
+__device__ __forceinline__ void rein_mmq_split_tail(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                    float* __restrict__ y, float* __restrict__ part,
+                                                    unsigned in_dim, unsigned out_dim, unsigned p_rows, unsigned split)
+{
+    constexpr int NT = TM / 32;
+    constexpr unsigned kPart = (unsigned)NT * 16u * 256u;                // floats per partial tile
+    const unsigned n_rb = (out_dim + 127u) / 128u, n_tg = (p_rows + TM - 1u) / TM;
+    const unsigned n_chunk = ((in_dim >> 5) + 7u) >> 3, g = gridDim.x, n_unit = n_rb * n_tg;
+    const unsigned pos = (blockIdx.x & 7u) * (g >> 3) + (blockIdx.x >> 3);
+    const unsigned rounds = n_unit / g, n_tail = n_unit - rounds * g;
+    if (blockDim.x != 256u) return;
+
+    // the tail's ranges are dealt evenly over the XCDs, each XCD a contiguous run of them
+    const unsigned n_seg = n_tail * split, per_xcd = (n_seg + 7u) >> 3;
+    const unsigned seg = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    const unsigned lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned j = lane & 31u, h = lane >> 5;
+
+    for (unsigned r = 0; r <= rounds; r++) {                             // whole units, then this workgroup's tail range
+        unsigned u = r * g + pos, c0 = 0u, c1 = n_chunk;
+        float* dst = nullptr;
+        if (r == rounds) {
+            if ((blockIdx.x >> 3) >= per_xcd || seg >= n_seg) return;
+            const unsigned tu = seg / split, k = seg - tu * split;       // tail unit, range within it
+            u = rounds * g + tu;
+            c0 = n_chunk * k / split; c1 = n_chunk * (k + 1u) / split;
+            if (c0 == c1) return;                                        // more ranges than chunks: nothing to add
+            if (split > 1u) dst = part + (size_t)seg * kPart;
+        }
+        const unsigned rb = u / n_tg, tg = u % n_tg;
+        const unsigned tok_base = tg * TM, tok_end = min(p_rows, tok_base + TM);
+        const unsigned row = rb * 128u + wave * 32u + j;
+        rein_v16f acc[NT];
+        rein_mmq_pipelined_acc<FMT, TM>(w, xq, in_dim, out_dim, rb * 128u + wave * 32u, tok_base, tok_end, acc, c0 * 8u, c1 * 8u);
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const unsigned tok = tok_base + t * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+                if (dst) dst[(t * 16 + v) * 256 + threadIdx.x] = acc[t][v];
+                else if (tok < tok_end && row < out_dim) y[(size_t)tok * out_dim + row] = acc[t][v];
+            }
+    }
+}
+
+// y of the tail units = their partial tiles added in range order.  blockIdx.x = tail unit,
+// blockIdx.y = 32-token tile of the unit's NT, 256 threads as in the GEMM (thread -> weight
+// row, register -> token).  `first_unit` = the whole rounds' unit count, n_chunk = chunks of
+// the contraction (an empty range stored nothing).
+template <int NT>
+__device__ __forceinline__ void rein_mmq_tail_sum_body(const float* __restrict__ part, float* __restrict__ y,
+                                                       unsigned n_chunk, unsigned out_dim, unsigned p_rows,
+                                                       unsigned first_unit, unsigned split)
+{
+    constexpr unsigned kPart = (unsigned)NT * 16u * 256u;
+    const unsigned n_tg = (p_rows + 32u * NT - 1u) / (32u * NT);
+    const unsigned tu = blockIdx.x, t = blockIdx.y, u = first_unit + tu, rb = u / n_tg, tg = u % n_tg;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, j = lane & 31u, h = lane >> 5;
+    const unsigned row = rb * 128u + wave * 32u + j;
+    float sum[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) sum[v] = 0.0f;
+    for (unsigned q = 0; q < split; q++) {
+        if (n_chunk * q / split == n_chunk * (q + 1u) / split) continue;
+        const float* src = part + (size_t)(tu * split + q) * kPart;
+#pragma unroll
+        for (int v = 0; v < 16; v++) sum[v] += src[(t * 16 + v) * 256 + threadIdx.x];
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const unsigned tok = tg * 32u * NT + t * 32u + 8 * (v / 4) + 4 * h + (v % 4);
+        if (tok < p_rows && row < out_dim) y[(size_t)tok * out_dim + row] = sum[v];
+    }
 }
 
 // Dense GEMM: grid-stride over (row block, token tile).
@@ -1377,4 +1467,21 @@ __device__ __forceinline__ void rein_mmq_grouped_swiglu(const uint8_t* __restric
     {                                                                                            \
         rein_mmq_grouped_swiglu<FMT>(gate_slab, up_slab, bytes_per_expert, expert_off, tile_off, \
                                      n_expert, xq, out, in_dim, out_dim);                        \
+    }
+
+#define REIN_DEFINE_MMQ_SPLIT_TAIL(name, FMT, TM)                                                \
+    extern "C" __global__ __launch_bounds__(256) REIN_MMQ_OCC void name(                         \
+        const unsigned char* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y, \
+        float* __restrict__ part, unsigned int in_dim, unsigned int out_dim, unsigned int p_rows, \
+        unsigned int split)                                                                      \
+    {                                                                                            \
+        rein_mmq_split_tail<FMT, TM>(w, xq, y, part, in_dim, out_dim, p_rows, split);            \
+    }
+
+#define REIN_DEFINE_MMQ_TAIL_SUM(name, NT)                                                       \
+    extern "C" __global__ __launch_bounds__(256) void name(                                      \
+        const float* __restrict__ part, float* __restrict__ y, unsigned int n_chunk,             \
+        unsigned int out_dim, unsigned int p_rows, unsigned int first_unit, unsigned int split)  \
+    {                                                                                            \
+        rein_mmq_tail_sum_body<NT>(part, y, n_chunk, out_dim, p_rows, first_unit, split);        \
     }

@@ -11,6 +11,8 @@ REIN_DEFINE_MMQ(mmq_gemm_iq4xs_repacked_narrow_f32, REIN_IQ4_XS, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_iq4xs_t32, REIN_IQ4_XS, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_iq4xs_t64, REIN_IQ4_XS, 64)
 REIN_DEFINE_MMQ_MIXED(rein_mmq_iq4xs_mix, REIN_IQ4_XS)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_iq4xs_sk, REIN_IQ4_XS, 64)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_iq4xs_sk32, REIN_IQ4_XS, 32)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_iq4xs, REIN_IQ4_XS)
 
 // the same kernels with the IQ3_S codebook (src/runtime/prefill.rs:528-529)
@@ -19,4 +21,6 @@ REIN_DEFINE_MMQ(mmq_gemm_iq3s_repacked_narrow_f32, REIN_IQ3_S, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_iq3s_t32, REIN_IQ3_S, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_iq3s_t64, REIN_IQ3_S, 64)
 REIN_DEFINE_MMQ_MIXED(rein_mmq_iq3s_mix, REIN_IQ3_S)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_iq3s_sk, REIN_IQ3_S, 64)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_iq3s_sk32, REIN_IQ3_S, 32)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_iq3s, REIN_IQ3_S)

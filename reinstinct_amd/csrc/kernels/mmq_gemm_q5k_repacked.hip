@@ -11,4 +11,6 @@ REIN_DEFINE_MMQ(mmq_gemm_q5k_repacked_narrow_f32, REIN_Q5_K, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_q5k_t32, REIN_Q5_K, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_q5k_t64, REIN_Q5_K, 64)
 REIN_DEFINE_MMQ_MIXED(rein_mmq_q5k_mix, REIN_Q5_K)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_q5k_sk, REIN_Q5_K, 64)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_q5k_sk32, REIN_Q5_K, 32)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q5k, REIN_Q5_K)

@@ -11,4 +11,6 @@ REIN_DEFINE_MMQ(mmq_gemm_q8_0_repacked_narrow_f32, REIN_Q8_0, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_q8_0_t32, REIN_Q8_0, 32)
 REIN_DEFINE_MMQ_PIPE(rein_mmq_q8_0_t64, REIN_Q8_0, 64)
 REIN_DEFINE_MMQ_MIXED(rein_mmq_q8_0_mix, REIN_Q8_0)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_q8_0_sk, REIN_Q8_0, 64)
+REIN_DEFINE_MMQ_SPLIT_TAIL(rein_mmq_q8_0_sk32, REIN_Q8_0, 32)
 REIN_DEFINE_MMQ_DOTS(rein_mmq_dots_q8_0, REIN_Q8_0)
