@@ -835,7 +835,7 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
         if (int rc = launch(std::string("rein_mmq_") + fmt_tag(fmt) + (sk8.tm == 32 ? "_sk32" : "_sk"), sk8.g, 1, 1, 256, 0, s, a)) return rc;
         if (sk8.n_tail == 0 || split == 1) return 0;
         void* b[] = {(void*)&workspace, (void*)&y, (void*)&n_chunk, (void*)&out_dim, (void*)&p_rows, (void*)&first, (void*)&split};
-        return launch(sk8.tm == 32 ? "rein_mmq_tail_sum_t32" : "rein_mmq_tail_sum_t64", sk8.n_tail, sk8.tm / 32, 1, 256, 0, s, b);
+        return launch(sk8.tm == 32 ? "rein_mmq_tail_sum_t32" : "rein_mmq_tail_sum_t64", sk8.n_tail, sk8.tm / 32, 4, 256, 0, s, b);
     }
     if (!workspace || need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
@@ -855,7 +855,7 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
         if (int rc = launch("rein_mmq6_q4k_sk", g, 1, 1, 256, mmq6_lds_bytes(4), s, a)) return rc;
         if (n_tail == 0 || split == 1) return 0;
         void* b[] = {(void*)&part, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows, (void*)&first, (void*)&split};
-        return launch("rein_mmq6_tail_sum", n_tail, 4, 1, 256, 0, s, b);
+        return launch("rein_mmq6_tail_sum", n_tail, 4, 4, 256, 0, s, b);
     }
     unsigned n4, n2;
     mmq6_pick(out_dim, p_rows, &n4, &n2);

@@ -511,8 +511,8 @@ __device__ __forceinline__ void rein_mmq6_split_tail(const uint8_t* __restrict__
     rein_mmq6_tile<4, 0>(w, img, y, nullptr, in_dim, out_dim, rb, span);
 }
 
-// y of the tail units = their partial tiles added in range order.  blockIdx.x = tail unit,
-// blockIdx.y = 32-token tile of the unit's four, 256 threads as in the GEMM (thread -> weight
+// y of the tail units = their partial tiles added in range order.  Grid (tail units, 4, 4): blockIdx.x = tail unit,
+// blockIdx.y = 32-token tile of the unit's four, blockIdx.z = register quad, 256 threads as in the GEMM (thread -> weight
 // row, register -> token).  `first_unit` = the whole rounds' unit count.
 __device__ __forceinline__ void rein_mmq6_tail_sum_body(const float* __restrict__ part, float* __restrict__ y,
                                                         unsigned in_dim, unsigned out_dim, unsigned p_rows,
@@ -523,18 +523,19 @@ __device__ __forceinline__ void rein_mmq6_tail_sum_body(const float* __restrict_
     const unsigned tu = blockIdx.x, t = blockIdx.y, u = first_unit + tu, rb = u / n_tg, tg = u % n_tg;
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, j = lane & 31u, h = lane >> 5;
     const unsigned row = rb * 128u + wave * 32u + j;
-    float sum[16];
-#pragma unroll
-    for (int v = 0; v < 16; v++) sum[v] = 0.0f;
+    // blockIdx.z = which four of the sixteen registers: four times the workgroups, a quarter of the serial loads each
+    const unsigned v0 = 4u * blockIdx.z;
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 4
     for (unsigned q = 0; q < split; q++) {
         if (n_chunk * q / split == n_chunk * (q + 1u) / split) continue;           // an empty range stored nothing
-        const float* src = part + (size_t)(tu * split + q) * kPart;
+        const float* src = part + (size_t)(tu * split + q) * kPart + (t * 16u + v0) * 256u + threadIdx.x;
 #pragma unroll
-        for (int v = 0; v < 16; v++) sum[v] += src[(t * 16 + v) * 256 + threadIdx.x];
+        for (int v = 0; v < 4; v++) sum[v] += src[v * 256];
     }
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-        const unsigned tok = tg * 128u + t * 32u + 8 * (v / 4) + 4 * h + (v % 4);
+    for (int v = 0; v < 4; v++) {
+        const unsigned tok = tg * 128u + t * 32u + 8u * blockIdx.z + 4u * h + v;
         if (tok < p_rows && row < out_dim) y[(size_t)tok * out_dim + row] = sum[v];
     }
 }
