@@ -766,34 +766,55 @@ bool mmq6_split_tail(unsigned in_dim, unsigned out_dim, unsigned p_rows)
 // workgroup (32 KiB at 64 tokens).  Small GEMMs are what it is for: 17408 -> 5120 at 64 tokens is 40 units
 // on 256 CUs as whole tiles (126 us for Q8_0, 228 for Q6_K) and 480 ranges split twelve ways (46 and 83 us).
 constexpr size_t kSk8PartBytes = (size_t)2 * 16 * 256 * 4;
-struct Sk8Plan { unsigned tm, g, n_unit, n_tail, split; bool take; };
-Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
+struct Sk8Plan { unsigned tm, g, n_unit, n_tail, split; bool take; double cost; };
+// One unit width: units, ranges per tail unit, whether the launch pays, and a cost to compare widths by (a
+// 64-token unit costs 1.68 32-token units; workgroups that have a CU to themselves run 1.4 times faster).
+Sk8Plan sk8_width(unsigned tm, unsigned g, unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
-    Sk8Plan p{64, kSkGrid, 0, 0, 1, false};
-    const unsigned mode = env_u("REIN_MMQ_SK", 1);
-    if (mode == 0 || p_rows <= 16 || in_dim == 0 || out_dim == 0 || !fmt_tag(fmt) || fmt == REIN_TYPE_Q5_1) return p;
-    if (std::getenv("REIN_MMQ_TM") || std::getenv("REIN_MMQ_N64")) return p;           // a forced tiling
-    const unsigned gg = env_u("REIN_MMQ_SK_GRID", kSkGrid) & ~7u;        // fewer workgroups: tests of several rounds
-    p.g = gg >= 8 && gg <= kSkGrid ? gg : kSkGrid;
-    const unsigned n_tt = (p_rows + 31) / 32;
-    p.tm = 8 * (2 * ((n_tt + 1) / 2) - n_tt) > n_tt ? 32 : 64;           // more than an eighth of the 64-token units' tiles empty
-    if (unsigned forced_tm = env_u("REIN_MMQ_SK_TM", 0)) p.tm = forced_tm == 32 ? 32 : 64;
+    Sk8Plan p{tm, g, 0, 0, 1, false, 0.0};
     const unsigned n_chunk = (in_dim + 255) / 256;
-    p.n_unit = ((out_dim + 127) / 128) * ((p_rows + p.tm - 1) / p.tm);
-    p.n_tail = p.n_unit % p.g;
-    const unsigned rounds = p.n_unit / p.g;
+    p.n_unit = ((out_dim + 127) / 128) * ((p_rows + tm - 1) / tm);
+    p.n_tail = p.n_unit % g;
+    const unsigned rounds = p.n_unit / g;
     if (p.n_tail) {
         // behind whole rounds: ranges that fill one workgroup per CU, at most 8; without them both slots, ranges
         // of two chunks and more, at most 12 (us at 4 / 8 / 10 / 12 ranges, Q8_0 17408 -> 5120 at 64 tokens:
         // 62 / 54 / 48 / 46; 5120 -> 1024: 20 / 18 / 16 / 16 at 5 / 8 / 10 / 20)
-        const unsigned room = (rounds ? p.g / 2 : p.g) / p.n_tail, cap = rounds ? 8u : std::min(12u, std::max(1u, n_chunk / 2));
+        const unsigned room = (rounds ? g / 2 : g) / p.n_tail, cap = rounds ? 8u : std::min(12u, std::max(1u, n_chunk / 2));
         const unsigned forced = env_u("REIN_MMQ_SK_SPLIT", 0);
-        p.split = std::max(1u, std::min(std::min(forced ? forced : std::min(cap, room), p.g / p.n_tail), n_chunk));
+        p.split = std::max(1u, std::min(std::min(forced ? forced : std::min(cap, room), g / p.n_tail), n_chunk));
     }
-    // it pays where the tail decides: no whole round and a tail that splits, or up to three rounds and a tail that
-    // splits four ways (5120 x 17408 at 256 tokens: 117 -> 106 us Q8_0, 210 -> 184 Q6_K; at 512 tokens and more the
+    // it pays where the tail decides: no whole round and a tail that splits, or one whole round and a tail that
+    // splits four ways (5120 x 17408 at 256 tokens: 117 -> 106 us Q8_0, 210 -> 184 Q6_K; with more rounds the
     // mixed launch, whose workgroups drift apart, is level or ahead)
-    p.take = mode == 2 || std::getenv("REIN_MMQ_SK_GRID") || (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4);
+    p.take = (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4);
+    const unsigned n_seg = p.n_tail * p.split;
+    const double alone = rounds || n_seg >= g ? 1.0 : n_seg <= g / 2 ? 0.71 : 0.71 + 0.29 * (n_seg - g / 2) / (g / 2);
+    p.cost = (tm == 64 ? 1.68 : 1.0) * (rounds + (p.n_tail ? alone / p.split : 0.0));
+    return p;
+}
+Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
+{
+    const Sk8Plan none{64, kSkGrid, 0, 0, 1, false, 0.0};
+    const unsigned mode = env_u("REIN_MMQ_SK", 1);
+    if (mode == 0 || p_rows <= 16 || in_dim == 0 || out_dim == 0 || !fmt_tag(fmt) || fmt == REIN_TYPE_Q5_1) return none;
+    if (std::getenv("REIN_MMQ_TM") || std::getenv("REIN_MMQ_N64")) return none;        // a forced tiling
+    const unsigned gg = env_u("REIN_MMQ_SK_GRID", kSkGrid) & ~7u;        // fewer workgroups: tests of several rounds
+    const unsigned g = gg >= 8 && gg <= kSkGrid ? gg : kSkGrid;
+    const bool force = mode == 2 || std::getenv("REIN_MMQ_SK_GRID");
+    const unsigned n_tt = (p_rows + 31) / 32;
+    const bool half_empty = 8 * (2 * ((n_tt + 1) / 2) - n_tt) > n_tt;   // more than an eighth of the 64-token units' tiles
+    Sk8Plan w64 = sk8_width(64, g, in_dim, out_dim, p_rows), w32 = sk8_width(32, g, in_dim, out_dim, p_rows);
+    if (const unsigned forced_tm = env_u("REIN_MMQ_SK_TM", 0)) {
+        Sk8Plan p = forced_tm == 32 ? w32 : w64;
+        p.take = p.take || force;
+        return p;
+    }
+    if (half_empty) w64.take = false;
+    // 128 tokens x 17408 rows: 544 units of 32 tokens are one round and a tail split eight ways (Q8_0 93 -> 73 us,
+    // Q6_K 143 -> 117), 272 units of 64 tokens fill half the slots and do not split
+    Sk8Plan p = w64.take && (!w32.take || w64.cost <= w32.cost) ? w64 : w32.take ? w32 : half_empty ? w32 : w64;
+    p.take = p.take || force;
     return p;
 }
 
@@ -822,7 +843,7 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
 {
     const char* who = "rein_mmq_xq8_ws";
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    const Sk8Plan sk8 = need == 0 ? sk8_plan(fmt, in_dim, out_dim, p_rows) : Sk8Plan{64, 0, 0, 0, 1, false};
+    const Sk8Plan sk8 = need == 0 ? sk8_plan(fmt, in_dim, out_dim, p_rows) : Sk8Plan{64, 0, 0, 0, 1, false, 0.0};
     if (workspace && sk8.take && workspace_bytes >= (size_t)kSkGrid * kSk8PartBytes) {
         if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
         if (int rc = check_dense_fmt(who, fmt)) return rc;
