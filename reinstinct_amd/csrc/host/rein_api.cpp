@@ -1015,8 +1015,10 @@ int rein_matmul_ws(int fmt, const void* w, const float* x, float* y, unsigned in
     const size_t xq = ((size_t)n_rows * (in_dim / 32) * 40 + 255) & ~(size_t)255;
     if (scratch_bytes < (size_t)n_rows * (in_dim / 32) * 40)
         return fail(REIN_E_BAD_SHAPE, "rein_matmul_ws: scratch smaller than the quantized activations");
-    if (rein_matmul_path(fmt, n_rows) != 2 || rein_mmq_workspace_min_bytes(fmt, in_dim, n_rows) == 0 ||
-        scratch_bytes < xq + rein_mmq_workspace_min_bytes(fmt, in_dim, n_rows))
+    // nothing behind the activations that a workspace launch could use: the plain dispatch
+    const size_t least = rein_mmq_workspace_min_bytes(fmt, in_dim, n_rows);
+    if (rein_matmul_path(fmt, n_rows) != 2 || rein_mmq_workspace_bytes(fmt, in_dim, n_rows) == 0 ||
+        scratch_bytes < xq + std::max<size_t>(least, 16))
         return rein_matmul(fmt, w, x, y, in_dim, out_dim, n_rows, scratch, s);
     if (int rc = rein_quantize_q8(x, scratch, in_dim, n_rows, s)) return rc;
     return rein_mmq_xq8_ws(fmt, w, scratch, y, in_dim, out_dim, n_rows, static_cast<char*>(scratch) + xq, scratch_bytes - xq, s);

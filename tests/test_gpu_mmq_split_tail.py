@@ -137,3 +137,21 @@ def test_the_library_takes_it_for_small_gemms_only_with_the_workspace():
     want = orc.matvec_q8(fmt, sub, in_dim, len(rows), dq.to_host(np.uint8), p_rows)
     assert_close_f32(first[:, rows], want, what="split-tail at 17408 -> 5120, every 37th row")
     assert np.array_equal(first.view(np.uint32), second.view(np.uint32))
+
+
+def test_matmul_ws_carries_the_partial_tile_room():
+    # quantize + GEMM out of one scratch buffer: the scratch size includes the 16 MiB, and the GEMM takes the
+    # same launch and gives the same bits as the two calls
+    fmt, p_rows, in_dim, out_dim = rein.Q6_K, 40, 2048, 512
+    packed = weights(fmt, in_dim, out_dim, seed=9)
+    x = np.random.default_rng(10).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dw, dq = dev(packed), quantized(x)
+    assert runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)) == 3
+    two_calls, _ = run(fmt, dw, dq, in_dim, out_dim, p_rows)
+    sb = runtime.matmul_scratch_bytes(fmt, in_dim, p_rows)
+    assert sb >= p_rows * (in_dim // 32) * 40 + runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
+    scratch = hip.DeviceBuf(sb)
+    dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    runtime.matmul_ws(fmt, dw, dev(x), dy, in_dim, out_dim, p_rows, scratch, sb)
+    hip.synchronize()
+    assert np.array_equal(dy.to_host(np.uint32).reshape(p_rows, out_dim), two_calls.view(np.uint32))
