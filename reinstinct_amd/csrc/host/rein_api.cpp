@@ -820,6 +820,26 @@ Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
 
 }  // namespace
 
+size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
+
+namespace {
+// Which launch a workspace of `bytes` gets: 0 plain int8, 1 fp6 one token group per workgroup, 2 fp6 split-tail,
+// 3 int8 split-tail.  The mixed fp6 launch wants a machine full of 4-tile groups: below three 32-token tiles per
+// resident slot (Q4_K 17408 -> 5120 at 448 tokens: 289 us against 176 on the int8 tile, 5120 -> 5120: 96 against
+// 60; 5120 -> 17408 at 384 tokens, 3.2 tiles per slot: 139 against 142-152) the GEMM stays on the int8 tile, unless
+// REIN_MMQ6_FROM asks for the fp6 path by name.
+int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t bytes)
+{
+    const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
+    if (need != 0 && bytes >= need) {
+        if (bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows)) return 2;
+        const unsigned long long tiles = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 31) / 32);
+        if (tiles >= 3ull * kSkGrid || std::getenv("REIN_MMQ6_FROM") || std::getenv("REIN_MMQ6_N4") || std::getenv("REIN_MMQ6_N2")) return 1;
+    }
+    return bytes >= (size_t)kSkGrid * kSk8PartBytes && sk8_plan(fmt, in_dim, out_dim, p_rows).take ? 3 : 0;
+}
+}  // namespace
+
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
     if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < env_u("REIN_MMQ6_FROM", 320)) return 0;
@@ -843,8 +863,11 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
 {
     const char* who = "rein_mmq_xq8_ws";
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    const Sk8Plan sk8 = need == 0 ? sk8_plan(fmt, in_dim, out_dim, p_rows) : Sk8Plan{64, 0, 0, 0, 1, false, 0.0};
-    if (workspace && sk8.take && workspace_bytes >= (size_t)kSkGrid * kSk8PartBytes) {
+    if (workspace && need != 0 && workspace_bytes < need)
+        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace of " + std::to_string(workspace_bytes) + " bytes, rein_mmq_workspace_min_bytes asks for " + std::to_string(need));
+    const int form = workspace ? mmq_form(fmt, in_dim, out_dim, p_rows, workspace_bytes) : 0;
+    if (form == 3) {
+        const Sk8Plan sk8 = sk8_plan(fmt, in_dim, out_dim, p_rows);
         if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
         if (int rc = check_dense_fmt(who, fmt)) return rc;
         if (int rc = check_ptr(who, w, 16, "w")) return rc;
@@ -858,15 +881,13 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
         void* b[] = {(void*)&workspace, (void*)&y, (void*)&n_chunk, (void*)&out_dim, (void*)&p_rows, (void*)&first, (void*)&split};
         return launch(sk8.tm == 32 ? "rein_mmq_tail_sum_t32" : "rein_mmq_tail_sum_t64", sk8.n_tail, sk8.tm / 32, 4, 256, 0, s, b);
     }
-    if (!workspace || need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (form == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     if (int rc = check_ptr(who, workspace, 16, "workspace")) return rc;
-    if (workspace_bytes < need)
-        return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace of " + std::to_string(workspace_bytes) + " bytes, rein_mmq_workspace_min_bytes asks for " + std::to_string(need));
-    if (workspace_bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows)) {
+    if (form == 2) {
         char* base = static_cast<char*>(workspace);
         float* part = reinterpret_cast<float*>(base + sk_image_bytes(in_dim, p_rows));
         const unsigned split = sk_split(in_dim, out_dim, p_rows), g = sk_grid();
@@ -937,9 +958,8 @@ int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsig
 int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes)
 {
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    if (need == 0) return workspace_bytes >= (size_t)kSkGrid * kSk8PartBytes && sk8_plan(fmt, in_dim, out_dim, p_rows).take ? 3 : 0;
-    if (workspace_bytes < need) return 0;
-    return workspace_bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows) ? 2 : 1;
+    if (need != 0 && workspace_bytes < need) return 0;                   // rein_mmq_xq8_ws refuses such a workspace
+    return mmq_form(fmt, in_dim, out_dim, p_rows, workspace_bytes);
 }
 
 int rein_mmq_tile_plan_ws(int fmt, unsigned out_dim, unsigned p_rows, unsigned* n4, unsigned* n2)
