@@ -1288,6 +1288,41 @@ __device__ __forceinline__ unsigned rein_mmq_tile_expert(const int* __restrict__
     return n_le - 1u;                              // tile_off[0] = 0 <= tile: at least one
 }
 
+// The same with the expert's rows in the same round trip: every lane also loads its experts' expert_off[e],
+// expert_off[e + 1] and keeps tile_off[e], and the three words of the expert found are read out of the lane
+// that holds them -- one memory latency in front of a workgroup's first fetch instead of two.  Up to 256
+// experts; beyond, the words are loaded once the expert is known.
+struct ReinTileRows { unsigned expert, tok_base, tok_end; };
+__device__ __forceinline__ ReinTileRows rein_mmq_tile_rows(const int* __restrict__ tile_off, const int* __restrict__ expert_off,
+                                                           unsigned n_expert, unsigned tile)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    if (n_expert > 256u) {
+        const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
+        return ReinTileRows{lo, (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u, (unsigned)expert_off[lo + 1]};
+    }
+    int to[4], e0[4], e1[4];
+    unsigned n_le = 0;
+#pragma unroll
+    for (unsigned k = 0; k < 4u; k++) {
+        const unsigned e = min(k * 64u + lane, n_expert - 1u);
+        to[k] = tile_off[e]; e0[k] = expert_off[e]; e1[k] = expert_off[e + 1u];
+    }
+#pragma unroll
+    for (unsigned k = 0; k < 4u; k++) {
+        const bool le = k * 64u + lane < n_expert && (unsigned)to[k] <= tile;
+        n_le += (unsigned)__popcll(__ballot(le));
+    }
+    const unsigned lo = n_le - 1u, src = lo & 63u;                       // tile_off[0] = 0 <= tile: at least one
+    int t = 0, a = 0, b = 0;
+#pragma unroll
+    for (unsigned k = 0; k < 4u; k++) {
+        const int tk = __builtin_amdgcn_readlane(to[k], src), ak = __builtin_amdgcn_readlane(e0[k], src), bk = __builtin_amdgcn_readlane(e1[k], src);
+        if ((lo >> 6) == k) { t = tk; a = ak; b = bk; }
+    }
+    return ReinTileRows{lo, (unsigned)a + (tile - (unsigned)t) * 32u, (unsigned)b};
+}
+
 template <int FMT>
 __device__ __forceinline__ void rein_mmq_grouped(const uint8_t* __restrict__ slab, unsigned bytes_per_expert,
                                                  const int* __restrict__ expert_off, const int* __restrict__ tile_off,
@@ -1335,9 +1370,8 @@ __device__ __forceinline__ void rein_mmq_grouped_one(const uint8_t* __restrict__
     const unsigned n_tile = (unsigned)tile_off[n_expert], per_xcd = (n_tile + 7u) >> 3;
     const unsigned tile = xcd * per_xcd + k / per, rb = (k % per) % n_rb, z = (k % per) / n_rb;
     if (blockDim.x != 256u || k / per >= per_xcd || tile >= n_tile) return;
-    const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
-    const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
-    const unsigned tok_end = (unsigned)expert_off[lo + 1];
+    const ReinTileRows tr = rein_mmq_tile_rows(tile_off, expert_off, n_expert, tile);
+    const unsigned lo = tr.expert, tok_base = tr.tok_base, tok_end = tr.tok_end;
     if (tok_base >= tok_end) return;
     const uint8_t* slab = z ? slab1 : slab0;
     rein_mmq_pipelined_tile<FMT, 32>(slab + (size_t)lo * bytes_per_expert, xq, z ? y1 : y0, in_dim, out_dim, rb,
@@ -1370,9 +1404,8 @@ __device__ __forceinline__ void rein_mmq_grouped_swiglu(const uint8_t* __restric
     const unsigned n_tile = (unsigned)tile_off[n_expert], per_xcd = (n_tile + 7u) >> 3;
     const unsigned tile = xcd * per_xcd + k / n_cb, cb = k % n_cb;
     if (blockDim.x != 256u || k / n_cb >= per_xcd || tile >= n_tile) return;
-    const unsigned lo = rein_mmq_tile_expert(tile_off, n_expert, tile);
-    const unsigned tok_base = (unsigned)expert_off[lo] + (tile - (unsigned)tile_off[lo]) * 32u;
-    const unsigned tok_end = min((unsigned)expert_off[lo + 1], tok_base + 32u);
+    const ReinTileRows tr = rein_mmq_tile_rows(tile_off, expert_off, n_expert, tile);
+    const unsigned lo = tr.expert, tok_base = tr.tok_base, tok_end = min(tr.tok_end, tok_base + 32u);
     if (tok_base >= tok_end) return;
 
     const unsigned lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
