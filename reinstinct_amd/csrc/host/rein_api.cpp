@@ -1491,6 +1491,9 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
         const int32_t* inv = (const int32_t*)(base + w.inv);
         void* a[] = {(void*)&sorted, (void*)&inv, (void*)&ids, (void*)&weights, (void*)&down_exps_s, (void*)&out,
                      (void*)&sh.hidden, (void*)&sh.n_used};
+        // four columns per thread where the rows allow 128-bit accesses (the same bits)
+        if (sh.hidden % 4 == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)sorted & 15) == 0)
+            return launch("rein_moe_combine_sorted4_f32", (sh.hidden / 4 + 127) / 128, sh.n_tok, 1, 128, 0, s, a);
         return launch("rein_moe_combine_sorted_f32", (sh.hidden + 255) / 256, sh.n_tok, 1, 256, 0, s, a);
     }
 }
