@@ -155,3 +155,29 @@ def test_matmul_ws_carries_the_partial_tile_room():
     runtime.matmul_ws(fmt, dw, dev(x), dy, in_dim, out_dim, p_rows, scratch, sb)
     hip.synchronize()
     assert np.array_equal(dy.to_host(np.uint32).reshape(p_rows, out_dim), two_calls.view(np.uint32))
+
+
+def test_split_tail_replays_from_a_graph():
+    # the two launches (GEMM with partial tiles, tail sum) captured once and replayed with the program's own
+    # eager work between the replays: every replay gives the eager bits
+    fmt, p_rows, in_dim, out_dim = rein.Q8_0, 48, 2048, 640
+    packed = weights(fmt, in_dim, out_dim, seed=12)
+    x = np.random.default_rng(13).standard_normal((p_rows, in_dim)).astype(np.float32)
+    dw, dq = dev(packed), quantized(x)
+    ws_bytes = runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
+    assert runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, ws_bytes) == 3
+    eager, _ = run(fmt, dw, dq, in_dim, out_dim, p_rows)
+    stream = hip.Stream()
+    ws = hip.DeviceBuf(ws_bytes)
+    dy = dev(np.zeros(p_rows * out_dim, np.float32))
+    stream.begin_capture()
+    runtime.mmq_xq8_ws(fmt, dw, dq, dy, in_dim, out_dim, p_rows, ws, ws_bytes, stream)
+    graph = stream.end_capture()
+    ex = graph.instantiate()
+    for replay in range(3):
+        dy.copy_from_host(np.zeros(p_rows * out_dim, np.float32))
+        other, _ = run(fmt, dw, dq, in_dim, out_dim, p_rows)               # eager work between the replays
+        assert np.array_equal(other.view(np.uint32), eager.view(np.uint32))
+        ex.launch(stream)
+        stream.synchronize()
+        assert np.array_equal(dy.to_host(np.uint32).reshape(p_rows, out_dim), eager.view(np.uint32)), f"replay {replay}"
