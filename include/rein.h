@@ -280,8 +280,9 @@ int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_d
  * p_rows) bytes (16-byte aligned; 0 = the row count has no use for one, and NULL
  * falls back to rein_mmq_xq8).  With it Q4_K from 320 rows up runs on the block-scaled fp6
  * matrix instruction: the activations are first brought into operand form in the workspace
- * (one extra launch), then the GEMM streams them from there (GEMMs below three 32-token tiles
- * per resident workgroup that do not take the split-tail form below stay on the int8 tile).  The reference keeps such
+ * (one extra launch), then the GEMM streams them from there (GEMMs of less than 2.8e10 operations
+ * 2 M N K, about 50 us, and GEMMs below three 32-token tiles per resident workgroup that do not take
+ * the split-tail form below stay on the int8 tile).  The reference keeps such
  * scratch in its PrefillGemm object (src/runtime/prefill.rs:479-495); here the caller owns
  * it, so nothing allocates and the call can be captured into a graph.  Calls that share a
  * workspace must be ordered on one stream.
@@ -299,8 +300,9 @@ int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_d
  * room for the partial tiles of the same split-tail scheme on the int8 tile (64-token units, or
  * 32-token units where those would be half empty).  The library takes that launch where a GEMM
  * has too few workgroup tiles for the machine or a tail that splits well -- 17408 -> 5120 at 64
- * tokens is 40 workgroup tiles on 256 CUs -- and the plain launch of rein_mmq_xq8 everywhere
- * else, and whenever the workspace is smaller. */
+ * tokens is 40 workgroup tiles on 256 CUs -- and its own estimate puts it ahead of the plain
+ * launch with the second launch counted; the plain launch of rein_mmq_xq8 everywhere else, and
+ * whenever the workspace is smaller. */
 size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 /* Which launch rein_mmq_xq8_ws takes for this shape and workspace size: 0 = the int8 launch of

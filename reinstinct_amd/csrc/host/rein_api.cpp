@@ -811,6 +811,24 @@ Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
         return p;
     }
     if (half_empty) w64.take = false;
+    // Without a whole round the launch competes with the plain one, whose workgroups are then all resident at
+    // once.  Both are priced in chunk times of a 32-token workgroup that shares its CU with one other (alone
+    // 0.71, three on a CU 1.75 each, in between by the fill; a 64-token unit 1.68 of a 32-token one), plus three
+    // chunk times for the second launch and the partial tiles.  Over 282 measured shapes x formats that removes
+    // the losses of 5-46 % (1536 -> 6144 at 320 tokens: 26.5 us against 18.2 plain; 2048 -> 1536 at 512 tokens:
+    // 21-23 against 17-19) and gives up two gains of 3-5 %.  Q6_K and Q5_K, whose chunk costs more against the
+    // same second launch, gained in every measured shape and are left alone.
+    if (!force && fmt != REIN_TYPE_Q6_K && fmt != REIN_TYPE_Q5_K) {
+        const unsigned n_chunk = (in_dim + 255) / 256, n_rb = (out_dim + 127) / 128;
+        const unsigned long long wg32 = (unsigned long long)n_rb * n_tt, u64 = (unsigned long long)n_rb * ((p_rows + 63) / 64);
+        double plain;
+        if (wg32 <= kCUs) plain = 0.71;
+        else if (wg32 <= 2ull * kCUs) plain = 0.71 + 0.29 * (double)(wg32 - kCUs) / kCUs;
+        else if (wg32 <= 3ull * kCUs) plain = 1.0 + 0.75 * (double)(wg32 - 2ull * kCUs) / kCUs;
+        else { const unsigned long long r = u64 % kSkGrid; plain = 1.68 * ((double)(u64 / kSkGrid) + (r == 0 ? 0.0 : r <= kCUs ? 0.71 : 1.0)); }
+        for (Sk8Plan* w : {&w64, &w32})
+            if (w->take && w->n_unit < g && !(w->cost * n_chunk + 3.0 < plain * n_chunk)) w->take = false;
+    }
     // 128 tokens x 17408 rows: 544 units of 32 tokens are one round and a tail split eight ways (Q8_0 93 -> 73 us,
     // Q6_K 143 -> 117), 272 units of 64 tokens fill half the slots and do not split
     Sk8Plan p = w64.take && (!w32.take || w64.cost <= w32.cost) ? w64 : w32.take ? w32 : half_empty ? w32 : w64;
@@ -831,10 +849,15 @@ namespace {
 int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t bytes)
 {
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    if (need != 0 && bytes >= need) {
+    const bool asked = std::getenv("REIN_MMQ6_FROM") || std::getenv("REIN_MMQ6_N4") || std::getenv("REIN_MMQ6_N2");
+    // The fp6 launches carry the image kernel in front and, split-tail, the sum behind: below about 50 us of
+    // GEMM (2 M N K < 2.8e10) that costs more than the tile saves (768 -> 2048 at 512 tokens: 21 us against 9,
+    // 2048 -> 1536: 26 against 19, 1536 -> 6144: 38 against 24; 5120 -> 2560 at 1536 tokens, 4.0e10: 90 against 139).
+    const bool large = 2.0 * p_rows * (double)out_dim * in_dim >= 2.8e10;
+    if (need != 0 && bytes >= need && (large || asked)) {
         if (bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows)) return 2;
         const unsigned long long tiles = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 31) / 32);
-        if (tiles >= 3ull * kSkGrid || std::getenv("REIN_MMQ6_FROM") || std::getenv("REIN_MMQ6_N4") || std::getenv("REIN_MMQ6_N2")) return 1;
+        if (tiles >= 3ull * kSkGrid || asked) return 1;
     }
     return bytes >= (size_t)kSkGrid * kSk8PartBytes && sk8_plan(fmt, in_dim, out_dim, p_rows).take ? 3 : 0;
 }

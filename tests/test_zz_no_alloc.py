@@ -36,18 +36,20 @@ def run_pair(fmt, p_rows, in_dim, out_dim, seed):
 def test_no_alloc_entry_matches_the_workspace_entry_twice_in_a_row():
     init()
     hip.set_device(0)
-    # Q4_K from 320 rows up and three 32-token tiles per resident workgroup (here 147 row blocks x 16 and x 14
-    # token tiles) runs out of the fixed array; the second call is smaller than the first
-    assert run_pair(rein.Q4_K, 512, 512, 18816, seed=1) > 0
-    assert runtime.mmq_form_ws(rein.Q4_K, 512, 18816, 512, runtime.mmq_workspace_min_bytes(rein.Q4_K, 512, 512)) == 1
-    assert run_pair(rein.Q4_K, 448, 512, 18816, seed=2) > 0
-    assert runtime.mmq_form_ws(rein.Q4_K, 512, 18816, 448, runtime.mmq_workspace_min_bytes(rein.Q4_K, 512, 448)) == 1
+    # Q4_K from 320 rows up, three 32-token tiles per resident workgroup (here 112 row blocks x 16 and x 14 token
+    # tiles) and 2 M N K of 2.8e10 and more runs out of the fixed array; the second call is smaller than the first
+    big = (2304, 14336)
+    assert run_pair(rein.Q4_K, 512, *big, seed=1) > 0
+    assert runtime.mmq_form_ws(rein.Q4_K, *big, 512, runtime.mmq_workspace_min_bytes(rein.Q4_K, big[0], 512)) == 1
+    assert run_pair(rein.Q4_K, 448, *big, seed=2) > 0
+    assert runtime.mmq_form_ws(rein.Q4_K, *big, 448, runtime.mmq_workspace_min_bytes(rein.Q4_K, big[0], 448)) == 1
     # launches that use no scratch go straight through: other formats, few rows, GEMMs too small for the fp6 launch
     assert run_pair(rein.Q6_K, 64, 512, 136, seed=3) == 0
     assert run_pair(rein.Q4_K, 40, 512, 136, seed=4) == 0
     assert run_pair(rein.Q4_K, 448, 2048, 264, seed=6) > 0
+    assert runtime.mmq_form_ws(rein.Q4_K, 2048, 264, 448, runtime.mmq_workspace_min_bytes(rein.Q4_K, 2048, 448)) == 0
     # and once more the larger shape, after the smaller ones
-    assert run_pair(rein.Q4_K, 512, 512, 18816, seed=5) > 0
+    assert run_pair(rein.Q4_K, 512, *big, seed=5) > 0
 
 
 def test_no_alloc_entry_refuses_what_the_fixed_array_cannot_hold():
