@@ -233,6 +233,10 @@ unsigned skinny_from_rows(int fmt)
 //           5..8 rows below 16384 rows     13.3 -> 12.4, 32.4 -> 32.3 (34816 rows: 35.3 vs 45.6, stays)
 // The formats with a cheap unpack (Q4_K, Q4_0, Q8_0, IQ3_S) stay on dot4 / skinny MMQ
 // (Q4_K 4 rows at 34816 output rows: skinny 29.6, this 34.3).
+// ... except at 3-4 rows against 8192-20480 output rows, where the skinny MMQ's 32-row tiles do not fill the
+// machine as evenly as four-row groups do (us, skinny -> this: Q4_K 4096 -> 14336 17.7 -> 14.0, 5120 -> 17408 21.8 ->
+// 19.4, 8192 -> 8192 19.7 -> 17.0; Q4_0 17.0 -> 13.1, 21.1 -> 17.4, 18.4 -> 17.2; Q8_0 23.0 -> 21.0, 25.9 -> 25.6, 25.5 ->
+// 21.3; level at 7168 rows, behind at 5120 and 34816).
 bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
 {
     const unsigned forced = env_u("REIN_QUAD_FROM", 0);
@@ -242,8 +246,29 @@ bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
     case REIN_TYPE_Q6_K:   return true;
     case REIN_TYPE_Q5_K:
     case REIN_TYPE_IQ4_XS: return n_rows <= 4 || out_dim < 16384;
+    case REIN_TYPE_Q4_K:
+    case REIN_TYPE_Q4_0:
+    case REIN_TYPE_Q8_0:   return n_rows <= 4 && out_dim >= 8192 && out_dim <= 20480;
     default:               return false;
     }
+}
+
+// Small matrices stay on dot4 at every row count: the matrix-core kernels hand out 32-row tiles or 16-row
+// workgroups, too few of them for 256 CUs, and carry a pipeline fill that a 5 us launch does not earn back.
+// One run of all kernel families over 12 shapes x 6 formats (us, matrix-core choice -> dot4): 5120 -> 1024 at 3-4
+// rows Q4_K 8.6 -> 4.8, Q8_0 9.1 -> 5.2, Q5_K 8.4 -> 5.6, IQ4_XS 8.5 -> 4.9, Q6_K 10.8 -> 7.9; 5120 -> 2048 8.8 -> 6.3
+// ... 11.2 -> 9.7; 2048 -> 1536 6.0 -> 3.5.  Beyond 2048 output rows only the formats of the skinny MMQ gain, up to
+// 2^24 weights (4096 -> 4096 Q4_K 9.0 -> 7.1, Q8_0 11.0 -> 8.6; 2048 -> 5120 6.5 -> 5.5; 5120 -> 5120: 9.8 against
+// 11.6, stays), the 4x4x4 kernel of the others is level there (Q5_K 2048 -> 5120 5.8 = 5.8).  At 5-8 rows dot4 is
+// ahead up to about six million weights (5120 -> 1024 Q4_K 9.5 -> 7.7, Q5_K 9.8 -> 6.8; 2048 -> 1536 6.2 -> 5.1;
+// 5120 -> 2048 9.7 against 10.7, stays).
+bool small_for_matrix_cores(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    if (n_rows < 3 || std::getenv("REIN_QUAD_FROM") || std::getenv("REIN_SKINNY_FROM")) return false;
+    const unsigned long long weights = (unsigned long long)in_dim * out_dim;
+    if (n_rows > 4) return weights <= (6ull << 20);
+    const bool quad_family = fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS;
+    return out_dim <= 2048 || (!quad_family && weights <= (1ull << 24));
 }
 
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
@@ -255,14 +280,15 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    if (use_quad(fmt, out_dim, n_rows)) {
+    const bool small = small_for_matrix_cores(fmt, in_dim, out_dim, n_rows);
+    if (!small && use_quad(fmt, out_dim, n_rows)) {
         // four output rows per wavefront, four wavefronts per workgroup
         const std::string name = std::string("rein_mvq_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
         void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
         return launch(name, ((out_dim + 3) / 4 + 3) / 4, 1, 1, 256, 0, s, args);
     }
     // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
-    if (n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (!small && n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(fmt, out_dim, b);
     const unsigned wpb = 4;

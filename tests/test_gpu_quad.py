@@ -67,10 +67,53 @@ def test_quad_matvec_ragged_contraction(fmt, in_dim, monkeypatch):
 
 @pytest.mark.parametrize("fmt,n_rows", [(rein.Q6_K, 3), (rein.Q6_K, 8), (rein.Q5_K, 4), (rein.IQ4_XS, 3), (rein.IQ4_XS, 6)])
 def test_default_dispatch_at_benchmark_width(fmt, n_rows):
-    # the row counts the library sends to these kernels by itself, at the K of the decode shapes
-    in_dim, out_dim = 5120, 1100
+    # the row counts the library sends to these kernels by itself, at the K of the decode shapes (a matrix
+    # large enough that the library does not keep it on dot4)
+    in_dim, out_dim = 5120, 4100
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
     want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
     assert_close_f32(run(fmt, packed, xq, in_dim, out_dim, n_rows), want, what="default dispatch")
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q8_0, rein.Q4_0])
+def test_mid_width_matrices_take_these_kernels_at_3_and_4_rows(fmt, monkeypatch):
+    # 8192..20480 output rows: the library's own choice for the formats that otherwise run the skinny MMQ;
+    # the same bits as with the kernels forced, and the oracle's values
+    in_dim, out_dim = 2304, 8200
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in (3, 4):
+        print("quad by default", fmt, n_rows, flush=True)
+        xq = orc.quantize_q8(np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32))
+        got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+        assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what=f"fmt {fmt} rows {n_rows}")
+        monkeypatch.setenv("REIN_QUAD_FROM", "1")
+        forced = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+        monkeypatch.delenv("REIN_QUAD_FROM")
+        assert np.array_equal(bits(got), bits(forced)), "the default launch is not the 4x4x4 kernel"
+
+
+@pytest.mark.parametrize("fmt", DENSE)
+def test_small_matrices_stay_on_dot4(fmt, monkeypatch):
+    # up to 2^24 weights at 3-4 rows and 6 * 2^20 at 5-8 the library keeps the dot4 kernels: the same bits as
+    # with both matrix-core families switched off, and the oracle's values
+    in_dim, out_dim = 2048, 1536
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + 1)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in (3, 4, 8):
+        print("dot4 by default", fmt, n_rows, flush=True)
+        xq = orc.quantize_q8(np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32))
+        got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+        assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what=f"fmt {fmt} rows {n_rows}")
+        monkeypatch.setenv("REIN_QUAD_FROM", "99")
+        monkeypatch.setenv("REIN_SKINNY_FROM", "99")
+        forced = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+        monkeypatch.delenv("REIN_QUAD_FROM")
+        monkeypatch.delenv("REIN_SKINNY_FROM")
+        assert np.array_equal(bits(got), bits(forced)), "the default launch is not a dot4 kernel"
