@@ -248,7 +248,7 @@ def mmq_kernel_name(fmt, in_dim, out_dim, p_rows):
     if form == 1:
         n4, n2 = runtime.mmq_tile_plan_ws(fmt, out_dim, p_rows)
         return f"rein_mmq6_prep + rein_mmq6_{tag}_mix (n4 = {n4}, n2 = {n2})"
-    n64 = runtime.mmq_tile_plan(fmt, out_dim, p_rows)
+    n64 = runtime.mmq_tile_plan(fmt, in_dim, out_dim, p_rows)
     return f"rein_mmq_{tag}_mix (n64 = {n64})" if n64 else f"rein_mmq_{tag}_t32"
 
 

@@ -281,8 +281,8 @@ int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_d
  * falls back to rein_mmq_xq8).  With it Q4_K from 320 rows up runs on the block-scaled fp6
  * matrix instruction: the activations are first brought into operand form in the workspace
  * (one extra launch), then the GEMM streams them from there (GEMMs of less than 2.8e10 operations
- * 2 M N K, about 50 us, and GEMMs below three 32-token tiles per resident workgroup that do not take
- * the split-tail form below stay on the int8 tile).  The reference keeps such
+ * 2 M N K, about 50 us, and GEMMs whose 128-token workgroups do not come out even over the CUs and
+ * that do not take the split-tail form below stay on the int8 tile).  The reference keeps such
  * scratch in its PrefillGemm object (src/runtime/prefill.rs:479-495); here the caller owns
  * it, so nothing allocates and the call can be captured into a graph.  Calls that share a
  * workspace must be ordered on one stream.
@@ -344,7 +344,7 @@ int rein_matmul_path(int fmt, unsigned n_rows);
  * tiles per 128-row block; the remaining tokens run in 32-token tiles (0: all of them).
  * The reference launches one fixed tile shape (prefill.rs:536-560); this choice has no
  * counterpart there.  <0 on error. */
-int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows);
+int rein_mmq_tile_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows);
 
 /* Debug / parity: per-block int32 dots exactly as the kernels form them.
  * out [n_rows][out_dim][in_dim/32][parts], parts = rein_block_dot_parts(fmt)

@@ -92,7 +92,7 @@ SIGNATURES = {
     "rein_matmul_scratch_bytes": (_sz, [_i, _u, _u]),
     "rein_matmul_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
     "rein_matmul_path": (_i, [_i, _u]),
-    "rein_mmq_tile_plan": (_i, [_i, _u, _u]),
+    "rein_mmq_tile_plan": (_i, [_i, _u, _u, _u]),
     "rein_block_dot_parts": (_i, [_i]),
     "rein_block_dots": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _i, _vp]),
     "rein_moe_topk": (_i, [_vp, _u, _u, _u, _vp, _vp, _vp]),

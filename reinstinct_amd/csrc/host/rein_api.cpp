@@ -576,29 +576,53 @@ int rein_matvec_q8_0_splitk(const void* w, const void* xq, float* y_partials, un
 }
 
 // How many 64-token tiles per row block the MMQ launch uses (0 = the 32-token kernel).
-// A 64-token tile costs 1.68 times a 32-token tile of the 32-token kernel (one weight unpack
+// A 64-token tile costs c64 times a 32-token tile of the 32-token kernel (one weight unpack
 // feeds two MFMA tiles); a 32-token tile inside the mixed kernel costs 1.17 (two workgroups
-// per CU there, three in its own kernel) -- ratios measured at 5120 x 17408 and 5120 x 5120.
+// per CU there, three in its own kernel).  c64 is per format, from the 32- and 64-token kernels
+// at 1024 and 2048 tokens against 17408 and 34816 rows: Q8_0 1.56, Q6_K and Q5_K 1.74, and Q4_K,
+// whose 32-token kernel is the leanest, 2.1 -- unless the rows of the slab are padded (a
+// power-of-two sub-block count), where every fetch of a weight tile straddles cache lines and
+// sharing it between two token tiles is worth more: 0.3 less for every format (Q4_K 1.77 at
+// 8192 x 8192 and 4096 x 14336).
 // Workgroups are handed to CUs in launch order, 64-token tiles first; a CU's finish time is
 // the sum of what it was handed.  The candidate with the earliest last finish wins.  Up to
 // three 32-token workgroups per CU (everything resident at once) nothing beats the fine
 // grain.  The estimate walks at most a few thousand workgroups, so it is kept per shape.
-static unsigned mmq_pick_n64(unsigned out_dim, unsigned p_rows)
+static double mmq_c64(int fmt, unsigned in_dim)
+{
+    const unsigned n_sub = in_dim / 32;
+    const double padded = n_sub != 0 && (n_sub & (n_sub - 1)) == 0 ? 0.3 : 0.0;
+    switch (fmt) {
+    case REIN_TYPE_Q8_0: return 1.56 - padded;
+    case REIN_TYPE_Q6_K:
+    case REIN_TYPE_Q5_K: return 1.74 - padded;
+    case REIN_TYPE_Q4_K: return 2.1 - padded;
+    default:             return 1.68 - padded;
+    }
+}
+static unsigned mmq_pick_n64(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
     const unsigned n_rb = (out_dim + 127) / 128, t32 = (p_rows + 31) / 32;
     const unsigned long long wg32 = (unsigned long long)n_rb * t32;
-    if (p_rows < 64 || wg32 <= 3ull * kCUs) return 0;
+    if (p_rows < 64 || wg32 <= 2ull * kCUs) return 0;
+    const double c64 = mmq_c64(fmt, in_dim), c32mix = 1.17;
+    if (wg32 <= 3ull * kCUs) {
+        // everything resident at once either way: three 32-token workgroups on the fullest CUs (1.75 each)
+        // against one or two 64-token ones (0.71 or 1.0 x c64) -- Q8_0 8192 x 8192 at 384 tokens 155 -> 133 us,
+        // 17408 -> 5120 at 512 tokens 274 -> 251; Q4_K stays (119 against 140)
+        const unsigned long long u64 = (unsigned long long)n_rb * ((p_rows + 63) / 64);
+        return c64 * (u64 <= kCUs ? 0.71 : 1.0) < 0.97 * 1.75 ? p_rows / 64 : 0;
+    }
     static std::mutex mu;
     static std::unordered_map<unsigned long long, unsigned> memo;
-    const unsigned long long key = ((unsigned long long)out_dim << 32) | p_rows;
+    const unsigned long long key = ((unsigned long long)out_dim << 32) | ((unsigned long long)p_rows << 8) | (unsigned)(c64 * 100.0 - 100.0);
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = memo.find(key);
         if (it != memo.end()) return it->second;
     }
-    const double c64 = 1.68, c32mix = 1.17;
     const unsigned a_max = p_rows / 64;
-    unsigned best_n64 = a_max;                                 // very large grids: granularity no longer matters
+    unsigned best_n64 = c64 > 2.0 ? 0 : a_max;                 // very large grids: granularity no longer matters
     if (wg32 <= 64ull * kCUs) {
         double best = std::ceil((double)wg32 / kCUs);          // the 32-token kernel
         best_n64 = 0;
@@ -636,11 +660,14 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     // Token tiles: 32 tokens (rein_mmq_<fmt>_t32, three workgroups per CU) or the mixed launch
     // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).
     const unsigned n_rb = (out_dim + 127) / 128;
-    unsigned n64 = mmq_pick_n64(out_dim, p_rows);
+    unsigned n64 = mmq_pick_n64(fmt, in_dim, out_dim, p_rows);
     const unsigned forced_tm = env_u("REIN_MMQ_TM", 0), forced_n64 = env_u("REIN_MMQ_N64", 0xFFFFFFFFu);
     if (forced_n64 != 0xFFFFFFFFu) n64 = std::min(forced_n64, p_rows / 64);
     if (forced_tm == 32) n64 = 0;
-    if (forced_tm == 64) {
+    // every token in a 64-token tile: the 64-token kernel itself, 5-7 % ahead of the mixed kernel launched without
+    // fillers (Q8_0 5120 x 34816 at 1024 tokens 681 -> 639 us, 8192 x 8192 at 2048 527 -> 501)
+    const bool all64 = forced_n64 == 0xFFFFFFFFu && forced_tm == 0 && n64 > 0 && n64 * 64 >= p_rows;
+    if (forced_tm == 64 || all64) {
         const unsigned long long g = 8ull * ((n_rb + 7) / 8) * ((p_rows + 63) / 64);
         if (g > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, "rein_mmq_xq8: too many tiles for one launch");
         void* a[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
@@ -852,8 +879,13 @@ Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
         else if (wg32 <= 2ull * kCUs) plain = 0.71 + 0.29 * (double)(wg32 - kCUs) / kCUs;
         else if (wg32 <= 3ull * kCUs) plain = 1.0 + 0.75 * (double)(wg32 - 2ull * kCUs) / kCUs;
         else { const unsigned long long r = u64 % kSkGrid; plain = 1.68 * ((double)(u64 / kSkGrid) + (r == 0 ? 0.0 : r <= kCUs ? 0.71 : 1.0)); }
-        for (Sk8Plan* w : {&w64, &w32})
+        for (Sk8Plan* w : {&w64, &w32}) {
             if (w->take && w->n_unit < g && !(w->cost * n_chunk + 3.0 < plain * n_chunk)) w->take = false;
+            // behind one whole round the same, against a plain launch that is resident at once (its fullest CUs
+            // set its time: 1536 -> 6144 at 384 tokens 25.9 us against 22.8 plain)
+            if (w->take && w->n_unit >= g && wg32 <= 3ull * kCUs &&
+                !(w->cost * n_chunk + 3.0 < (wg32 <= kCUs ? 0.71 : wg32 <= 2ull * kCUs ? 1.0 : 1.75) * n_chunk)) w->take = false;
+        }
     }
     // 128 tokens x 17408 rows: 544 units of 32 tokens are one round and a tail split eight ways (Q8_0 93 -> 73 us,
     // Q6_K 143 -> 117), 272 units of 64 tokens fill half the slots and do not split
@@ -882,8 +914,15 @@ int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t
     const bool large = 2.0 * p_rows * (double)out_dim * in_dim >= 2.8e10;
     if (need != 0 && bytes >= need && (large || asked)) {
         if (bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows)) return 2;
+        // The mixed launch wants its 128-token workgroups to come out even over the CUs' two slots: up to two per
+        // CU (from 1.5, i.e. three 32-token tiles per slot), whole multiples, or five and more.  In between, the
+        // int8 launch with its finer grain is level or ahead (units per CU -> us fp6 against int8: 2.1 184 / 168,
+        // 2.5 233 / 212 and 722 / 660, 2.7 234 / 224, 3.2 281 / 262, 3.5 324 / 289, 4.25 318 / 300; but 1.9 153 / 172,
+        // 2.0 129 / 151, 3.0 193 / 233, 5.0 385 / 399, 8.5 622 / 665, 17 1115 / 1282).
+        const unsigned long long units = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 127) / 128);
         const unsigned long long tiles = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 31) / 32);
-        if (tiles >= 3ull * kSkGrid || asked) return 1;
+        const bool even = tiles >= 3ull * kSkGrid && (units <= kSkGrid || units % kCUs == 0 || units >= 5ull * kCUs);
+        if (even || asked) return 1;
     }
     return bytes >= (size_t)kSkGrid * kSk8PartBytes && sk8_plan(fmt, in_dim, out_dim, p_rows).take ? 3 : 0;
 }
@@ -1040,11 +1079,11 @@ int rein_mmq_block_dots_ws(int fmt, const void* w, const void* xq, int32_t* out,
     return launch("rein_mmq6_q4k_dots", (unsigned)grid, 1, 1, 256, mmq6_lds_bytes(1), s, a);
 }
 
-int rein_mmq_tile_plan(int fmt, unsigned out_dim, unsigned p_rows)
+int rein_mmq_tile_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
     if (!rein_block_size(fmt)) return fail(REIN_E_BAD_FORMAT, "rein_mmq_tile_plan: unknown format " + std::to_string(fmt));
-    if (out_dim == 0 || p_rows == 0) return fail(REIN_E_BAD_SHAPE, "rein_mmq_tile_plan: empty shape");
-    return (int)mmq_pick_n64(out_dim, p_rows);
+    if (in_dim == 0 || out_dim == 0 || p_rows == 0) return fail(REIN_E_BAD_SHAPE, "rein_mmq_tile_plan: empty shape");
+    return (int)mmq_pick_n64(fmt, in_dim, out_dim, p_rows);
 }
 
 int rein_matmul_path(int fmt, unsigned n_rows)

@@ -135,9 +135,9 @@ def matmul_path(fmt, n_rows):
     return ("matvec", "batched_matvec", "mmq")[rc]
 
 
-def mmq_tile_plan(fmt, out_dim, p_rows):
+def mmq_tile_plan(fmt, in_dim, out_dim, p_rows):
     """64-token tiles per 128-row block that mmq_xq8 launches for this shape (0: 32-token tiles only)"""
-    rc = lib.rein_mmq_tile_plan(fmt, out_dim, p_rows)
+    rc = lib.rein_mmq_tile_plan(fmt, in_dim, out_dim, p_rows)
     if rc < 0:
         check(rc)
     return rc

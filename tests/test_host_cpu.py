@@ -116,18 +116,29 @@ def test_mmq_tile_plan():
     # with 32-token fillers in between (512 x 17408: 2176 small workgroups on 256 CUs)
     for fmt in ALL:
         for out_dim, p_rows in [(200, 70), (5120, 96), (17408, 128), (17408, 512), (5120, 2048), (151936, 4096)]:
-            n64 = runtime.mmq_tile_plan(fmt, out_dim, p_rows)
+            n64 = runtime.mmq_tile_plan(fmt, 5120, out_dim, p_rows)
             assert 0 <= n64 <= p_rows // 64
-    assert runtime.mmq_tile_plan(rein.Q4_K, 200, 70) == 0
-    assert runtime.mmq_tile_plan(rein.Q4_K, 17408, 128) == 0
-    assert 1 <= runtime.mmq_tile_plan(rein.Q4_K, 17408, 512) < 8
-    assert runtime.mmq_tile_plan(rein.Q4_K, 17408, 2048) == 32
-    assert runtime.mmq_tile_plan(rein.Q8_0, 151936, 4096) == 64
-    assert runtime.mmq_tile_plan(rein.Q4_K, 17408, 512) == runtime.mmq_tile_plan(rein.Q4_K, 17408, 512)
+    assert runtime.mmq_tile_plan(rein.Q8_0, 5120, 200, 70) == 0
+    assert runtime.mmq_tile_plan(rein.Q8_0, 5120, 5120, 128) == 0           # two 32-token workgroups per CU at most
+    # three per CU resident: the 64-token kernel where its tile is cheap enough (Q8_0), else the 32-token one
+    assert runtime.mmq_tile_plan(rein.Q8_0, 5120, 17408, 128) == 2
+    assert runtime.mmq_tile_plan(rein.Q4_K, 5120, 17408, 128) == 0
+    assert 1 <= runtime.mmq_tile_plan(rein.Q8_0, 5120, 17408, 512) <= 8
+    assert runtime.mmq_tile_plan(rein.Q8_0, 5120, 17408, 2048) == 32
+    assert runtime.mmq_tile_plan(rein.Q8_0, 5120, 151936, 4096) == 64
+    # the price of a 64-token tile is per format: Q4_K's 32-token kernel is the leaner one unless the rows of
+    # the slab are padded (a power-of-two sub-block count)
+    assert runtime.mmq_tile_plan(rein.Q4_K, 5120, 151936, 4096) == 0
+    assert runtime.mmq_tile_plan(rein.Q4_K, 8192, 151936, 4096) == 64
+    assert runtime.mmq_tile_plan(rein.Q4_K, 5120, 34816, 256) == 0
+    assert runtime.mmq_tile_plan(rein.Q8_0, 5120, 34816, 256) >= 1
+    assert runtime.mmq_tile_plan(rein.Q4_K, 5120, 17408, 512) == runtime.mmq_tile_plan(rein.Q4_K, 5120, 17408, 512)
     with pytest.raises(rein.ReinError):
-        runtime.mmq_tile_plan(99, 128, 128)
+        runtime.mmq_tile_plan(99, 128, 128, 128)
     with pytest.raises(rein.ReinError):
-        runtime.mmq_tile_plan(rein.Q4_K, 0, 128)
+        runtime.mmq_tile_plan(rein.Q4_K, 128, 0, 128)
+    with pytest.raises(rein.ReinError):
+        runtime.mmq_tile_plan(rein.Q4_K, 0, 128, 128)
 
 
 def test_compute_calls_fail_loudly_without_runtime():
