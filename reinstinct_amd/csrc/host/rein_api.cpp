@@ -1528,6 +1528,19 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     const unsigned ne = sh.n_tok * sh.n_used;
 
     if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
+    // Few tokens: with at most one routing entry per expert on average nearly every entry meets an expert of its
+    // own, a 32-token tile of the grouped GEMM holds one or two tokens, and the sort is pure overhead.  The decode
+    // kernels (qwen35.rs:3071-3167, here in their two fused launches) read an expert per entry and are ahead up to
+    // there: 128 experts top-8 at 1 / 4 / 16 tokens 21.8 / 39.5 / 107 us against 50.2 / 64.7 / 127 for the pipeline
+    // below, at 32 tokens 194 against 147.  Same integer dots, fp32 sums in the decode kernels' order.
+    if (ne <= sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 && env_u("REIN_MOE_CHAIN", 1) != 0) {
+        const unsigned ns_h = sh.hidden / 32, ns_f = sh.expert_ff / 32;
+        if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
+        if (int rc = rein_moe_gate_up_swiglu_q8(sh.gate_up_fmt, gate_exps, up_exps, ids, base + w.xq_in, base + w.xq_exp, sh.hidden,
+                                                sh.expert_ff, (unsigned)bpe_gu, ns_h, 0, sh.n_used, sh.n_tok, s)) return rc;
+        return rein_moe_down_combine(sh.down_fmt, down_exps, ids, weights, down_exps_s, base + w.xq_exp, out, sh.expert_ff, sh.hidden,
+                                     (unsigned)bpe_dn, sh.n_used * ns_f, ns_f, sh.n_used, sh.n_tok, s);
+    }
     // counting sort by expert (moe_expert_sort.hip), with the inverse permutation kept so
     // that the combine can read the sorted expert outputs in place
     int32_t* count = (int32_t*)(base + w.count);
