@@ -1,6 +1,6 @@
 """Seeded random shapes through the dispatching entry points against the oracle: the dense product
 (rein_matmul / rein_matmul_ws: matvec, batched matvec on every kernel family, MMQ in its plain and
-workspace forms) and the MoE expert FFN (decode launches, fused and unfused pipeline, strided grouped
+workspace forms; larger GEMMs through rein_mmq_xq8_ws in all four launch forms against rein_mmq_xq8) and the MoE expert FFN (decode launches, fused and unfused pipeline, strided grouped
 GEMM).  The fixed-shape tests pin each kernel; these pin the launch choices in between."""
 import os
 
@@ -57,6 +57,46 @@ def test_dense_dispatch_on_random_shapes(seed):
         assert not np.isnan(got).any(), f"case {case}: output not fully written"
         want = orc.matvec_q8(fmt, packed, in_dim, out_dim, orc.quantize_q8(x), n_rows)
         assert_close_f32(got, want, what=f"seed {seed} case {case}")
+
+
+def test_workspace_gemm_matches_the_plain_gemm_on_random_large_shapes():
+    # rein_mmq_xq8_ws in whichever of its four launch forms the library picks (ragged row counts, contractions and
+    # widths around the thresholds) against rein_mmq_xq8, which the fixed-shape tests hold against the oracle
+    rng = np.random.default_rng(9)
+    seen = set()
+    # the fp6 split-tail form wants few, even tiles: two shapes that take it, beside the random ones
+    fixed = {36: (rein.Q4_K, 5120, 5120, 640), 37: (rein.Q4_K, 8192, 8192, 512)}
+    for case in range(38):
+        big = case % 3 != 0
+        fmt = rein.Q4_K if big else DENSE[rng.integers(len(DENSE))]
+        in_dim = int(rng.integers(8 if big else 2, 36)) * 256
+        out_dim = int(rng.integers(3000, 36000)) if big else int(rng.integers(100, 9000))
+        p_rows = int(rng.integers(320, 2100)) if big else int(rng.integers(17, 520))
+        while in_dim * out_dim * 0.6 > 3.5e8:
+            out_dim //= 2
+        while p_rows * out_dim * 4 > 4e8:
+            p_rows //= 2
+        if case in fixed:
+            fmt, in_dim, out_dim, p_rows = fixed[case]
+        nbytes = runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
+        form = runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, nbytes)
+        seen.add(form)
+        print(f"workspace case {case}: fmt {fmt} K {in_dim} N {out_dim} rows {p_rows} form {form}", flush=True)
+        packed = quant.repack_for_matvec(fmt, random_raw_weights(fmt, in_dim, out_dim, seed=case), in_dim, out_dim)
+        x = rng.standard_normal((p_rows, in_dim)).astype(np.float32)
+        dw, dx = dev(packed), dev(x)
+        dq = hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
+        runtime.quantize_q8(dx, dq, in_dim, p_rows)
+        ws = hip.DeviceBuf(max(nbytes, 16))
+        d_ws = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+        d_plain = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+        runtime.mmq_xq8_ws(fmt, dw, dq, d_ws, in_dim, out_dim, p_rows, ws, nbytes)
+        runtime.mmq_xq8(fmt, dw, dq, d_plain, in_dim, out_dim, p_rows)
+        hip.synchronize()
+        got, want = d_ws.to_host(np.float32), d_plain.to_host(np.float32)
+        assert not np.isnan(got).any() and not np.isnan(want).any(), f"workspace case {case}: output not fully written"
+        assert_close_f32(got, want, what=f"workspace case {case}")
+    assert seen == {0, 1, 2, 3}, f"launch forms reached: {sorted(seen)}"
 
 
 def gaussian_slab(fmt, in_dim, out_dim, n_expert, seed):
