@@ -363,7 +363,9 @@ int rein_mmq_block_dots_ws(int fmt, const void *w, const void *xq, int32_t *out,
                            size_t workspace_bytes, rein_stream_t s);
 
 /* ------------------------------------------------------------------- MoE */
-/* moe_topk_f32 (kernels/moe_topk.cpp:17-108; launcher qwen35.rs:2873-2886) */
+/* moe_topk_f32 (kernels/moe_topk.cpp:17-108; launcher qwen35.rs:2873-2886).  Up to 256 experts
+ * run on rein_moe_topk_wave (one wavefront per token, same ids and weight bits); the
+ * reference-named kernel serves larger expert counts and stays in the code object. */
 int rein_moe_topk(const float *logits, unsigned n_tok, unsigned n_expert, unsigned n_used,
                   int32_t *out_ids, float *out_weights, rein_stream_t s);
 /* launch_moe_sort (qwen35.rs:2892-2938; kernels/moe_expert_sort.cpp:27-75):

@@ -1168,6 +1168,13 @@ int rein_moe_topk(const float* logits, unsigned n_tok, unsigned n_expert, unsign
     if (int rc = check_ptr("rein_moe_topk", out_ids, 4, "out_ids")) return rc;
     if (int rc = check_ptr("rein_moe_topk", out_weights, 4, "out_weights")) return rc;
     int ne = (int)n_expert, nu = (int)n_used;
+    if (n_expert <= 256 && env_u("REIN_TOPK_WAVE", 1) != 0) {
+        // one wavefront per token, the tree's decisions as register reductions (no LDS, no barrier): the same ids
+        // and weight bits as moe_topk_f32
+        int nt = (int)n_tok;
+        void* a[] = {(void*)&logits, (void*)&ne, (void*)&nu, (void*)&out_ids, (void*)&out_weights, (void*)&nt};
+        return launch("rein_moe_topk_wave", (n_tok + 3) / 4, 1, 1, 256, 0, s, a);
+    }
     void* args[] = {(void*)&logits, (void*)&ne, (void*)&nu, (void*)&out_ids, (void*)&out_weights};
     return launch("moe_topk_f32", n_tok, 1, 1, 128, n_expert * 4, s, args);
 }
@@ -1527,15 +1534,28 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     int32_t* toff = (int32_t*)(base + w.toff);
     const unsigned ne = sh.n_tok * sh.n_used;
 
-    if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
+    const bool chain = ne <= sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 &&
+                       env_u("REIN_MOE_CHAIN", 1) != 0;
+    // the few-token form routes and quantizes in one launch where the one-wavefront router applies
+    const bool route_quant = chain && sh.n_expert <= 256 && sh.n_used <= 64 && sh.n_used <= sh.n_expert &&
+                             env_u("REIN_TOPK_WAVE", 1) != 0;
+    if (route_quant) {
+        int n_e = (int)sh.n_expert, n_u = (int)sh.n_used, n_t = (int)sh.n_tok;
+        void* xq = base + w.xq_in;
+        unsigned q_per_tok = (sh.hidden + 511) / 512;
+        void* a[] = {(void*)&logits, (void*)&n_e, (void*)&n_u, (void*)&ids, (void*)&weights, (void*)&n_t,
+                     (void*)&x, (void*)&xq, (void*)&sh.hidden, (void*)&q_per_tok};
+        if (int rc = launch("rein_moe_route_quantize", (sh.n_tok + 3) / 4 + sh.n_tok * q_per_tok, 1, 1, 256, 0, s, a)) return rc;
+    } else if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
     // Few tokens: with at most one routing entry per expert on average nearly every entry meets an expert of its
     // own, a 32-token tile of the grouped GEMM holds one or two tokens, and the sort is pure overhead.  The decode
     // kernels (qwen35.rs:3071-3167, here in their two fused launches) read an expert per entry and are ahead up to
     // there: 128 experts top-8 at 1 / 4 / 16 tokens 21.8 / 39.5 / 107 us against 50.2 / 64.7 / 127 for the pipeline
     // below, at 32 tokens 194 against 147.  Same integer dots, fp32 sums in the decode kernels' order.
-    if (ne <= sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 && env_u("REIN_MOE_CHAIN", 1) != 0) {
+    if (chain) {
         const unsigned ns_h = sh.hidden / 32, ns_f = sh.expert_ff / 32;
-        if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
+        if (!route_quant)
+            if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
         if (int rc = rein_moe_gate_up_swiglu_q8(sh.gate_up_fmt, gate_exps, up_exps, ids, base + w.xq_in, base + w.xq_exp, sh.hidden,
                                                 sh.expert_ff, (unsigned)bpe_gu, ns_h, 0, sh.n_used, sh.n_tok, s)) return rc;
         return rein_moe_down_combine(sh.down_fmt, down_exps, ids, weights, down_exps_s, base + w.xq_exp, out, sh.expert_ff, sh.hidden,

@@ -366,6 +366,37 @@ def test_moe_topk_parity():
     assert np.array_equal(d_ids.to_host(np.int32).reshape(ids.shape), ids)
 
 
+def test_moe_topk_wave_kernel_equals_the_workgroup_kernel(monkeypatch):
+    # up to 256 experts the router runs one wavefront per token; it must give the ids and the weight bits of the
+    # workgroup kernel (REIN_TOPK_WAVE=0): random logits, ties, NaN and -inf entries, every tail of the 4-token group
+    rng = np.random.default_rng(77)
+    cases = [(1, 2, 1), (1, 2, 2), (3, 64, 8), (5, 65, 4), (7, 127, 8), (512, 128, 8), (513, 129, 8), (9, 200, 4),
+             (33, 256, 64), (2, 256, 1), (6, 17, 17), (4, 192, 33)]
+    cases += [(int(rng.integers(1, 70)), int(ne), int(rng.integers(1, min(ne, 64) + 1)))
+              for ne in rng.integers(2, 257, 40)]
+    for n_tok, n_expert, n_used in cases:
+        logits = (rng.standard_normal((n_tok, n_expert)) * rng.choice([0.01, 1.0, 30.0])).astype(np.float32)
+        if n_tok > 1:
+            logits[1] = np.round(logits[1])                     # many exact ties
+            logits[0, rng.integers(0, n_expert, 3)] = np.nan
+            logits[-1, rng.integers(0, n_expert, 3)] = -np.inf
+        if n_tok > 4:
+            logits[2] = 0.0
+            logits[3] = np.nan
+            logits[4] = -np.inf
+        d_logits = dev(logits)
+        got = []
+        for wave in ("1", "0"):
+            monkeypatch.setenv("REIN_TOPK_WAVE", wave)
+            d_ids = dev(np.full(n_tok * n_used, -7, np.int32))
+            d_w = dev(np.full(n_tok * n_used, np.nan, np.float32))
+            runtime.moe_topk(d_logits, n_tok, n_expert, n_used, d_ids, d_w)
+            hip.synchronize()
+            got.append((d_ids.to_host(np.int32), d_w.to_host(np.uint32)))
+        assert np.array_equal(got[0][0], got[1][0]), (n_tok, n_expert, n_used)
+        assert np.array_equal(got[0][1], got[1][1]), (n_tok, n_expert, n_used)
+
+
 def gpu_sort(ids, n_expert, bn):
     n = ids.size
     bufs = [hip.DeviceBuf(n_expert * 4), hip.DeviceBuf(n_expert * 4), dev(np.full(n, -1, np.int32)),
@@ -592,3 +623,10 @@ def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, mo
         assert rel_l2(got, want) < 2e-3, what
         assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what=f"moe_ffn few tokens, {what}")
     assert rel_l2(outs[0], outs[1]) < 2e-3
+    # the router and the quantizer share one launch there; as two launches (REIN_TOPK_WAVE=0) the bits are the same
+    monkeypatch.setenv("REIN_MOE_CHAIN", "1")
+    monkeypatch.setenv("REIN_TOPK_WAVE", "0")
+    d_out = dev(np.full(n_tok * hidden, np.nan, np.float32))
+    runtime.moe_ffn(sh, dx, dl, dg, du, dd, ds, ws, d_out)
+    hip.synchronize()
+    assert np.array_equal(d_out.to_host(np.uint32).reshape(n_tok, hidden), outs[0].view(np.uint32))
