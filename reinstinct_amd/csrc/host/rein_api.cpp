@@ -928,6 +928,17 @@ int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t
 }
 }  // namespace
 
+namespace {
+// ---- Q4_K on the fp16 matrix instruction, superblocks accumulated in the matrix unit (kernels/mmq_f16.h)
+size_t x16_image_bytes(unsigned n_sub, unsigned p_rows)                        // rein_x16_bytes
+{
+    const size_t n_grp = (p_rows + 63) / 64;
+    return (size_t)(n_sub / 2) * n_grp * 16384 + (size_t)(n_sub / 8) * n_grp * 2048 + n_grp * 256 + 1024;
+}
+constexpr unsigned kMmq16Lds = 2 * 16384 + 2 * 2048 + 4 * 2 * 2 * 2048 + 4 * 2 * 1280;    // rein_mmq16_lds_bytes()
+bool mmq16_asked(int fmt, unsigned in_dim) { return fmt == REIN_TYPE_Q4_K && in_dim != 0 && in_dim % 256 == 0 && env_u("REIN_MMQ16", 0) != 0; }
+}  // namespace
+
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
     if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < env_u("REIN_MMQ6_FROM", 320)) return 0;
@@ -943,7 +954,8 @@ size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows)
         const bool dense = fmt_tag(fmt) && fmt != REIN_TYPE_Q5_1 && in_dim != 0 && p_rows > 16;
         return dense && env_u("REIN_MMQ_SK", 1) != 0 ? (size_t)kSkGrid * kSk8PartBytes : 0;
     }
-    return env_u("REIN_MMQ6_SK", 1) != 0 ? sk_workspace_bytes(in_dim, p_rows) : x6_image_bytes(in_dim / 32, p_rows);
+    const size_t fp6 = env_u("REIN_MMQ6_SK", 1) != 0 ? sk_workspace_bytes(in_dim, p_rows) : x6_image_bytes(in_dim / 32, p_rows);
+    return mmq16_asked(fmt, in_dim) ? std::max(fp6, x16_image_bytes(in_dim / 32, p_rows)) : fp6;
 }
 
 int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
@@ -953,6 +965,20 @@ int rein_mmq_xq8_ws(int fmt, const void* w, const void* xq, float* y, unsigned i
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
     if (workspace && need != 0 && workspace_bytes < need)
         return fail(REIN_E_BAD_SHAPE, std::string(who) + ": workspace of " + std::to_string(workspace_bytes) + " bytes, rein_mmq_workspace_min_bytes asks for " + std::to_string(need));
+    if (workspace && mmq16_asked(fmt, in_dim) && p_rows > 16 && workspace_bytes >= x16_image_bytes(in_dim / 32, p_rows)) {
+        if (int rc = check_shape(who, fmt, in_dim, out_dim, p_rows)) return rc;
+        if (int rc = check_ptr(who, w, 16, "w")) return rc;
+        if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
+        if (int rc = check_ptr(who, y, 4, "y")) return rc;
+        if (int rc = check_ptr(who, workspace, 16, "workspace")) return rc;
+        const unsigned n_sub = in_dim / 32, n_grp = (p_rows + 63) / 64, n_rb = (out_dim + 255) / 256;
+        void* pa[] = {(void*)&xq, (void*)&workspace, (void*)&n_sub, (void*)&p_rows};
+        if (int rc = launch("rein_mmq16_prep", 2 * n_grp, n_sub / 8, 1, 256, 0, s, pa)) return rc;
+        const unsigned long long grid = 8ull * ((n_rb + 7) / 8) * n_grp;
+        if (grid > 0x7FFFFFFFull) return fail(REIN_E_TOO_LARGE, std::string(who) + ": too many tiles for one launch");
+        void* a[] = {(void*)&w, (void*)&workspace, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&p_rows};
+        return launch("rein_mmq16_q4k", (unsigned)grid, 1, 1, 256, kMmq16Lds, s, a);
+    }
     const int form = workspace ? mmq_form(fmt, in_dim, out_dim, p_rows, workspace_bytes) : 0;
     if (form == 3) {
         const Sk8Plan sk8 = sk8_plan(fmt, in_dim, out_dim, p_rows);
