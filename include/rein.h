@@ -307,7 +307,8 @@ size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 /* Which launch rein_mmq_xq8_ws takes for this shape and workspace size: 0 = the int8 launch of
  * rein_mmq_xq8, 1 = fp6 with one token group per workgroup, 2 = fp6 split-tail, 3 = int8
- * split-tail. */
+ * split-tail, 4 = the fp16 formulation that sums whole superblocks in the matrix unit (only
+ * with REIN_MMQ16=1 in the environment: slower than the others, kept for study). */
 int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes);
 int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                     unsigned out_dim, unsigned p_rows, void *workspace, size_t workspace_bytes,

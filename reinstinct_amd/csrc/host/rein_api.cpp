@@ -1073,6 +1073,7 @@ int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows
 {
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
     if (need != 0 && workspace_bytes < need) return 0;                   // rein_mmq_xq8_ws refuses such a workspace
+    if (mmq16_asked(fmt, in_dim) && p_rows > 16 && workspace_bytes >= x16_image_bytes(in_dim / 32, p_rows)) return 4;
     return mmq_form(fmt, in_dim, out_dim, p_rows, workspace_bytes);
 }
 

@@ -82,7 +82,8 @@ def mmq_workspace_bytes(fmt, in_dim, p_rows):
 
 
 def mmq_form_ws(fmt, in_dim, out_dim, p_rows, workspace_bytes):
-    """0: int8 launch, 1: fp6 with one token group per workgroup, 2: fp6 split-tail"""
+    """0: int8 launch, 1: fp6 with one token group per workgroup, 2: fp6 split-tail, 3: int8 split-tail,
+    4: fp16 with superblocks summed in the matrix unit (REIN_MMQ16=1)"""
     return int(lib.rein_mmq_form_ws(fmt, in_dim, out_dim, p_rows, workspace_bytes))
 
 

@@ -46,6 +46,7 @@ def run(packed, x, in_dim, out_dim):
     dq = hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
     runtime.quantize_q8(dev(x), dq, in_dim, p_rows)
     ws_bytes = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows)
+    assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, p_rows, ws_bytes) == 4
     ws = hip.DeviceBuf(ws_bytes)
     dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
     runtime.mmq_xq8_ws(rein.Q4_K, dev(packed), dq, dy, in_dim, out_dim, p_rows, ws, ws_bytes)
