@@ -145,7 +145,8 @@ extern "C" __global__ void moe_topk_f32(const float* __restrict__ logits, int n_
 //    lowest differing bit, so among equal probabilities the winner is the expert with the smallest bit-reversed
 //    8-bit index (bit 7 = second expert of a slot, lowest priority).  That is a total order, so each round is two
 //    order-free reductions: the maximum probability, then the minimum bit-reversed index among its holders.
-// Same ids and same weight bits as moe_topk_f32 (tested), at 5.6 instead of 6.6 us for one token.
+// Same ids and same weight bits as moe_topk_f32 (tested); 128 experts, top-8: 4.6 instead of 6.5 us for one token,
+// 7.9 instead of 11.4 us for 4096.
 namespace {
 
 template <int CTRL, int ROW_MASK = 0xf>
