@@ -470,7 +470,8 @@ size_t rein_moe_workspace_bytes(const rein_moe_shape *shape);
  * No host synchronisation, no allocation.  With at most one routing entry per expert on average
  * (n_tok * n_used <= n_expert) and Q4_K gate / up experts the same result comes from the decode
  * kernels instead (top-k -> quantize -> rein_moe_gate_up_swiglu_q8 -> rein_moe_down_combine, the
- * launches of qwen35.rs:3071-3167 fused in pairs): no sort, one expert read per entry. */
+ * launches of qwen35.rs:3071-3167 fused in pairs): no sort, one expert read per entry; for one
+ * and two tokens the gate / up launch also routes and quantizes, so the FFN is two launches. */
 int rein_moe_ffn(const rein_moe_shape *shape, const float *x, const float *logits,
                  const void *gate_exps, const void *up_exps, const void *down_exps,
                  const float *down_exps_s, void *workspace, float *out, rein_stream_t s);

@@ -1563,31 +1563,43 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
 
     const bool chain = ne <= sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 &&
                        env_u("REIN_MOE_CHAIN", 1) != 0;
-    // the few-token form routes and quantizes in one launch where the one-wavefront router applies
-    const bool route_quant = chain && sh.n_expert <= 256 && sh.n_used <= 64 && sh.n_used <= sh.n_expert &&
-                             env_u("REIN_TOPK_WAVE", 1) != 0;
-    if (route_quant) {
-        int n_e = (int)sh.n_expert, n_u = (int)sh.n_used, n_t = (int)sh.n_tok;
-        void* xq = base + w.xq_in;
-        unsigned q_per_tok = (sh.hidden + 511) / 512;
-        void* a[] = {(void*)&logits, (void*)&n_e, (void*)&n_u, (void*)&ids, (void*)&weights, (void*)&n_t,
-                     (void*)&x, (void*)&xq, (void*)&sh.hidden, (void*)&q_per_tok};
-        if (int rc = launch("rein_moe_route_quantize", (sh.n_tok + 3) / 4 + sh.n_tok * q_per_tok, 1, 1, 256, 0, s, a)) return rc;
-    } else if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
     // Few tokens: with at most one routing entry per expert on average nearly every entry meets an expert of its
     // own, a 32-token tile of the grouped GEMM holds one or two tokens, and the sort is pure overhead.  The decode
     // kernels (qwen35.rs:3071-3167, here in their two fused launches) read an expert per entry and are ahead up to
-    // there: 128 experts top-8 at 1 / 4 / 16 tokens 21.8 / 39.5 / 107 us against 50.2 / 64.7 / 127 for the pipeline
+    // there: 128 experts top-8 at 1 / 4 / 16 tokens 17 / 36 / 105 us against 50.2 / 64.7 / 127 for the pipeline
     // below, at 32 tokens 194 against 147.  Same integer dots, fp32 sums in the decode kernels' order.
     if (chain) {
         const unsigned ns_h = sh.hidden / 32, ns_f = sh.expert_ff / 32;
-        if (!route_quant)
-            if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
-        if (int rc = rein_moe_gate_up_swiglu_q8(sh.gate_up_fmt, gate_exps, up_exps, ids, base + w.xq_in, base + w.xq_exp, sh.hidden,
-                                                sh.expert_ff, (unsigned)bpe_gu, ns_h, 0, sh.n_used, sh.n_tok, s)) return rc;
+        // Where the one-wavefront router applies it shares a launch: for one or two tokens the gate / up launch
+        // routes and quantizes its token itself (every workgroup again: 15.9 / 23.8 us against 17.3 / 25.4), beyond
+        // that router and quantizer run as one small launch in front (16 tokens: 105 us against 111)
+        const bool wave = sh.n_expert <= 256 && sh.n_used <= 64 && sh.n_used <= sh.n_expert && env_u("REIN_TOPK_WAVE", 1) != 0;
+        const bool routed = wave && sh.n_tok <= 2 && ns_h * 40u <= 48u * 1024u;
+        if (routed) {
+            void* xq_exp = base + w.xq_exp;
+            const unsigned bpe = (unsigned)bpe_gu;
+            void* a[] = {(void*)&gate_exps, (void*)&up_exps, (void*)&logits, (void*)&x, (void*)&ids, (void*)&weights, (void*)&xq_exp,
+                         (void*)&sh.hidden, (void*)&sh.expert_ff, (void*)&bpe, (void*)&sh.n_expert, (void*)&sh.n_used};
+            if (int rc = launch("rein_moe_route_gate_up_swiglu_q8_q4k", sh.expert_ff / 32, sh.n_used, sh.n_tok, 1024, ns_h * 40u, s, a)) return rc;
+        } else {
+            if (wave) {
+                int n_e = (int)sh.n_expert, n_u = (int)sh.n_used, n_t = (int)sh.n_tok;
+                void* xq = base + w.xq_in;
+                unsigned q_per_tok = (sh.hidden + 511) / 512;
+                void* a[] = {(void*)&logits, (void*)&n_e, (void*)&n_u, (void*)&ids, (void*)&weights, (void*)&n_t,
+                             (void*)&x, (void*)&xq, (void*)&sh.hidden, (void*)&q_per_tok};
+                if (int rc = launch("rein_moe_route_quantize", (sh.n_tok + 3) / 4 + sh.n_tok * q_per_tok, 1, 1, 256, 0, s, a)) return rc;
+            } else {
+                if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
+                if (int rc = rein_quantize_q8(x, base + w.xq_in, sh.hidden, sh.n_tok, s)) return rc;
+            }
+            if (int rc = rein_moe_gate_up_swiglu_q8(sh.gate_up_fmt, gate_exps, up_exps, ids, base + w.xq_in, base + w.xq_exp, sh.hidden,
+                                                    sh.expert_ff, (unsigned)bpe_gu, ns_h, 0, sh.n_used, sh.n_tok, s)) return rc;
+        }
         return rein_moe_down_combine(sh.down_fmt, down_exps, ids, weights, down_exps_s, base + w.xq_exp, out, sh.expert_ff, sh.hidden,
                                      (unsigned)bpe_dn, sh.n_used * ns_f, ns_f, sh.n_used, sh.n_tok, s);
     }
+    if (int rc = rein_moe_topk(logits, sh.n_tok, sh.n_expert, sh.n_used, ids, weights, s)) return rc;
     // counting sort by expert (moe_expert_sort.hip), with the inverse permutation kept so
     // that the combine can read the sorted expert outputs in place
     int32_t* count = (int32_t*)(base + w.count);

@@ -20,6 +20,7 @@
 // writes silu(gate) * up with the deterministic silu of q8_block.h.
 #include "rein_formats.h"
 #include "q8_block.h"
+#include "moe_topk_wave.h"
 
 // Dot products of rows row0 .. row0+R-1 of one expert (w0; GATE_UP: also w1) with the
 // BlockQ8 row xqs, for a team of LANES lanes (lane = index in the team).  s0 / s1 are valid
@@ -131,20 +132,14 @@ __device__ __forceinline__ void rein_moe_matvec(const uint8_t* __restrict__ slab
 // computes rows 2w, 2w + 1 (the mapping of the two-launch form), the 32 values meet in LDS and
 // one 16-lane row quantizes them.  grid = (out_dim / 32, n_used, n_tok); out_dim % 32 == 0.
 template <int FMT>
-__device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
-                                                           const int* __restrict__ ids, const BlockQ8* __restrict__ xq,
-                                                           BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
-                                                           unsigned bytes_per_expert, unsigned xq_tok_stride,
-                                                           unsigned xq_slot_stride, unsigned n_used)
+__device__ __forceinline__ void rein_moe_gate_up_swiglu_q8_core(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
+                                                                unsigned eid, const BlockQ8* __restrict__ xqs,
+                                                                BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
+                                                                unsigned bytes_per_expert, unsigned n_used, float* vals)
 {
     using F = Fmt<FMT>;
-    __shared__ float vals[32];
-    if (blockDim.x != 1024u) return;
     const unsigned tok = blockIdx.z, slot = blockIdx.y, blk = blockIdx.x;
     const unsigned n_blk = out_dim >> 5;
-    if (blk >= n_blk) return;
-    const unsigned eid = (unsigned)ids[(size_t)tok * n_used + slot];
-    const BlockQ8* xqs = xq + (size_t)tok * xq_tok_stride + (size_t)slot * xq_slot_stride;
     const unsigned n_sub = in_dim >> 5;
     const F w0(gate_slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
     const F w1(up_slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
@@ -156,6 +151,61 @@ __device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __rest
     __syncthreads();
     if (threadIdx.x < 16u)
         rein_q8_store_sub(xq_out + ((size_t)tok * n_used + slot) * n_blk + blk, threadIdx.x, vals[threadIdx.x], vals[threadIdx.x + 16u]);
+}
+
+template <int FMT>
+__device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
+                                                           const int* __restrict__ ids, const BlockQ8* __restrict__ xq,
+                                                           BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
+                                                           unsigned bytes_per_expert, unsigned xq_tok_stride,
+                                                           unsigned xq_slot_stride, unsigned n_used)
+{
+    __shared__ float vals[32];
+    if (blockDim.x != 1024u) return;
+    const unsigned tok = blockIdx.z, slot = blockIdx.y;
+    if (blockIdx.x >= (out_dim >> 5)) return;
+    const unsigned eid = (unsigned)ids[(size_t)tok * n_used + slot];
+    rein_moe_gate_up_swiglu_q8_core<FMT>(gate_slab, up_slab, eid, xq + (size_t)tok * xq_tok_stride + (size_t)slot * xq_slot_stride,
+                                         xq_out, in_dim, out_dim, bytes_per_expert, n_used, vals);
+}
+
+// The same with the router and quantize_q8_f32 in front, for the few-token expert FFN: every workgroup routes its
+// token on its first wavefront (rein_topk::topk_one_wave: the ids and weight bits of moe_topk_f32) while all
+// sixteen quantize the token's row into LDS (the bytes of quantize_q8_f32), then runs the launch above on its
+// expert.  The workgroup (0, 0, tok) stores the token's ids and weights for the down projection.  One launch
+// instead of three in front of the down projection: the router is a few microseconds of one wavefront's time,
+// the launch it replaces costs as much on the whole GPU.  Up to 256 experts and 64 used; dynamic shared memory =
+// in_dim / 32 * 40 bytes; grid = (out_dim / 32, n_used, n_tok) x 1024 threads.
+template <int FMT>
+__device__ __forceinline__ void rein_moe_route_gate_up_swiglu_q8(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
+                                                                 const float* __restrict__ logits, const float* __restrict__ x,
+                                                                 int* __restrict__ ids_out, float* __restrict__ weights_out,
+                                                                 BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
+                                                                 unsigned bytes_per_expert, unsigned n_expert, unsigned n_used)
+{
+    extern __shared__ BlockQ8 rein_moe_xq_row[];             // in_dim / 32 blocks
+    __shared__ float vals[32];
+    __shared__ int ids_s[64];
+    __shared__ float weights_s[64];
+    if (blockDim.x != 1024u) return;
+    const unsigned tok = blockIdx.z, slot = blockIdx.y;
+    if (blockIdx.x >= (out_dim >> 5)) return;
+    const unsigned n_sub = in_dim >> 5;
+    if (threadIdx.x < 64u)
+        rein_topk::topk_one_wave(logits + (size_t)tok * n_expert, (int)n_expert, (int)n_used, ids_s, weights_s, (int)threadIdx.x);
+    const float* xr = x + (size_t)tok * in_dim;
+    const unsigned l = threadIdx.x & 15u;
+    for (unsigned sb = threadIdx.x >> 4; sb < n_sub; sb += 64u) {
+        const float* v = xr + (size_t)sb * 32 + l;
+        rein_q8_store_sub(rein_moe_xq_row + sb, l, v[0], v[16]);
+    }
+    __syncthreads();
+    if (blockIdx.x == 0u && slot == 0u && threadIdx.x < n_used) {
+        ids_out[(size_t)tok * n_used + threadIdx.x] = ids_s[threadIdx.x];
+        weights_out[(size_t)tok * n_used + threadIdx.x] = weights_s[threadIdx.x];
+    }
+    rein_moe_gate_up_swiglu_q8_core<FMT>(gate_slab, up_slab, (unsigned)ids_s[slot], rein_moe_xq_row, xq_out, in_dim, out_dim,
+                                         bytes_per_expert, n_used, vals);
 }
 
 // down projection + weighted combine in one launch:
@@ -270,6 +320,16 @@ void moe_gate_up_swiglu_q4k_repacked_f32(const unsigned char* __restrict__ gate_
                                         bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used);         \
     }
 REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k, REIN_Q4_K)
+
+extern "C" __global__ __launch_bounds__(1024) void rein_moe_route_gate_up_swiglu_q8_q4k(
+    const unsigned char* __restrict__ gate_slab, const unsigned char* __restrict__ up_slab,
+    const float* __restrict__ logits, const float* __restrict__ x, int* __restrict__ ids_out,
+    float* __restrict__ weights_out, BlockQ8* __restrict__ xq_out, unsigned int in_dim, unsigned int out_dim,
+    unsigned int bytes_per_expert, unsigned int n_expert, unsigned int n_used)
+{
+    rein_moe_route_gate_up_swiglu_q8<REIN_Q4_K>(gate_slab, up_slab, logits, x, ids_out, weights_out, xq_out, in_dim,
+                                                out_dim, bytes_per_expert, n_expert, n_used);
+}
 
 #define REIN_DEFINE_MOE_DC(name, FMT, R, LANES)                                                           \
     extern "C" __global__ __launch_bounds__(512) void name(                                               \

@@ -589,7 +589,7 @@ def test_moe_ffn_end_to_end_small():
     assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what="moe_ffn")
 
 
-@pytest.mark.parametrize("n_tok,n_expert,n_used", [(1, 16, 4), (3, 64, 4), (8, 32, 4), (16, 64, 4)])
+@pytest.mark.parametrize("n_tok,n_expert,n_used", [(1, 16, 4), (2, 128, 8), (1, 200, 3), (3, 64, 4), (8, 32, 4), (16, 64, 4)])
 def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, monkeypatch):
     # at most one routing entry per expert on average: rein_moe_ffn runs the two decode launches instead of
     # sort + grouped GEMMs; against the CPU chain, and against its own pipeline (REIN_MOE_CHAIN=0)
@@ -623,7 +623,8 @@ def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, mo
         assert rel_l2(got, want) < 2e-3, what
         assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what=f"moe_ffn few tokens, {what}")
     assert rel_l2(outs[0], outs[1]) < 2e-3
-    # the router and the quantizer share one launch there; as two launches (REIN_TOPK_WAVE=0) the bits are the same
+    # the router and the quantizer share a launch there (one and two tokens: the gate / up launch itself, more: one
+    # small launch in front); as separate launches (REIN_TOPK_WAVE=0) the bits are the same
     monkeypatch.setenv("REIN_MOE_CHAIN", "1")
     monkeypatch.setenv("REIN_TOPK_WAVE", "0")
     d_out = dev(np.full(n_tok * hidden, np.nan, np.float32))
