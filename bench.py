@@ -369,11 +369,27 @@ def extras_moe_decode(stream):
         runtime.moe_down_combine(rein.Q6_K, down, ids[t], wts, ones, aq, out, ff, hidden, down1.nbytes, n_used * ns_f, ns_f,
                                  n_used, 1, stream)
 
+    # the whole routed FFN of one token through rein_moe_ffn (router and quantizer included): the logits of token t
+    # peak on its own eight experts, so the sixteen tokens of a graph stream disjoint experts as above
+    shape = runtime.moe_shape(1, hidden, n_expert, n_used, ff, rein.Q4_K, rein.Q6_K)
+    wsb = hip.DeviceBuf(runtime.moe_workspace_bytes(shape))
+    dx = hip.DeviceBuf.from_host(x)
+    lg = np.zeros((toks, n_expert), np.float32)
+    for t in range(toks):
+        lg[t, t * n_used:(t + 1) * n_used] = 4.0 + 0.1 * np.arange(n_used, dtype=np.float32)
+    dlg = [hip.DeviceBuf.from_host(lg[t:t + 1]) for t in range(toks)]
+
+    def token_ffn(t):
+        runtime.moe_ffn(shape, dx, dlg[t], gate, up, down, ones, wsb, out, stream)
+
     sec4 = time_graph(stream, lambda: [token(t) for t in range(toks)], toks)
     sec = time_graph(stream, lambda: [token_fused(t) for t in range(toks)], toks)
+    sec_ffn = time_graph(stream, lambda: [token_ffn(t) for t in range(toks)], toks)
     res = {"workload": "MoE decode expert FFN, 1 token, 128 experts top-8, hidden 2048, ff 768: gate+up+SwiGLU+quantize "
                        "(Q4_K) -> down+combine (Q6_K), 2 launches",
            "us_per_token": round(sec * 1e6, 2), "us_per_token_4_launch_chain": round(sec4 * 1e6, 2),
+           "us_per_token_rein_moe_ffn": round(sec_ffn * 1e6, 2),
+           "rein_moe_ffn_note": "router + quantizer + the two launches above from fp32 x and logits: 2 launches per token",
            "expert_bytes_per_token": per_token,
            "GBs": round(per_token / sec / 1e9, 0), "frac_hbm_peak": round(per_token / sec / 1e9 / HBM_PEAK_GBS, 4)}
     log("moe decode", res)
