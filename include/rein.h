@@ -467,8 +467,8 @@ size_t rein_moe_workspace_bytes(const rein_moe_shape *shape);
  * gate_exps / up_exps: n_expert slabs [hidden -> expert_ff]; down_exps:
  * [expert_ff -> hidden]; down_exps_s [n_expert] fp32 (the reference passes
  * ones).  `workspace` holds rein_moe_workspace_bytes; out [n_tok][hidden].
- * No host synchronisation, no allocation.  With at most one routing entry per expert on average
- * (n_tok * n_used <= n_expert) and Q4_K gate / up experts the same result comes from the decode
+ * No host synchronisation, no allocation.  With at most 1.6 routing entries per expert on average
+ * (5 n_tok n_used <= 8 n_expert) and Q4_K gate / up experts the same result comes from the decode
  * kernels instead (top-k -> quantize -> rein_moe_gate_up_swiglu_q8 -> rein_moe_down_combine, the
  * launches of qwen35.rs:3071-3167 fused in pairs): no sort, one expert read per entry; for one
  * and two tokens the gate / up launch also routes and quantizes, so the FFN is two launches. */

@@ -1429,7 +1429,12 @@ int rein_moe_gate_up_swiglu_q8(int fmt, const void* gate_slab, const void* up_sl
     if (int rc = check_ptr(who, xq_out, 8, "xq_out")) return rc;
     void* a[] = {(void*)&gate_slab, (void*)&up_slab, (void*)&ids, (void*)&xq, (void*)&xq_out, (void*)&in_dim, (void*)&out_dim,
                  (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
-    return launch("rein_moe_gate_up_swiglu_q8_q4k", out_dim / 32, n_used, n_tok, 1024, 0, s, a);
+    // two rows per wavefront (1024 threads per 32 outputs) or four (512): four once the launch is two workgroups
+    // per CU -- more bytes in flight per lane, half the wavefronts to start; 128 experts top-8, 2048 -> 768 at
+    // 4 / 8 / 16 tokens 32.9 / 51.9 / 88.4 us per FFN against 34.1 / 55.9 / 99.3, one token 16.9 against 15.9
+    const unsigned gu_rows = env_u("REIN_MOE_GU_ROWS", 0);
+    const bool r4 = gu_rows == 4 || (gu_rows != 2 && (unsigned long long)(out_dim / 32) * n_used * n_tok >= 2ull * kCUs);
+    return launch(r4 ? "rein_moe_gate_up_swiglu_q8_q4k_r4" : "rein_moe_gate_up_swiglu_q8_q4k", out_dim / 32, n_used, n_tok, r4 ? 512 : 1024, 0, s, a);
 }
 
 int rein_moe_down_combine(int fmt, const void* slab, const int32_t* ids, const float* weights, const float* down_exps_s,
@@ -1450,16 +1455,22 @@ int rein_moe_down_combine(int fmt, const void* slab, const int32_t* ids, const f
     if (int rc = check_ptr(who, down_exps_s, 4, "down_exps_s")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, out, 4, "out")) return rc;
-    // a workgroup owns two rows, one team per slot: half-wavefront teams for contractions of at most
-    // 32 sub-blocks, whole wavefronts otherwise; as many teams as slots, up to 512 threads
+    // A workgroup owns `rows` rows, one team per slot: half-wavefront teams for contractions of at most 32
+    // sub-blocks, whole wavefronts otherwise; as many teams as slots, up to 512 threads.  rows = the most of 8, 4, 2
+    // that leaves four workgroups per CU (REIN_MOE_DC_ROWS forces it); every choice gives the same bits.
     const bool half = in_dim / 32 <= 32;
     const unsigned lanes = half ? 32 : 64;
     unsigned threads = ((n_used * lanes + 63) / 64) * 64;
     if (threads > 512) threads = 512;
+    unsigned rows = env_u("REIN_MOE_DC_ROWS", 0);
+    if (rows != 2 && rows != 4 && rows != 8) {
+        rows = 8;
+        while (rows > 2 && (unsigned long long)((out_dim + rows - 1) / rows) * n_tok < 4ull * kCUs) rows /= 2;
+    }
     void* a[] = {(void*)&slab, (void*)&ids, (void*)&weights, (void*)&down_exps_s, (void*)&xq, (void*)&out, (void*)&in_dim,
                  (void*)&out_dim, (void*)&bytes_per_expert, (void*)&xq_tok_stride, (void*)&xq_slot_stride, (void*)&n_used};
-    return launch(std::string("rein_moe_down_combine_") + fmt_tag(fmt) + (half ? "_h" : ""),
-                  (out_dim + 1) / 2, 1, n_tok, threads, 0, s, a);
+    return launch(std::string("rein_moe_down_combine_") + fmt_tag(fmt) + (half ? "_h" : "") + (rows == 2 ? "" : rows == 4 ? "_r4" : "_r8"),
+                  (out_dim + rows - 1) / rows, 1, n_tok, threads, 0, s, a);
 }
 
 int rein_swiglu_mul(const float* gate, const float* up, float* out, unsigned n, rein_stream_t s)
@@ -1561,13 +1572,14 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     int32_t* toff = (int32_t*)(base + w.toff);
     const unsigned ne = sh.n_tok * sh.n_used;
 
-    const bool chain = ne <= sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 &&
+    // Few tokens: with about one routing entry per expert nearly every entry meets an expert of its own, a
+    // 32-token tile of the grouped GEMM holds one or two tokens, and the sort is pure overhead.  The decode kernels
+    // (qwen35.rs:3071-3167, here in their two fused launches) read an expert per entry -- streaming, where a
+    // mostly empty tile pays its full matrix work -- and are ahead up to 1.6 entries per expert: 128 experts top-8
+    // at 1 / 4 / 16 / 24 tokens 16 / 33 / 89 / 125 us against 48 / 61 / 126 / 141 for the pipeline below, at 28
+    // tokens 141 against 143, at 32 tokens 160 against 145.  Same integer dots, fp32 sums in the decode kernels' order.
+    const bool chain = 5ull * ne <= 8ull * sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 &&
                        env_u("REIN_MOE_CHAIN", 1) != 0;
-    // Few tokens: with at most one routing entry per expert on average nearly every entry meets an expert of its
-    // own, a 32-token tile of the grouped GEMM holds one or two tokens, and the sort is pure overhead.  The decode
-    // kernels (qwen35.rs:3071-3167, here in their two fused launches) read an expert per entry and are ahead up to
-    // there: 128 experts top-8 at 1 / 4 / 16 tokens 17 / 36 / 105 us against 50.2 / 64.7 / 127 for the pipeline
-    // below, at 32 tokens 194 against 147.  Same integer dots, fp32 sums in the decode kernels' order.
     if (chain) {
         const unsigned ns_h = sh.hidden / 32, ns_f = sh.expert_ff / 32;
         // Where the one-wavefront router applies it shares a launch: for one or two tokens the gate / up launch
@@ -1580,7 +1592,10 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
             const unsigned bpe = (unsigned)bpe_gu;
             void* a[] = {(void*)&gate_exps, (void*)&up_exps, (void*)&logits, (void*)&x, (void*)&ids, (void*)&weights, (void*)&xq_exp,
                          (void*)&sh.hidden, (void*)&sh.expert_ff, (void*)&bpe, (void*)&sh.n_expert, (void*)&sh.n_used};
-            if (int rc = launch("rein_moe_route_gate_up_swiglu_q8_q4k", sh.expert_ff / 32, sh.n_used, sh.n_tok, 1024, ns_h * 40u, s, a)) return rc;
+            const unsigned gu_rows = env_u("REIN_MOE_GU_ROWS", 0);
+            const bool r4 = gu_rows == 4 || (gu_rows != 2 && (unsigned long long)(sh.expert_ff / 32) * sh.n_used * sh.n_tok >= 2ull * kCUs);
+            if (int rc = launch(r4 ? "rein_moe_route_gate_up_swiglu_q8_q4k_r4" : "rein_moe_route_gate_up_swiglu_q8_q4k", sh.expert_ff / 32,
+                                sh.n_used, sh.n_tok, r4 ? 512 : 1024, ns_h * 40u, s, a)) return rc;
         } else {
             if (wave) {
                 int n_e = (int)sh.n_expert, n_u = (int)sh.n_used, n_t = (int)sh.n_tok;

@@ -131,7 +131,7 @@ __device__ __forceinline__ void rein_moe_matvec(const uint8_t* __restrict__ slab
 // same block quantizer).  One workgroup of 1024 threads per block of 32 outputs: wavefront w
 // computes rows 2w, 2w + 1 (the mapping of the two-launch form), the 32 values meet in LDS and
 // one 16-lane row quantizes them.  grid = (out_dim / 32, n_used, n_tok); out_dim % 32 == 0.
-template <int FMT>
+template <int FMT, int R>
 __device__ __forceinline__ void rein_moe_gate_up_swiglu_q8_core(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
                                                                 unsigned eid, const BlockQ8* __restrict__ xqs,
                                                                 BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
@@ -144,16 +144,18 @@ __device__ __forceinline__ void rein_moe_gate_up_swiglu_q8_core(const uint8_t* _
     const F w0(gate_slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
     const F w1(up_slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const unsigned row0 = blk * 32u + wave * 2u;
-    float s0[2], s1[2];
-    rein_moe_row_sums<FMT, 2, 64, true>(w0, w1, xqs, n_sub, row0, out_dim - 1u, lane, s0, s1);
-    if (lane < 2u) vals[wave * 2u + lane] = lane ? rein_silu_det(s0[1]) * s1[1] : rein_silu_det(s0[0]) * s1[0];
+    const unsigned row0 = blk * 32u + wave * R;
+    float s0[R], s1[R];
+    rein_moe_row_sums<FMT, R, 64, true>(w0, w1, xqs, n_sub, row0, out_dim - 1u, lane, s0, s1);
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        if (lane == (unsigned)r) vals[wave * R + r] = rein_silu_det(s0[r]) * s1[r];
     __syncthreads();
     if (threadIdx.x < 16u)
         rein_q8_store_sub(xq_out + ((size_t)tok * n_used + slot) * n_blk + blk, threadIdx.x, vals[threadIdx.x], vals[threadIdx.x + 16u]);
 }
 
-template <int FMT>
+template <int FMT, int R>
 __device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
                                                            const int* __restrict__ ids, const BlockQ8* __restrict__ xq,
                                                            BlockQ8* __restrict__ xq_out, unsigned in_dim, unsigned out_dim,
@@ -161,11 +163,11 @@ __device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __rest
                                                            unsigned xq_slot_stride, unsigned n_used)
 {
     __shared__ float vals[32];
-    if (blockDim.x != 1024u) return;
+    if (blockDim.x != 64u * (32u / R)) return;
     const unsigned tok = blockIdx.z, slot = blockIdx.y;
     if (blockIdx.x >= (out_dim >> 5)) return;
     const unsigned eid = (unsigned)ids[(size_t)tok * n_used + slot];
-    rein_moe_gate_up_swiglu_q8_core<FMT>(gate_slab, up_slab, eid, xq + (size_t)tok * xq_tok_stride + (size_t)slot * xq_slot_stride,
+    rein_moe_gate_up_swiglu_q8_core<FMT, R>(gate_slab, up_slab, eid, xq + (size_t)tok * xq_tok_stride + (size_t)slot * xq_slot_stride,
                                          xq_out, in_dim, out_dim, bytes_per_expert, n_used, vals);
 }
 
@@ -176,7 +178,7 @@ __device__ __forceinline__ void rein_moe_gate_up_swiglu_q8(const uint8_t* __rest
 // instead of three in front of the down projection: the router is a few microseconds of one wavefront's time,
 // the launch it replaces costs as much on the whole GPU.  Up to 256 experts and 64 used; dynamic shared memory =
 // in_dim / 32 * 40 bytes; grid = (out_dim / 32, n_used, n_tok) x 1024 threads.
-template <int FMT>
+template <int FMT, int R>
 __device__ __forceinline__ void rein_moe_route_gate_up_swiglu_q8(const uint8_t* __restrict__ gate_slab, const uint8_t* __restrict__ up_slab,
                                                                  const float* __restrict__ logits, const float* __restrict__ x,
                                                                  int* __restrict__ ids_out, float* __restrict__ weights_out,
@@ -187,7 +189,7 @@ __device__ __forceinline__ void rein_moe_route_gate_up_swiglu_q8(const uint8_t* 
     __shared__ float vals[32];
     __shared__ int ids_s[64];
     __shared__ float weights_s[64];
-    if (blockDim.x != 1024u) return;
+    if (blockDim.x != 64u * (32u / R)) return;
     const unsigned tok = blockIdx.z, slot = blockIdx.y;
     if (blockIdx.x >= (out_dim >> 5)) return;
     const unsigned n_sub = in_dim >> 5;
@@ -195,7 +197,7 @@ __device__ __forceinline__ void rein_moe_route_gate_up_swiglu_q8(const uint8_t* 
         rein_topk::topk_one_wave(logits + (size_t)tok * n_expert, (int)n_expert, (int)n_used, ids_s, weights_s, (int)threadIdx.x);
     const float* xr = x + (size_t)tok * in_dim;
     const unsigned l = threadIdx.x & 15u;
-    for (unsigned sb = threadIdx.x >> 4; sb < n_sub; sb += 64u) {
+    for (unsigned sb = threadIdx.x >> 4; sb < n_sub; sb += blockDim.x >> 4) {
         const float* v = xr + (size_t)sb * 32 + l;
         rein_q8_store_sub(rein_moe_xq_row + sb, l, v[0], v[16]);
     }
@@ -204,7 +206,7 @@ __device__ __forceinline__ void rein_moe_route_gate_up_swiglu_q8(const uint8_t* 
         ids_out[(size_t)tok * n_used + threadIdx.x] = ids_s[threadIdx.x];
         weights_out[(size_t)tok * n_used + threadIdx.x] = weights_s[threadIdx.x];
     }
-    rein_moe_gate_up_swiglu_q8_core<FMT>(gate_slab, up_slab, (unsigned)ids_s[slot], rein_moe_xq_row, xq_out, in_dim, out_dim,
+    rein_moe_gate_up_swiglu_q8_core<FMT, R>(gate_slab, up_slab, (unsigned)ids_s[slot], rein_moe_xq_row, xq_out, in_dim, out_dim,
                                          bytes_per_expert, n_used, vals);
 }
 
@@ -243,6 +245,15 @@ __device__ __forceinline__ void rein_moe_down_combine(const uint8_t* __restrict_
             // a team past the last slot repeats the last slot and stores nothing
             const unsigned j = min(j0 + team, n_used - 1u);
             const unsigned eid = (unsigned)ids[j];
+            // the slots' scales are requested in front of the weights, so that the sum behind the barrier finds
+            // them in registers instead of starting two dependent loads (ids -> down_exps_s) there
+            const unsigned n_here = min(n_teams, n_used - j0);
+            float scl[kMaxTeams];
+            if (threadIdx.x < (unsigned)R) {
+#pragma unroll
+                for (unsigned t = 0; t < kMaxTeams; t++)
+                    scl[t] = t < n_here ? weights[j0 + t] * down_exps_s[ids[j0 + t]] : 0.0f;
+            }
             const F w(slab + (size_t)eid * bytes_per_expert, n_sub, out_dim);
             const BlockQ8* xqs = xq + (size_t)tok * xq_tok_stride + (size_t)j * xq_slot_stride;
             float s0[R], s1[R];
@@ -253,11 +264,9 @@ __device__ __forceinline__ void rein_moe_down_combine(const uint8_t* __restrict_
             }
             __syncthreads();
             if (threadIdx.x < (unsigned)R) {
-                const unsigned n_here = min(n_teams, n_used - j0);
-                for (unsigned t = 0; t < n_here; t++) {
-                    const float sc = weights[j0 + t] * down_exps_s[ids[j0 + t]];
-                    acc += sc * vals[t][threadIdx.x];
-                }
+#pragma unroll
+                for (unsigned t = 0; t < kMaxTeams; t++)
+                    if (t < n_here) acc += scl[t] * vals[t][threadIdx.x];
             }
             __syncthreads();
         }
@@ -309,27 +318,33 @@ void moe_gate_up_swiglu_q4k_repacked_f32(const unsigned char* __restrict__ gate_
 
 // The two fused launches of the one-token expert FFN (no counterpart in the reference, which
 // runs the four-launch chain of src/runtime/qwen35.rs:3071-3167).
-#define REIN_DEFINE_MOE_GUQ8(name, FMT)                                                                   \
-    extern "C" __global__ __launch_bounds__(1024) void name(                                              \
+#define REIN_DEFINE_MOE_GUQ8(name, FMT, R)                                                                \
+    extern "C" __global__ __launch_bounds__(64 * (32 / R)) void name(                                     \
         const unsigned char* __restrict__ gate_slab, const unsigned char* __restrict__ up_slab,           \
         const int* __restrict__ ids, const BlockQ8* __restrict__ xq, BlockQ8* __restrict__ xq_out,        \
         unsigned int in_dim, unsigned int out_dim, unsigned int bytes_per_expert,                         \
         unsigned int xq_tok_stride, unsigned int xq_slot_stride, unsigned int n_used)                     \
     {                                                                                                     \
-        rein_moe_gate_up_swiglu_q8<FMT>(gate_slab, up_slab, ids, xq, xq_out, in_dim, out_dim,             \
-                                        bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used);         \
+        rein_moe_gate_up_swiglu_q8<FMT, R>(gate_slab, up_slab, ids, xq, xq_out, in_dim, out_dim,          \
+                                           bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used);      \
     }
-REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k, REIN_Q4_K)
+// two rows per wavefront and 1024 threads, or four and 512 (more bytes in flight per lane, half the wavefronts)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k, REIN_Q4_K, 2)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k_r4, REIN_Q4_K, 4)
 
-extern "C" __global__ __launch_bounds__(1024) void rein_moe_route_gate_up_swiglu_q8_q4k(
-    const unsigned char* __restrict__ gate_slab, const unsigned char* __restrict__ up_slab,
-    const float* __restrict__ logits, const float* __restrict__ x, int* __restrict__ ids_out,
-    float* __restrict__ weights_out, BlockQ8* __restrict__ xq_out, unsigned int in_dim, unsigned int out_dim,
-    unsigned int bytes_per_expert, unsigned int n_expert, unsigned int n_used)
-{
-    rein_moe_route_gate_up_swiglu_q8<REIN_Q4_K>(gate_slab, up_slab, logits, x, ids_out, weights_out, xq_out, in_dim,
-                                                out_dim, bytes_per_expert, n_expert, n_used);
-}
+#define REIN_DEFINE_MOE_RGUQ8(name, FMT, R)                                                               \
+    extern "C" __global__ __launch_bounds__(64 * (32 / R)) void name(                                     \
+        const unsigned char* __restrict__ gate_slab, const unsigned char* __restrict__ up_slab,           \
+        const float* __restrict__ logits, const float* __restrict__ x, int* __restrict__ ids_out,         \
+        float* __restrict__ weights_out, BlockQ8* __restrict__ xq_out, unsigned int in_dim,               \
+        unsigned int out_dim, unsigned int bytes_per_expert, unsigned int n_expert, unsigned int n_used)  \
+    {                                                                                                     \
+        rein_moe_route_gate_up_swiglu_q8<FMT, R>(gate_slab, up_slab, logits, x, ids_out, weights_out,     \
+                                                 xq_out, in_dim, out_dim, bytes_per_expert, n_expert,     \
+                                                 n_used);                                                 \
+    }
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q4k, REIN_Q4_K, 2)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q4k_r4, REIN_Q4_K, 4)
 
 #define REIN_DEFINE_MOE_DC(name, FMT, R, LANES)                                                           \
     extern "C" __global__ __launch_bounds__(512) void name(                                               \
@@ -341,15 +356,19 @@ extern "C" __global__ __launch_bounds__(1024) void rein_moe_route_gate_up_swiglu
         rein_moe_down_combine<FMT, R, LANES>(slab, ids, weights, down_exps_s, xq, out, in_dim, out_dim,   \
                                              bytes_per_expert, xq_tok_stride, xq_slot_stride, n_used);    \
     }
-// two rows per workgroup; short contractions (at most 32 sub-blocks): half-wavefront teams,
-// as the *_down symbols
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q4k_h, REIN_Q4_K, 2, 32)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5k_h, REIN_Q5_K, 2, 32)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q6k_h, REIN_Q6_K, 2, 32)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q8_0_h, REIN_Q8_0, 2, 32)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5_1_h, REIN_Q5_1, 2, 32)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q4k, REIN_Q4_K, 2, 64)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5k, REIN_Q5_K, 2, 64)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q6k, REIN_Q6_K, 2, 64)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q8_0, REIN_Q8_0, 2, 64)
-REIN_DEFINE_MOE_DC(rein_moe_down_combine_q5_1, REIN_Q5_1, 2, 64)
+// Two, four or eight rows per workgroup (the host takes the most rows that still leave the machine four workgroups
+// per CU: more rows are more bytes in flight per lane and fewer workgroups to start -- 16 tokens x 128 experts
+// top-8, Q6_K 768 -> 2048: 110 / 99 / 96 us per FFN at 2 / 4 / 8 rows, one token 15.6 / 15.5 / 16.0).  Short
+// contractions (at most 32 sub-blocks): half-wavefront teams (_h), as the *_down symbols.
+#define REIN_DEFINE_MOE_DC_ROWS(stem, FMT)                      \
+    REIN_DEFINE_MOE_DC(stem##_h, FMT, 2, 32)                    \
+    REIN_DEFINE_MOE_DC(stem##_h_r4, FMT, 4, 32)                 \
+    REIN_DEFINE_MOE_DC(stem##_h_r8, FMT, 8, 32)                 \
+    REIN_DEFINE_MOE_DC(stem, FMT, 2, 64)                        \
+    REIN_DEFINE_MOE_DC(stem##_r4, FMT, 4, 64)                   \
+    REIN_DEFINE_MOE_DC(stem##_r8, FMT, 8, 64)
+REIN_DEFINE_MOE_DC_ROWS(rein_moe_down_combine_q4k, REIN_Q4_K)
+REIN_DEFINE_MOE_DC_ROWS(rein_moe_down_combine_q5k, REIN_Q5_K)
+REIN_DEFINE_MOE_DC_ROWS(rein_moe_down_combine_q6k, REIN_Q6_K)
+REIN_DEFINE_MOE_DC_ROWS(rein_moe_down_combine_q8_0, REIN_Q8_0)
+REIN_DEFINE_MOE_DC_ROWS(rein_moe_down_combine_q5_1, REIN_Q5_1)
