@@ -291,7 +291,14 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (!small && n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(fmt, out_dim, b);
-    const unsigned wpb = 4;
+    // Wavefronts per workgroup (they share nothing): four, or two where the finer grain deals the wavefronts more
+    // evenly over the CUs -- every format at two activation rows (Q4_K 17408 -> 5120: 18.5 -> 15.4 us, 5120 -> 5120:
+    // 7.5 -> 6.7; IQ3_S 16.4 -> 14.5), Q8_0 also at one (19.8 -> 17.1, 7.1 -> 6.5), and one to three percent for
+    // Q4_K / Q5_K at one row; Q4_0, IQ4_XS and IQ3_S at one row lose 3-10 % on 5120 -> 5120 and stay at four
+    unsigned wpb = 4;
+    if (b == 2 || (fmt == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q5_K))) wpb = 2;
+    const unsigned wpb_forced = env_u("REIN_MV_WPB", 0);
+    if (wpb_forced == 1 || wpb_forced == 2 || wpb_forced == 4) wpb = wpb_forced;
     const unsigned groups = (out_dim + r - 1) / r;
     const unsigned grid = (groups + wpb - 1) / wpb;
     const std::string name = std::string("rein_mv_") + fmt_tag(fmt) + "_r" + std::to_string(r) + "_b" + std::to_string(b);
