@@ -370,7 +370,7 @@ def test_moe_topk_wave_kernel_equals_the_workgroup_kernel(monkeypatch):
     # up to 256 experts the router runs one wavefront per token; it must give the ids and the weight bits of the
     # workgroup kernel (REIN_TOPK_WAVE=0): random logits, ties, NaN and -inf entries, every tail of the 4-token group
     rng = np.random.default_rng(77)
-    cases = [(1, 2, 1), (1, 2, 2), (3, 64, 8), (5, 65, 4), (7, 127, 8), (512, 128, 8), (513, 129, 8), (9, 200, 4),
+    cases = [(1, 1, 1), (5, 1, 1), (1, 2, 1), (1, 2, 2), (3, 64, 8), (5, 65, 4), (7, 127, 8), (512, 128, 8), (513, 129, 8), (9, 200, 4),
              (33, 256, 64), (2, 256, 1), (6, 17, 17), (4, 192, 33)]
     cases += [(int(rng.integers(1, 70)), int(ne), int(rng.integers(1, min(ne, 64) + 1)))
               for ne in rng.integers(2, 257, 40)]
@@ -589,11 +589,12 @@ def test_moe_ffn_end_to_end_small():
     assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what="moe_ffn")
 
 
-@pytest.mark.parametrize("n_tok,n_expert,n_used", [(1, 16, 4), (2, 128, 8), (1, 200, 3), (3, 64, 4), (8, 32, 4), (16, 64, 4), (25, 64, 4)])
-def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, monkeypatch):
+@pytest.mark.parametrize("n_tok,n_expert,n_used,hidden", [(1, 16, 4, 512), (2, 128, 8, 512), (1, 200, 3, 768), (2, 9, 9, 1280),
+                                                          (3, 64, 4, 512), (8, 32, 4, 768), (16, 64, 4, 512), (25, 64, 4, 512)])
+def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hidden, monkeypatch):
     # up to 1.6 routing entries per expert on average: rein_moe_ffn runs the two decode launches instead of
     # sort + grouped GEMMs; against the CPU chain, and against its own pipeline (REIN_MOE_CHAIN=0)
-    hidden, ff = 512, 256
+    ff = 256
     rng = np.random.default_rng(n_tok + n_expert)
     x = rng.standard_normal((n_tok, hidden)).astype(np.float32)
     logits = rng.standard_normal((n_tok, n_expert)).astype(np.float32)
