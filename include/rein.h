@@ -426,7 +426,9 @@ int rein_moe_down(int fmt, const void *slab, const int32_t *ids, const void *xq,
  * single counterpart in the reference; each is byte / bit identical to the launches it
  * replaces).  rein_moe_gate_up_swiglu_q8: moe_gate_up_swiglu_q4k_repacked_f32 followed by
  * quantize_q8_f32 -- xq_out[tok][slot] receives out_dim/32 BlockQ8 blocks of
- * silu(gate . x) * (up . x); Q4_K experts, out_dim a multiple of 32.
+ * silu(gate . x) * (up . x); out_dim a multiple of 32; formats Q4_K, Q5_K, Q6_K, Q8_0, Q5_1 (for
+ * the formats other than Q4_K, which the reference runs as two moe_matvec_* launches, the bytes of
+ * those two followed by swiglu_q8_f32).
  * rein_moe_down_combine: moe_matvec_*_f32 (or its *_down form) followed by moe_combine_f32 --
  * out[tok][i] = sum_j weights[tok][j] * down_exps_s[ids[tok][j]] * (W[ids[tok][j]] . xq[tok][j])[i]
  * in slot order.  Formats Q4_K, Q5_K, Q6_K, Q8_0, Q5_1. */
@@ -468,7 +470,7 @@ size_t rein_moe_workspace_bytes(const rein_moe_shape *shape);
  * [expert_ff -> hidden]; down_exps_s [n_expert] fp32 (the reference passes
  * ones).  `workspace` holds rein_moe_workspace_bytes; out [n_tok][hidden].
  * No host synchronisation, no allocation.  With at most 1.6 routing entries per expert on average
- * (5 n_tok n_used <= 8 n_expert) and Q4_K gate / up experts the same result comes from the decode
+ * (5 n_tok n_used <= 8 n_expert) the same result comes from the decode
  * kernels instead (top-k -> quantize -> rein_moe_gate_up_swiglu_q8 -> rein_moe_down_combine, the
  * launches of qwen35.rs:3071-3167 fused in pairs): no sort, one expert read per entry; for one
  * and two tokens the gate / up launch also routes and quantizes, so the FFN is two launches. */

@@ -1421,7 +1421,7 @@ int rein_moe_gate_up_swiglu_q8(int fmt, const void* gate_slab, const void* up_sl
                                rein_stream_t s)
 {
     const char* who = "rein_moe_gate_up_swiglu_q8";
-    if (fmt != REIN_TYPE_Q4_K) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": the fused form exists for Q4_K experts");
+    if (!moe_mv_fmt(fmt)) return fail(REIN_E_BAD_FORMAT, std::string(who) + ": formats are Q4_K, Q5_K, Q6_K, Q8_0, Q5_1");
     if (int rc = check_shape(who, fmt, in_dim, out_dim, n_tok)) return rc;
     if (out_dim % 32 != 0) return fail(REIN_E_BAD_SHAPE, std::string(who) + ": out_dim must be a multiple of 32 (whole BlockQ8 blocks)");
     if (n_used == 0 || n_used > 65535 || n_tok > 65535)
@@ -1441,7 +1441,7 @@ int rein_moe_gate_up_swiglu_q8(int fmt, const void* gate_slab, const void* up_sl
     // 4 / 8 / 16 tokens 32.9 / 51.9 / 88.4 us per FFN against 34.1 / 55.9 / 99.3, one token 16.9 against 15.9
     const unsigned gu_rows = env_u("REIN_MOE_GU_ROWS", 0);
     const bool r4 = gu_rows == 4 || (gu_rows != 2 && (unsigned long long)(out_dim / 32) * n_used * n_tok >= 2ull * kCUs);
-    return launch(r4 ? "rein_moe_gate_up_swiglu_q8_q4k_r4" : "rein_moe_gate_up_swiglu_q8_q4k", out_dim / 32, n_used, n_tok, r4 ? 512 : 1024, 0, s, a);
+    return launch(std::string("rein_moe_gate_up_swiglu_q8_") + fmt_tag(fmt) + (r4 ? "_r4" : ""), out_dim / 32, n_used, n_tok, r4 ? 512 : 1024, 0, s, a);
 }
 
 int rein_moe_down_combine(int fmt, const void* slab, const int32_t* ids, const float* weights, const float* down_exps_s,
@@ -1585,8 +1585,7 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     // mostly empty tile pays its full matrix work -- and are ahead up to 1.6 entries per expert: 128 experts top-8
     // at 1 / 4 / 16 / 24 tokens 16 / 33 / 89 / 125 us against 48 / 61 / 126 / 141 for the pipeline below, at 28
     // tokens 141 against 143, at 32 tokens 160 against 145.  Same integer dots, fp32 sums in the decode kernels' order.
-    const bool chain = 5ull * ne <= 8ull * sh.n_expert && sh.gate_up_fmt == REIN_TYPE_Q4_K && sh.expert_ff % 32 == 0 &&
-                       env_u("REIN_MOE_CHAIN", 1) != 0;
+    const bool chain = 5ull * ne <= 8ull * sh.n_expert && sh.expert_ff % 32 == 0 && env_u("REIN_MOE_CHAIN", 1) != 0;
     if (chain) {
         const unsigned ns_h = sh.hidden / 32, ns_f = sh.expert_ff / 32;
         // Where the one-wavefront router applies it shares a launch: for one or two tokens the gate / up launch
@@ -1601,7 +1600,7 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
                          (void*)&sh.hidden, (void*)&sh.expert_ff, (void*)&bpe, (void*)&sh.n_expert, (void*)&sh.n_used};
             const unsigned gu_rows = env_u("REIN_MOE_GU_ROWS", 0);
             const bool r4 = gu_rows == 4 || (gu_rows != 2 && (unsigned long long)(sh.expert_ff / 32) * sh.n_used * sh.n_tok >= 2ull * kCUs);
-            if (int rc = launch(r4 ? "rein_moe_route_gate_up_swiglu_q8_q4k_r4" : "rein_moe_route_gate_up_swiglu_q8_q4k", sh.expert_ff / 32,
+            if (int rc = launch(std::string("rein_moe_route_gate_up_swiglu_q8_") + fmt_tag(sh.gate_up_fmt) + (r4 ? "_r4" : ""), sh.expert_ff / 32,
                                 sh.n_used, sh.n_tok, r4 ? 512 : 1024, ns_h * 40u, s, a)) return rc;
         } else {
             if (wave) {

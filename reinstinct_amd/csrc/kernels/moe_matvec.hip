@@ -331,6 +331,15 @@ void moe_gate_up_swiglu_q4k_repacked_f32(const unsigned char* __restrict__ gate_
 // two rows per wavefront and 1024 threads, or four and 512 (more bytes in flight per lane, half the wavefronts)
 REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k, REIN_Q4_K, 2)
 REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k_r4, REIN_Q4_K, 4)
+// the other expert formats (the reference fuses gate + up + SwiGLU for Q4_K only and runs two matvecs otherwise)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q5k, REIN_Q5_K, 2)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q5k_r4, REIN_Q5_K, 4)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q6k, REIN_Q6_K, 2)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q6k_r4, REIN_Q6_K, 4)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q8_0, REIN_Q8_0, 2)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q8_0_r4, REIN_Q8_0, 4)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q5_1, REIN_Q5_1, 2)
+REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q5_1_r4, REIN_Q5_1, 4)
 
 #define REIN_DEFINE_MOE_RGUQ8(name, FMT, R)                                                               \
     extern "C" __global__ __launch_bounds__(64 * (32 / R)) void name(                                     \
@@ -345,6 +354,14 @@ REIN_DEFINE_MOE_GUQ8(rein_moe_gate_up_swiglu_q8_q4k_r4, REIN_Q4_K, 4)
     }
 REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q4k, REIN_Q4_K, 2)
 REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q4k_r4, REIN_Q4_K, 4)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q5k, REIN_Q5_K, 2)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q5k_r4, REIN_Q5_K, 4)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q6k, REIN_Q6_K, 2)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q6k_r4, REIN_Q6_K, 4)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q8_0, REIN_Q8_0, 2)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q8_0_r4, REIN_Q8_0, 4)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q5_1, REIN_Q5_1, 2)
+REIN_DEFINE_MOE_RGUQ8(rein_moe_route_gate_up_swiglu_q8_q5_1_r4, REIN_Q5_1, 4)
 
 #define REIN_DEFINE_MOE_DC(name, FMT, R, LANES)                                                           \
     extern "C" __global__ __launch_bounds__(512) void name(                                               \

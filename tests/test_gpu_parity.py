@@ -589,20 +589,21 @@ def test_moe_ffn_end_to_end_small():
     assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what="moe_ffn")
 
 
+@pytest.mark.parametrize("gu_fmt", [rein.Q4_K, rein.Q6_K, rein.Q8_0])
 @pytest.mark.parametrize("n_tok,n_expert,n_used,hidden", [(1, 16, 4, 512), (2, 128, 8, 512), (1, 200, 3, 768), (2, 9, 9, 1280),
                                                           (3, 64, 4, 512), (8, 32, 4, 768), (16, 64, 4, 512), (25, 64, 4, 512)])
-def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hidden, monkeypatch):
+def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hidden, gu_fmt, monkeypatch):
     # up to 1.6 routing entries per expert on average: rein_moe_ffn runs the two decode launches instead of
     # sort + grouped GEMMs; against the CPU chain, and against its own pipeline (REIN_MOE_CHAIN=0)
     ff = 256
     rng = np.random.default_rng(n_tok + n_expert)
     x = rng.standard_normal((n_tok, hidden)).astype(np.float32)
     logits = rng.standard_normal((n_tok, n_expert)).astype(np.float32)
-    gate = np.concatenate([make_weights(rein.Q4_K, hidden, ff, 300 + e, True)[1] for e in range(n_expert)])
-    up = np.concatenate([make_weights(rein.Q4_K, hidden, ff, 400 + e, True)[1] for e in range(n_expert)])
+    gate = np.concatenate([make_weights(gu_fmt, hidden, ff, 300 + e, True)[1] for e in range(n_expert)])
+    up = np.concatenate([make_weights(gu_fmt, hidden, ff, 400 + e, True)[1] for e in range(n_expert)])
     down = np.concatenate([make_weights(rein.Q6_K, ff, hidden, 500 + e, True)[1] for e in range(n_expert)])
     ones = np.ones(n_expert, np.float32)
-    sh = runtime.moe_shape(n_tok, hidden, n_expert, n_used, ff, rein.Q4_K, rein.Q6_K)
+    sh = runtime.moe_shape(n_tok, hidden, n_expert, n_used, ff, gu_fmt, rein.Q6_K)
     ws = hip.DeviceBuf(runtime.moe_workspace_bytes(sh))
     dx, dl, dg, du, dd, ds = dev(x), dev(logits), dev(gate), dev(up), dev(down), dev(ones)
     outs = []
@@ -615,9 +616,9 @@ def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hi
     ids, wts = orc.moe_topk(logits, n_used)
     perm, eoff, _ = orc.moe_sort(ids, n_expert, 32)
     gin = orc.moe_gather_xq(orc.quantize_q8(x), perm, hidden // 32, n_used)
-    bpe_gu, bpe_dn = orc.repacked_len(orc.Q4_K, hidden, ff), orc.repacked_len(orc.Q6_K, ff, hidden)
-    eg = orc.grouped_gemm(orc.Q4_K, gate, bpe_gu, eoff, gin, hidden, ff)
-    eu = orc.grouped_gemm(orc.Q4_K, up, bpe_gu, eoff, gin, hidden, ff)
+    bpe_gu, bpe_dn = orc.repacked_len(gu_fmt, hidden, ff), orc.repacked_len(orc.Q6_K, ff, hidden)
+    eg = orc.grouped_gemm(gu_fmt, gate, bpe_gu, eoff, gin, hidden, ff)
+    eu = orc.grouped_gemm(gu_fmt, up, bpe_gu, eoff, gin, hidden, ff)
     gout = orc.grouped_gemm(orc.Q6_K, down, bpe_dn, eoff, orc.quantize_q8(orc.swiglu_mul(eg, eu)), ff, hidden)
     want = orc.moe_combine(orc.moe_scatter_rows(gout, perm, hidden).reshape(n_tok, n_used, hidden), ids, wts, ones)
     for got, what in zip(outs, ("decode launches", "pipeline")):
