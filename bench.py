@@ -685,7 +685,8 @@ def main():
 
     if not args.no_configs:
         out["configs"] = {"mmq_configs2": extras_mmq(stream), "mmq_short_prompts": extras_mmq_small(stream),
-                          "moe_configs3": extras_moe(stream), "decode_stream_configs4": extras_decode_stream(stream)}
+                          "moe_configs3": extras_moe(stream), "moe_configs3_one_token": extras_moe_decode(stream),
+                          "decode_stream_configs4": extras_decode_stream(stream)}
 
     if args.sweep:
         sweep = []
@@ -704,7 +705,7 @@ def main():
 
     if args.extras:
         out["extras"] = {"fused_producers": extras_fused(stream),
-                         "moe_decode": extras_moe_decode(stream), "other_matvec_sites": extras_ondisk(stream),
+                         "other_matvec_sites": extras_ondisk(stream),
                          "decode_ffn_chain": extras_decode_ffn(stream)}
 
     if not args.no_cpu:
