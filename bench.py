@@ -241,6 +241,8 @@ def mmq_kernel_name(fmt, in_dim, out_dim, p_rows):
     tag = {rein.Q4_K: "q4k", rein.Q5_K: "q5k", rein.Q6_K: "q6k"}.get(fmt, FMT_NAME[fmt])
     ws_bytes = runtime.mmq_workspace_bytes(fmt, in_dim, p_rows)
     form = runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, ws_bytes)
+    if form == 4:
+        return "rein_mmq16_prep + rein_mmq16_q4k (fp16 formulation, REIN_MMQ16=1)"
     if form == 2:
         return f"rein_mmq6_prep + rein_mmq6_{tag}_sk (split-tail launch) + rein_mmq6_tail_sum"
     if form == 3:
