@@ -40,6 +40,7 @@ from reinstinct_amd._lib import init  # noqa: E402
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 CACHE_BYTES = 512 << 20        # rotate over more than L2 (32 MB) + Infinity Cache (256 MB)
+MMQ_ROTATION_BYTES = 320 << 20  # the same for the GEMM legs (fewer, longer launches)
 
 FMT_NAME = {rein.Q4_0: "q4_0", rein.Q4_K: "q4_k", rein.Q5_K: "q5_k", rein.Q6_K: "q6_k", rein.Q8_0: "q8_0",
             rein.IQ4_XS: "iq4_xs", rein.IQ3_S: "iq3_s"}
@@ -69,21 +70,28 @@ def matvec_bytes(fmt, in_dim, out_dim, batch):
     return quant.repacked_len(fmt, in_dim, out_dim) + batch * (in_dim // 32) * 40 + batch * out_dim * 4
 
 
+def weight_rotation(packed, min_bytes=CACHE_BYTES):
+    """Distinct device copies of one slab, together larger than L2 + Infinity Cache."""
+    first = hip.DeviceBuf.from_host(packed)
+    bufs = [first]
+    for _ in range(max(2, -(-min_bytes // packed.nbytes)) - 1):
+        b = hip.DeviceBuf(packed.nbytes)
+        rein.lib.rein_memcpy_d2d(b.ptr, first.ptr, packed.nbytes)
+        bufs.append(b)
+    return bufs
+
+
 class MatvecCase:
     """A rotation of weight buffers and a captured graph of one pass over them."""
 
-    def __init__(self, fmt, in_dim, out_dim, batch, stream, seed=0, min_bytes=CACHE_BYTES, packed=None):
+    def __init__(self, fmt, in_dim, out_dim, batch, stream, seed=0, min_bytes=CACHE_BYTES, packed=None, weights=None):
         self.fmt, self.in_dim, self.out_dim, self.batch, self.stream = fmt, in_dim, out_dim, batch, stream
-        if packed is None:
-            _, packed = synth_weights(fmt, in_dim, out_dim, seed)
-        self.packed = packed
-        self.n_buf = max(2, -(-min_bytes // packed.nbytes))
-        first = hip.DeviceBuf.from_host(packed)
-        self.weights = [first]
-        for _ in range(self.n_buf - 1):
-            b = hip.DeviceBuf(packed.nbytes)
-            rein.lib.rein_memcpy_d2d(b.ptr, first.ptr, packed.nbytes)
-            self.weights.append(b)
+        if weights is None:
+            if packed is None:
+                _, packed = synth_weights(fmt, in_dim, out_dim, seed)
+            weights = weight_rotation(packed, min_bytes)
+        self.weights = weights
+        self.n_buf = len(weights)
         x = np.random.default_rng(seed + 1).standard_normal((batch, in_dim)).astype(np.float32)
         self.x = x
         self.dx = hip.DeviceBuf.from_host(x)
@@ -127,12 +135,9 @@ class MmqCase:
     def __init__(self, fmt, p_rows, in_dim, out_dim, stream, seed=0):
         self.fmt, self.p, self.in_dim, self.out_dim, self.stream = fmt, p_rows, in_dim, out_dim, stream
         _, packed = synth_weights(fmt, in_dim, out_dim, seed)
-        self.n_buf = 4                                  # 4 x 89 MB of weights > Infinity Cache
-        self.weights = [hip.DeviceBuf.from_host(packed)]
-        for _ in range(self.n_buf - 1):
-            b = hip.DeviceBuf(packed.nbytes)
-            rein.lib.rein_memcpy_d2d(b.ptr, self.weights[0].ptr, packed.nbytes)
-            self.weights.append(b)
+        # more than L2 (32 MB) + Infinity Cache (256 MB) of distinct weights: Q4_K 5120 x 17408 is 51.5 MB -> 7 copies
+        self.weights = weight_rotation(packed, MMQ_ROTATION_BYTES)
+        self.n_buf = len(self.weights)
         x = np.random.default_rng(seed + 1).standard_normal((p_rows, in_dim)).astype(np.float32)
         self.dx = hip.DeviceBuf.from_host(x)
         self.dq = hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
@@ -255,12 +260,13 @@ def mmq_kernel_name(fmt, in_dim, out_dim, p_rows):
 
 
 def extras_mmq(stream):
-    """BASELINE configs[2]: B in {Q4_K, Q6_K, Q8_0} x M in {128, 512, 2048}, 5120 x 17408"""
+    """BASELINE configs[2]: B in {Q4_K, Q6_K, Q8_0} x M in {128, 512, 2048}, 5120 x 17408; Q5_K beside them (the
+    reference publishes its MMQ figure too, src/runtime/kernels.rs:2852-2944)"""
     out = []
     k, n = 5120, 17408
-    for f in (rein.Q4_K, rein.Q6_K, rein.Q8_0):
+    for f in (rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.Q8_0):
         packed = tiled_weights(f, k, n, seed=3)
-        ws = [hip.DeviceBuf.from_host(packed) for _ in range(4)]          # 4 x (52..95) MB > Infinity Cache
+        ws = weight_rotation(packed, MMQ_ROTATION_BYTES)                    # > L2 + Infinity Cache of distinct weights
         for m in (128, 512, 2048):
             x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
             dx, dq, dy = hip.DeviceBuf.from_host(x), hip.DeviceBuf(m * (k // 32) * 40), hip.DeviceBuf(m * n * 4)
@@ -573,11 +579,54 @@ def extras_fused(stream):
 
 
 HEADLINE_SHAPES = ((5120, 5120), (5120, 34816), (17408, 5120))      # (K, N) of configs[1]
-# HBM bytes per launch of the dominant kernel (Q4_K 5120 -> 34816, batch 1) from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by the same counter's reading for the
-# set-up device-to-device copies of known size (fetch x1.9992, write x1.0); it cannot be read
-# live, so it is the recorded figure and only reported for the configuration it was taken on
-DOMINANT_TRAFFIC_BYTES = 109573400
+# HBM bytes per launch of the three Q4_K batch-1 launches from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file, each scaled by the same counter's reading for the set-up
+# device-to-device copies of known size (fetch x1.9992, write x1.0).  Counters cannot be read
+# live from inside the process, so these are the recorded figures of
+# profiles/rein_mv_q4k_b1_decode_shapes.txt, reported only for the configuration they were taken on.
+RECORDED_TRAFFIC_BYTES = {(5120, 5120): 15259700, (5120, 34816): 109573400, (17408, 5120): 52919800}
+# the kernel each shape runs (rows per wavefront chosen by the library)
+HEADLINE_KERNELS = {(5120, 5120): "rein_mv_q4k_r2_b1", (5120, 34816): "rein_mv_q4k_r4_b1", (17408, 5120): "rein_mv_q4k_r2_b1"}
+
+
+def read_ceiling_us(stream, weights, nbytes):
+    """Microseconds per launch of the plain read-only kernel (16 B per lane, nothing else) over the same
+    rotation of buffers, in a graph of back-to-back launches like the matvecs: what a read of these bytes
+    takes on this machine.  Best of three grid sizes."""
+    import ctypes as C
+    f = hip.Module.builtin().function("rein_measure_read16")
+    sink = hip.DeviceBuf(16)
+    best = None
+    for grid in (2048, 4096, 8192):
+        sec = time_graph(stream, lambda: [f.launch((grid, 1, 1), (256, 1, 1), 0, stream,
+                                                   [C.c_void_p(b.ptr), C.c_size_t(nbytes // 16), C.c_void_p(sink.ptr)])
+                                          for b in weights], len(weights))
+        best = sec if best is None else min(best, sec)
+    return best * 1e6
+
+
+def decode_sweep(stream, steps):
+    """BASELINE configs[1] as a sweep: Q4_K and Q6_K over the three decode shapes at batch 1, 2, 4, 8, the
+    other four formats at the gate+up shape; every cell over its own rotation of > 512 MB of weights.
+    `vs_batch1` is the cell's time over the batch-1 time of the same format and shape."""
+    plan = [(f, HEADLINE_SHAPES) for f in (rein.Q4_K, rein.Q6_K)]
+    plan += [(f, ((5120, 34816),)) for f in (rein.Q4_0, rein.Q5_K, rein.Q8_0, rein.IQ4_XS)]
+    out = []
+    for f, shapes in plan:
+        for (k, n) in shapes:
+            rot = weight_rotation(tiled_weights(f, k, n, seed=5))
+            base = None
+            for b in (1, 2, 4, 8):
+                c = MatvecCase(f, k, n, b, stream, seed=5, weights=rot)
+                _, sl = c.time(max(3, steps // 4), 1)
+                base = sl if base is None else base
+                g = c.bytes_per_launch / sl / 1e9
+                out.append({"fmt": FMT_NAME[f], "K": k, "N": n, "batch": b, "us": round(sl * 1e6, 2), "GBs": round(g, 0),
+                            "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 3), "vs_batch1": round(sl / base, 3)})
+                log("decode sweep", out[-1])
+                del c
+            del rot
+    return out
 
 
 def main():
@@ -636,7 +685,16 @@ def main():
     step_bytes = sum(c.bytes_per_launch * c.n_buf for c in cases)
     value = step_bytes * args.steps / total_s / 1e9
     is_headline = fmt == rein.Q4_K and args.batch == 1
-    dom = shapes[1]                                   # gate+up: most bytes, its own kernel variant
+    # the roofline object describes the launch the target is quoted on: K = 5120 -> N = 5120 (it is also the
+    # launch furthest from the roof); the other two shapes and the step aggregate are in config.shapes / value
+    dom = shapes[0]
+    for sh, c in zip(shapes, cases):
+        sh["read_only_ceiling_us"] = round(read_ceiling_us(stream, c.weights, c.bytes_per_launch), 3)
+        sh["frac_of_read_only_ceiling"] = round(sh["read_only_ceiling_us"] / sh["us_per_launch"], 3)
+        if is_headline:
+            sh["kernel"] = HEADLINE_KERNELS[(sh["K"], sh["N"])]
+            sh["traffic_recorded"] = RECORDED_TRAFFIC_BYTES[(sh["K"], sh["N"])]
+        log(f"read-only kernel over the same {sh['bytes_per_launch']} bytes: {sh['read_only_ceiling_us']} us")
 
     out = {
         "metric": "Q4_K decode matvec HBM GB/s (% of peak) + MMQ pp512 int8 TOPS, 1 MI355X",
@@ -648,11 +706,15 @@ def main():
                                "/ total time; step = one pass of each shape over its rotation of distinct weight buffers",
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2), "shapes": shapes},
         "roofline": {"bound": "hbm", "achieved": dom["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": dom["frac_of_hbm_peak"], "traffic": DOMINANT_TRAFFIC_BYTES if is_headline else None,
+                     "frac": dom["frac_of_hbm_peak"], "traffic": dom.get("traffic_recorded"),
                      "traffic_source": "recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file "
-                                       "(profiles/rein_mv_q4k_b1_decode_shapes.txt), not read in this run" if is_headline else None,
-                     "kernel": "rein_mv_q4k_r4_b1 (K=5120 -> N=34816)", "us_per_launch": dom["us_per_launch"],
-                     "algorithmic_bytes_per_launch": dom["bytes_per_launch"]},
+                                       "(profiles/rein_mv_q4k_b1_decode_shapes.txt), not read in this run; the other two "
+                                       "shapes in config.shapes[].traffic_recorded" if is_headline else None,
+                     "kernel": f"{HEADLINE_KERNELS[(dom['K'], dom['N'])] if is_headline else 'decode matvec'} "
+                               f"(K={dom['K']} -> N={dom['N']}, the shape the 70 % target is quoted on)",
+                     "us_per_launch": dom["us_per_launch"], "algorithmic_bytes_per_launch": dom["bytes_per_launch"],
+                     "read_only_ceiling_us": dom["read_only_ceiling_us"],
+                     "step_aggregate_frac": round(value / HBM_PEAK_GBS, 4)},
     }
 
     if is_headline:
@@ -682,11 +744,15 @@ def main():
                       "us_per_launch": round(sec * 1e6, 2), "value": round(tops, 2), "unit": "int8 TOPS",
                       "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                    "frac": round(tops / INT8_PEAK_TOPS, 4),
-                                   "kernel": mmq_kernel_name(rein.Q4_K, 5120, 17408, 512)}}
+                                   "kernel": mmq_kernel_name(rein.Q4_K, 5120, 17408, 512),
+                                   "counters_recorded": {"mfma_busy_frac_of_simd_cycles": 0.337, "valu_issue_frac": 0.487,
+                                                         "hbm_fetch_bytes": 148.7e6, "input_bytes": 57.1e6,
+                                                         "source": "rocprofv3 --pmc runs of this file, profiles/rein_mmq6_q4k_sk_pp512.txt; "
+                                                                   "not read in this run"}}}
         del mm
 
     if not args.no_configs:
-        out["configs"] = {"mmq_configs2": extras_mmq(stream), "mmq_short_prompts": extras_mmq_small(stream),
+        out["configs"] = {"decode_sweep_configs1": decode_sweep(stream, args.steps), "mmq_configs2": extras_mmq(stream), "mmq_short_prompts": extras_mmq_small(stream),
                           "moe_configs3": extras_moe(stream), "moe_configs3_one_token": extras_moe_decode(stream),
                           "decode_stream_configs4": extras_decode_stream(stream)}
 

@@ -78,6 +78,39 @@ int rein_init(const char *hsaco_path);
 /* 1 when rein_init has succeeded in this process */
 int rein_is_loaded(void);
 
+/* ----------------------------------------------------------------- options */
+/* The switches that pin a launch choice (which kernel family, which tiling) instead of
+ * leaving it to the library's cost models.  No counterpart in the reference, whose launch
+ * shapes are fixed; the tests use them to reach every kernel family, and a host may pin a
+ * choice it has measured.  An option is unset (the library decides) or set to an unsigned
+ * decimal number.  The environment variables of the same names are read ONCE per process, when
+ * the table is first looked at (rein_init looks); after that only these calls change it, so
+ * what an entry point launches depends on its arguments and on this table alone.  A set option
+ * pins its choice whatever its value: several cost models step aside as soon as the option that
+ * overrides them is set, and setting it back to NULL / "" hands the choice back.  Entries are
+ * single atomic words; changing one while another thread launches is safe.
+ * Names (rein_option_name enumerates them): REIN_MV_ROWS, REIN_MV_WPB (decode matvec rows per
+ * wavefront 1/2/4, wavefronts per workgroup 1/2/4), REIN_SKINNY_FROM, REIN_SKINNY_KS,
+ * REIN_QUAD_FROM (batched decode: row count from which the skinny MMQ / the 4x4x4 kernel run,
+ * wavefronts per row tile), REIN_GROUPED_STRIDED (1: the reference-named strided grouped
+ * kernel), REIN_MMQ_TM, REIN_MMQ_N64 (int8 GEMM tile: 32 forces 32-token tiles; 64-token tiles
+ * per row block), REIN_MMQ_SK, REIN_MMQ_SK_GRID, REIN_MMQ_SK_SPLIT, REIN_MMQ_SK_TM (split-tail
+ * launch of the int8 tile: 0 off / 2 forced, resident workgroups, ranges per tail unit, unit
+ * width), REIN_MMQ6, REIN_MMQ6_FROM, REIN_MMQ6_N4, REIN_MMQ6_N2, REIN_MMQ6_SK,
+ * REIN_MMQ6_SK_GRID, REIN_MMQ6_SK_SPLIT (Q4_K fp6 launch: 0 off, first row count, token groups
+ * of four / two tiles per row block, split-tail 0 off / 2 forced, its grid and ranges),
+ * REIN_MMQ16 (1: the fp16 formulation where the code object holds it), REIN_TOPK_WAVE,
+ * REIN_MOE_SORT_SPLIT, REIN_MOE_CHAIN, REIN_MOE_FUSED, REIN_MOE_GU_ROWS, REIN_MOE_DC_ROWS (MoE
+ * glue: 0 = the workgroup router, 1 = the four-launch sort, 0 = no decode chain for few
+ * tokens, 0 = unfused gate/up, rows per workgroup of the two decode launches).
+ * Unknown name: REIN_E_NOT_FOUND; a value that is not an unsigned 32-bit decimal:
+ * REIN_E_BAD_SHAPE. */
+int rein_set_option(const char *name, const char *value);   /* value NULL or "": unset */
+int rein_get_option(const char *name, unsigned *value, int *is_set);
+int rein_reset_options(void);                                /* every option unset (the environment is not read again) */
+int rein_option_count(void);
+const char *rein_option_name(int index);                     /* NULL outside [0, rein_option_count()) */
+
 /* src/hip/mod.rs:25-58, 88-131 */
 int rein_device_count(int *n);
 int rein_set_device(int device);
@@ -308,7 +341,8 @@ size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 /* Which launch rein_mmq_xq8_ws takes for this shape and workspace size: 0 = the int8 launch of
  * rein_mmq_xq8, 1 = fp6 with one token group per workgroup, 2 = fp6 split-tail, 3 = int8
  * split-tail, 4 = the fp16 formulation that sums whole superblocks in the matrix unit (only
- * with REIN_MMQ16=1 in the environment: slower than the others, kept for study). */
+ * with the option REIN_MMQ16 set to 1 and a code object built with it: slower than the others,
+ * kept for study). */
 int rein_mmq_form_ws(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t workspace_bytes);
 int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                     unsigned out_dim, unsigned p_rows, void *workspace, size_t workspace_bytes,
@@ -320,7 +354,16 @@ int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned i
  * (librein_scratch.so, loaded from the directory of librein.so on the first call).  Shapes whose
  * rein_mmq_workspace_min_bytes exceeds 8 MiB are refused with REIN_E_TOO_LARGE (at in_dim 5120
  * that is above 768 rows); shapes that need no workspace run rein_mmq_xq8.  All calls on one
- * GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+ * GPU share the array: calls that overlap on one GPU (two streams, two threads) race.
+ * "Allocates nothing" holds once the array's address is known on the current device: the first
+ * look loads librein_scratch.so and asks the runtime for the symbol's address, which makes the
+ * runtime place (and zero) the array on that device.  That step must not fall into a stream
+ * capture: call rein_noalloc_prepare() once per device, with that device current and nothing
+ * capturing (it also looks up the kernel handles the entry point launches), or make the first
+ * call of rein_mmq_xq8_noalloc on the device outside any capture.  Neither this entry point nor
+ * rein_noalloc_prepare has a counterpart in the reference; both are for callers that cannot
+ * allocate. */
+int rein_noalloc_prepare(void);
 int rein_mmq_xq8_noalloc(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                          unsigned out_dim, unsigned p_rows, rein_stream_t s);
 /* How rein_mmq_xq8_ws cuts the tokens of a 128-row block: n4 groups of four 32-token tiles,

@@ -36,6 +36,11 @@ SIGNATURES = {
     "rein_last_error": (C.c_char_p, []),
     "rein_init": (_i, [C.c_char_p]),
     "rein_is_loaded": (_i, []),
+    "rein_set_option": (_i, [C.c_char_p, C.c_char_p]),
+    "rein_get_option": (_i, [C.c_char_p, _P(_u), _P(_i)]),
+    "rein_reset_options": (_i, []),
+    "rein_option_count": (_i, []),
+    "rein_option_name": (C.c_char_p, [_i]),
     "rein_device_count": (_i, [_P(_i)]),
     "rein_set_device": (_i, [_i]),
     "rein_get_device": (_i, [_P(_i)]),
@@ -86,6 +91,7 @@ SIGNATURES = {
     "rein_mmq_workspace_min_bytes": (_sz, [_i, _u, _u]),
     "rein_mmq_form_ws": (_i, [_i, _u, _u, _u, _sz]),
     "rein_mmq_xq8_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
+    "rein_noalloc_prepare": (_i, []),
     "rein_mmq_xq8_noalloc": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_mmq_tile_plan_ws": (_i, [_i, _u, _u, _vp, _vp]),
     "rein_mmq_block_dots_ws": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _sz, _vp]),
@@ -182,3 +188,19 @@ def check(rc):
 def init():
     """Bind libamdhip64.so and load the gfx950 code object (needs a GPU)."""
     check(load().rein_init(HSACO_PATH.encode()))
+
+
+def set_option(name, value):
+    """rein_set_option: pin a launch choice (value None: hand it back to the library)."""
+    check(load().rein_set_option(name.encode(), None if value is None else str(value).encode()))
+
+
+def get_option(name):
+    """-> the option's value, or None while it is unset"""
+    v, on = _u(0), _i(0)
+    check(load().rein_get_option(name.encode(), C.byref(v), C.byref(on)))
+    return v.value if on.value else None
+
+
+def reset_options():
+    check(load().rein_reset_options())

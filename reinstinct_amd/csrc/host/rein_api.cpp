@@ -10,6 +10,7 @@
 #include <cstring>
 #include <mutex>
 #include <algorithm>
+#include <atomic>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -130,11 +131,41 @@ int check_ptr(const char* who, const void* p, size_t align, const char* what)
     return 0;
 }
 
-unsigned env_u(const char* name, unsigned dflt)
+// ---- options ---------------------------------------------------------------------------------
+// Every switch that forces a launch choice (the tests use them to reach each kernel family; a host
+// may pin a choice it has measured) lives in this one table.  An option is either unset -- the
+// library decides -- or set to a number.  The environment variables of the same names are read
+// once per process, on the first look at the table (rein_init does one); afterwards only
+// rein_set_option changes an entry, so the launch an entry point chooses depends on its arguments
+// and on this table alone.  Entries are single atomic words: setting one while another thread
+// launches is safe, the launch sees the old or the new value.
+enum Opt : int { O_MV_ROWS, O_MV_WPB, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
+const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
+constexpr uint64_t kOptSet = 1ull << 63;
+std::atomic<uint64_t> g_opts[O_COUNT];          // zero = unset
+std::once_flag g_opts_env_once;
+
+void opts_from_env()
 {
-    const char* v = std::getenv(name);
-    return v && *v ? (unsigned)std::strtoul(v, nullptr, 10) : dflt;
+    for (int i = 0; i < O_COUNT; i++) {
+        const char* v = std::getenv(kOptNames[i]);
+        if (v && *v) g_opts[i].store(kOptSet | (uint32_t)std::strtoul(v, nullptr, 10), std::memory_order_relaxed);
+    }
 }
+
+uint64_t opt_raw(Opt id)
+{
+    std::call_once(g_opts_env_once, opts_from_env);
+    return g_opts[id].load(std::memory_order_relaxed);
+}
+// the option's value, or dflt while it is unset
+unsigned opt_u(Opt id, unsigned dflt)
+{
+    const uint64_t r = opt_raw(id);
+    return (r & kOptSet) ? (unsigned)(r & 0xFFFFFFFFull) : dflt;
+}
+// whether the option has been set (a set option pins a choice; several cost models step aside then)
+bool opt_is_set(Opt id) { return (opt_raw(id) & kOptSet) != 0; }
 
 constexpr unsigned kCUs = 256;    // MI355X
 
@@ -145,7 +176,7 @@ constexpr unsigned kCUs = 256;    // MI355X
 // below that.
 unsigned pick_rows_per_wave(int fmt, unsigned out_dim, unsigned batch)
 {
-    const unsigned forced = env_u("REIN_MV_ROWS", 0);
+    const unsigned forced = opt_u(O_MV_ROWS, 0);
     unsigned r = 1;
     if ((out_dim + 3) / 4 >= kCUs * 32) r = 4;
     else if ((out_dim + 1) / 2 >= kCUs * 8) r = 2;
@@ -201,7 +232,7 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
         }
         if (cost < best) { best = cost; ks = k; }
     }
-    const unsigned forced = env_u("REIN_SKINNY_KS", 0);
+    const unsigned forced = opt_u(O_SKINNY_KS, 0);
     if (forced >= 1 && forced <= ks_max) ks = forced;
     const std::string name = std::string("rein_mmqs_") + fmt_tag(fmt) + "_v" + std::to_string(nv);
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
@@ -218,7 +249,7 @@ unsigned skinny_from_rows(int fmt)
 {
     unsigned dflt = 3;
     if (fmt == REIN_TYPE_Q6_K) dflt = 5;
-    return env_u("REIN_SKINNY_FROM", dflt);
+    return opt_u(O_SKINNY_FROM, dflt);
 }
 
 // Whether a batched decode of n_rows (<= 8) activation rows runs on the 4x4x4 int8 matrix
@@ -239,7 +270,7 @@ unsigned skinny_from_rows(int fmt)
 // 21.3; level at 7168 rows, behind at 5120 and 34816).
 bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
 {
-    const unsigned forced = env_u("REIN_QUAD_FROM", 0);
+    const unsigned forced = opt_u(O_QUAD_FROM, 0);
     if (forced) return n_rows >= forced;
     if (n_rows < 3) return false;
     switch (fmt) {
@@ -264,7 +295,7 @@ bool use_quad(int fmt, unsigned out_dim, unsigned n_rows)
 // 5120 -> 2048 9.7 against 10.7, stays).
 bool small_for_matrix_cores(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    if (n_rows < 3 || std::getenv("REIN_QUAD_FROM") || std::getenv("REIN_SKINNY_FROM")) return false;
+    if (n_rows < 3 || opt_is_set(O_QUAD_FROM) || opt_is_set(O_SKINNY_FROM)) return false;
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
     if (n_rows > 4) return weights <= (6ull << 20);
     const bool quad_family = fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS;
@@ -297,7 +328,7 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     // Q4_K / Q5_K at one row; Q4_0, IQ4_XS and IQ3_S at one row lose 3-10 % on 5120 -> 5120 and stay at four
     unsigned wpb = 4;
     if (b == 2 || (fmt == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q5_K))) wpb = 2;
-    const unsigned wpb_forced = env_u("REIN_MV_WPB", 0);
+    const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
     if (wpb_forced == 1 || wpb_forced == 2 || wpb_forced == 4) wpb = wpb_forced;
     const unsigned groups = (out_dim + r - 1) / r;
     const unsigned grid = (groups + wpb - 1) / wpb;
@@ -319,7 +350,7 @@ int launch_grouped(int fmt, const void* slab0, const void* slab1, unsigned bytes
     const unsigned gx = (out_dim + 127) / 128;
     const unsigned n_slab = slab1 ? 2 : 1;
     const unsigned long long grid = 8ull * ((tile_ub + 7) / 8) * n_slab * gx;
-    if (grid <= 0x7FFFFFFFull && env_u("REIN_GROUPED_STRIDED", 0) == 0) {
+    if (grid <= 0x7FFFFFFFull && opt_u(O_GROUPED_STRIDED, 0) == 0) {
         const void* s1 = slab1 ? slab1 : slab0;
         float* o1 = y1 ? y1 : y0;
         void* a[] = {(void*)&slab0, (void*)&s1, (void*)&bytes_per_expert, (void*)&expert_off, (void*)&tile_off,
@@ -343,6 +374,54 @@ extern "C" {
 
 const char* rein_last_error(void) { return last_error(); }
 
+// ---- options (the table at the top of this file)
+namespace {
+int opt_find(const char* name)
+{
+    if (!name) return -1;
+    for (int i = 0; i < O_COUNT; i++)
+        if (std::strcmp(name, kOptNames[i]) == 0) return i;
+    return -1;
+}
+}  // namespace
+
+int rein_set_option(const char* name, const char* value)
+{
+    const int i = opt_find(name);
+    if (i < 0) return fail(REIN_E_NOT_FOUND, std::string("rein_set_option: no option named ") + (name ? name : "(null)"));
+    (void)opt_raw((Opt)i);               // the environment is read before the first explicit change, never after it
+    if (!value || !*value) {
+        g_opts[i].store(0, std::memory_order_relaxed);
+        return 0;
+    }
+    char* end = nullptr;
+    const unsigned long v = std::strtoul(value, &end, 10);
+    if (end == value || *end != 0 || v > 0xFFFFFFFFul)
+        return fail(REIN_E_BAD_SHAPE, std::string("rein_set_option: ") + name + " takes an unsigned 32-bit decimal number, got \"" + value + "\"");
+    g_opts[i].store(kOptSet | (uint64_t)v, std::memory_order_relaxed);
+    return 0;
+}
+
+int rein_get_option(const char* name, unsigned* value, int* is_set)
+{
+    const int i = opt_find(name);
+    if (i < 0) return fail(REIN_E_NOT_FOUND, std::string("rein_get_option: no option named ") + (name ? name : "(null)"));
+    const uint64_t r = opt_raw((Opt)i);
+    if (value) *value = (unsigned)(r & 0xFFFFFFFFull);
+    if (is_set) *is_set = (r & kOptSet) ? 1 : 0;
+    return 0;
+}
+
+int rein_option_count(void) { return O_COUNT; }
+const char* rein_option_name(int index) { return index >= 0 && index < O_COUNT ? kOptNames[index] : nullptr; }
+
+int rein_reset_options(void)
+{
+    (void)opt_raw(O_MV_ROWS);
+    for (int i = 0; i < O_COUNT; i++) g_opts[i].store(0, std::memory_order_relaxed);
+    return 0;
+}
+
 int rein_init(const char* hsaco_path)
 {
     std::lock_guard<std::mutex> lock(g_init_mu);
@@ -355,6 +434,7 @@ int rein_init(const char* hsaco_path)
     g_rt.api = api;
     g_rt.module = m;
     g_rt.loaded = true;
+    (void)opt_raw(O_MV_ROWS);            // the one read of the environment, if nothing looked at the table before
     return 0;
 }
 
@@ -668,7 +748,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).
     const unsigned n_rb = (out_dim + 127) / 128;
     unsigned n64 = mmq_pick_n64(fmt, in_dim, out_dim, p_rows);
-    const unsigned forced_tm = env_u("REIN_MMQ_TM", 0), forced_n64 = env_u("REIN_MMQ_N64", 0xFFFFFFFFu);
+    const unsigned forced_tm = opt_u(O_MMQ_TM, 0), forced_n64 = opt_u(O_MMQ_N64, 0xFFFFFFFFu);
     if (forced_n64 != 0xFFFFFFFFu) n64 = std::min(forced_n64, p_rows / 64);
     if (forced_tm == 32) n64 = 0;
     // every token in a 64-token tile: the 64-token kernel itself, 5-7 % ahead of the mixed kernel launched without
@@ -702,7 +782,7 @@ size_t x6_image_bytes(unsigned n_sub, unsigned p_rows)
 {
     return (size_t)((n_sub + 1) / 2) * ((p_rows + 31) / 32) * kX6Rec + 1024;      // rein_x6_bytes
 }
-bool mmq6_format(int fmt) { return fmt == REIN_TYPE_Q4_K && env_u("REIN_MMQ6", 1) != 0; }
+bool mmq6_format(int fmt) { return fmt == REIN_TYPE_Q4_K && opt_u(O_MMQ6, 1) != 0; }
 unsigned mmq6_lds_bytes(unsigned nt)       // rein_mmq6_lds_bytes<NT>(), depths of Mmq6Cfg<NT>
 {
     const unsigned r = nt == 4 ? 2 : nt == 2 ? 4 : 3, d = nt == 4 ? 3 : 4, sm = nt == 2 ? 2 : 1;
@@ -719,7 +799,7 @@ unsigned mmq6_lds_max() { return std::max(mmq6_lds_bytes(4), std::max(mmq6_lds_b
 void mmq6_pick(unsigned out_dim, unsigned p_rows, unsigned* n4_out, unsigned* n2_out)
 {
     const unsigned n_rb = (out_dim + 127) / 128, n_tt = (p_rows + 31) / 32;
-    const unsigned f4 = env_u("REIN_MMQ6_N4", 0xFFFFFFFFu), f2 = env_u("REIN_MMQ6_N2", 0xFFFFFFFFu);
+    const unsigned f4 = opt_u(O_MMQ6_N4, 0xFFFFFFFFu), f2 = opt_u(O_MMQ6_N2, 0xFFFFFFFFu);
     if (f4 != 0xFFFFFFFFu || f2 != 0xFFFFFFFFu) {
         unsigned n4 = f4 == 0xFFFFFFFFu ? 0 : std::min(f4, n_tt / 4);
         unsigned n2 = f2 == 0xFFFFFFFFu ? 0 : std::min(f2, (n_tt - 4 * n4) / 2);
@@ -785,7 +865,7 @@ size_t sk_workspace_bytes(unsigned in_dim, unsigned p_rows)
 }
 unsigned sk_grid()                 // REIN_MMQ6_SK_GRID: fewer workgroups (a multiple of 8), for tests of several rounds
 {
-    const unsigned g = env_u("REIN_MMQ6_SK_GRID", kSkGrid) & ~7u;
+    const unsigned g = opt_u(O_MMQ6_SK_GRID, kSkGrid) & ~7u;
     return g >= 8 && g <= kSkGrid ? g : kSkGrid;
 }
 // Workgroups per tail unit: at most 8 (every range pays a pipeline fill and a partial tile), at most one per
@@ -796,7 +876,7 @@ unsigned sk_split(unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
     const unsigned g = sk_grid(), n_unit = ((out_dim + 127) / 128) * (((p_rows + 31) / 32 + 3) / 4), n_tail = n_unit % g;
     if (n_tail == 0) return 1;
-    const unsigned forced = env_u("REIN_MMQ6_SK_SPLIT", 0);
+    const unsigned forced = opt_u(O_MMQ6_SK_SPLIT, 0);
     const unsigned room = (n_unit >= g ? g / 2 : g) / n_tail;
     const unsigned most = std::min(g / n_tail, in_dim / 256);
     return std::max(1u, std::min(forced ? forced : std::min(8u, room), most));
@@ -810,12 +890,12 @@ unsigned sk_split(unsigned in_dim, unsigned out_dim, unsigned p_rows)
 // forces the launch wherever it is valid.
 bool mmq6_split_tail(unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
-    const unsigned mode = env_u("REIN_MMQ6_SK", 1);
+    const unsigned mode = opt_u(O_MMQ6_SK, 1);
     if (mode == 0) return false;
-    if (std::getenv("REIN_MMQ6_N4") || std::getenv("REIN_MMQ6_N2")) return false;      // a forced token-group split
+    if (opt_is_set(O_MMQ6_N4) || opt_is_set(O_MMQ6_N2)) return false;      // a forced token-group split
     const unsigned n_tt = (p_rows + 31) / 32, n_tg = (n_tt + 3) / 4;
     if (8 * (4 * n_tg - n_tt) > n_tt) return false;                       // more than an eighth of the tiles empty
-    if (mode == 2 || std::getenv("REIN_MMQ6_SK_GRID")) return true;
+    if (mode == 2 || opt_is_set(O_MMQ6_SK_GRID)) return true;
     const unsigned rounds = ((out_dim + 127) / 128) * n_tg / sk_grid(), split = sk_split(in_dim, out_dim, p_rows);
     return (rounds == 0 && split >= 2) || (rounds == 1 && split >= 4);
 }
@@ -841,7 +921,7 @@ Sk8Plan sk8_width(unsigned tm, unsigned g, unsigned in_dim, unsigned out_dim, un
         // of two chunks and more, at most 12 (us at 4 / 8 / 10 / 12 ranges, Q8_0 17408 -> 5120 at 64 tokens:
         // 62 / 54 / 48 / 46; 5120 -> 1024: 20 / 18 / 16 / 16 at 5 / 8 / 10 / 20)
         const unsigned room = (rounds ? g / 2 : g) / p.n_tail, cap = rounds ? 8u : std::min(12u, std::max(1u, n_chunk / 2));
-        const unsigned forced = env_u("REIN_MMQ_SK_SPLIT", 0);
+        const unsigned forced = opt_u(O_MMQ_SK_SPLIT, 0);
         p.split = std::max(1u, std::min(std::min(forced ? forced : std::min(cap, room), g / p.n_tail), n_chunk));
     }
     // it pays where the tail decides: no whole round and a tail that splits, or one whole round and a tail that
@@ -856,16 +936,16 @@ Sk8Plan sk8_width(unsigned tm, unsigned g, unsigned in_dim, unsigned out_dim, un
 Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
     const Sk8Plan none{64, kSkGrid, 0, 0, 1, false, 0.0};
-    const unsigned mode = env_u("REIN_MMQ_SK", 1);
+    const unsigned mode = opt_u(O_MMQ_SK, 1);
     if (mode == 0 || p_rows <= 16 || in_dim == 0 || out_dim == 0 || !fmt_tag(fmt) || fmt == REIN_TYPE_Q5_1) return none;
-    if (std::getenv("REIN_MMQ_TM") || std::getenv("REIN_MMQ_N64")) return none;        // a forced tiling
-    const unsigned gg = env_u("REIN_MMQ_SK_GRID", kSkGrid) & ~7u;        // fewer workgroups: tests of several rounds
+    if (opt_is_set(O_MMQ_TM) || opt_is_set(O_MMQ_N64)) return none;        // a forced tiling
+    const unsigned gg = opt_u(O_MMQ_SK_GRID, kSkGrid) & ~7u;        // fewer workgroups: tests of several rounds
     const unsigned g = gg >= 8 && gg <= kSkGrid ? gg : kSkGrid;
-    const bool force = mode == 2 || std::getenv("REIN_MMQ_SK_GRID");
+    const bool force = mode == 2 || opt_is_set(O_MMQ_SK_GRID);
     const unsigned n_tt = (p_rows + 31) / 32;
     const bool half_empty = 8 * (2 * ((n_tt + 1) / 2) - n_tt) > n_tt;   // more than an eighth of the 64-token units' tiles
     Sk8Plan w64 = sk8_width(64, g, in_dim, out_dim, p_rows), w32 = sk8_width(32, g, in_dim, out_dim, p_rows);
-    if (const unsigned forced_tm = env_u("REIN_MMQ_SK_TM", 0)) {
+    if (const unsigned forced_tm = opt_u(O_MMQ_SK_TM, 0)) {
         Sk8Plan p = forced_tm == 32 ? w32 : w64;
         p.take = p.take || force;
         return p;
@@ -914,7 +994,7 @@ namespace {
 int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t bytes)
 {
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    const bool asked = std::getenv("REIN_MMQ6_FROM") || std::getenv("REIN_MMQ6_N4") || std::getenv("REIN_MMQ6_N2");
+    const bool asked = opt_is_set(O_MMQ6_FROM) || opt_is_set(O_MMQ6_N4) || opt_is_set(O_MMQ6_N2);
     // The fp6 launches carry the image kernel in front and, split-tail, the sum behind: below about 50 us of
     // GEMM (2 M N K < 2.8e10) that costs more than the tile saves (768 -> 2048 at 512 tokens: 21 us against 9,
     // 2048 -> 1536: 26 against 19, 1536 -> 6144: 38 against 24; 5120 -> 2560 at 1536 tokens, 4.0e10: 90 against 139).
@@ -943,12 +1023,30 @@ size_t x16_image_bytes(unsigned n_sub, unsigned p_rows)                        /
     return (size_t)(n_sub / 2) * n_grp * 16384 + (size_t)(n_sub / 8) * n_grp * 2048 + n_grp * 256 + 1024;
 }
 constexpr unsigned kMmq16Lds = 2 * 16384 + 2 * 2048 + 4 * 2 * 2 * 2048 + 4 * 2 * 1280;    // rein_mmq16_lds_bytes()
-bool mmq16_asked(int fmt, unsigned in_dim) { return fmt == REIN_TYPE_Q4_K && in_dim != 0 && in_dim % 256 == 0 && env_u("REIN_MMQ16", 0) != 0; }
+// The fp16 formulation is a study kernel: slower than the default launches and compiled into the code object
+// only when the build asks for it (make MMQ16=1).  The option is ignored where the kernel is absent.
+bool mmq16_built()
+{
+    static std::atomic<int> state{0};                   // 0 unknown, 1 present, 2 absent
+    int st = state.load(std::memory_order_relaxed);
+    if (st == 0) {
+        if (!g_rt.loaded) return false;
+        hipFunction_t f = nullptr;
+        std::lock_guard<std::mutex> lock(g_rt.mu);
+        st = g_rt.api->ModuleGetFunction(&f, g_rt.module, "rein_mmq16_q4k") == 0 && f ? 1 : 2;
+        state.store(st, std::memory_order_relaxed);
+    }
+    return st == 1;
+}
+bool mmq16_asked(int fmt, unsigned in_dim)
+{
+    return fmt == REIN_TYPE_Q4_K && in_dim != 0 && in_dim % 256 == 0 && opt_u(O_MMQ16, 0) != 0 && mmq16_built();
+}
 }  // namespace
 
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
-    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < env_u("REIN_MMQ6_FROM", 320)) return 0;
+    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < opt_u(O_MMQ6_FROM, 320)) return 0;
     return x6_image_bytes(in_dim / 32, p_rows);
 }
 
@@ -959,9 +1057,9 @@ size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows)
     if (rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows) == 0) {
         // the int8 launch needs none; with room for its partial tiles it may run as a split-tail launch
         const bool dense = fmt_tag(fmt) && fmt != REIN_TYPE_Q5_1 && in_dim != 0 && p_rows > 16;
-        return dense && env_u("REIN_MMQ_SK", 1) != 0 ? (size_t)kSkGrid * kSk8PartBytes : 0;
+        return dense && opt_u(O_MMQ_SK, 1) != 0 ? (size_t)kSkGrid * kSk8PartBytes : 0;
     }
-    const size_t fp6 = env_u("REIN_MMQ6_SK", 1) != 0 ? sk_workspace_bytes(in_dim, p_rows) : x6_image_bytes(in_dim / 32, p_rows);
+    const size_t fp6 = opt_u(O_MMQ6_SK, 1) != 0 ? sk_workspace_bytes(in_dim, p_rows) : x6_image_bytes(in_dim / 32, p_rows);
     return mmq16_asked(fmt, in_dim) ? std::max(fp6, x16_image_bytes(in_dim / 32, p_rows)) : fp6;
 }
 
@@ -1059,6 +1157,21 @@ int static_scratch(void** ptr, size_t* bytes)
     return 0;
 }
 }  // namespace
+
+int rein_noalloc_prepare(void)
+{
+    if (int rc = need_runtime()) return rc;
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    if (int rc = static_scratch(&ptr, &bytes)) return rc;
+    // the kernels the entry point can launch: their handles are looked up now, not under a capture
+    static const char* const names[] = {"rein_mmq6_prep", "rein_mmq6_q4k_mix", "rein_mmq_q4k_t32", "rein_mmq_q4k_t64", "rein_mmq_q4k_mix"};
+    for (const char* n : names) {
+        hipFunction_t f;
+        if (int rc = get_fn(n, &f)) return rc;
+    }
+    return 0;
+}
 
 int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
                          unsigned p_rows, rein_stream_t s)
@@ -1202,7 +1315,7 @@ int rein_moe_topk(const float* logits, unsigned n_tok, unsigned n_expert, unsign
     if (int rc = check_ptr("rein_moe_topk", out_ids, 4, "out_ids")) return rc;
     if (int rc = check_ptr("rein_moe_topk", out_weights, 4, "out_weights")) return rc;
     int ne = (int)n_expert, nu = (int)n_used;
-    if (n_expert <= 256 && env_u("REIN_TOPK_WAVE", 1) != 0) {
+    if (n_expert <= 256 && opt_u(O_TOPK_WAVE, 1) != 0) {
         // one wavefront per token, the tree's decisions as register reductions (no LDS, no barrier): the same ids
         // and weight bits as moe_topk_f32
         int nt = (int)n_tok;
@@ -1218,7 +1331,7 @@ namespace {
 // 4096 entries of 512 tokens x top-8 take it ~5 us, about one launch of the split form.
 bool moe_sort_in_one_block(unsigned n_entries, unsigned n_expert)
 {
-    return n_entries <= 32768 && n_expert <= 2048 && env_u("REIN_MOE_SORT_SPLIT", 0) == 0;
+    return n_entries <= 32768 && n_expert <= 2048 && opt_u(O_MOE_SORT_SPLIT, 0) == 0;
 }
 }  // namespace
 
@@ -1439,7 +1552,7 @@ int rein_moe_gate_up_swiglu_q8(int fmt, const void* gate_slab, const void* up_sl
     // two rows per wavefront (1024 threads per 32 outputs) or four (512): four once the launch is two workgroups
     // per CU -- more bytes in flight per lane, half the wavefronts to start; 128 experts top-8, 2048 -> 768 at
     // 4 / 8 / 16 tokens 32.9 / 51.9 / 88.4 us per FFN against 34.1 / 55.9 / 99.3, one token 16.9 against 15.9
-    const unsigned gu_rows = env_u("REIN_MOE_GU_ROWS", 0);
+    const unsigned gu_rows = opt_u(O_MOE_GU_ROWS, 0);
     const bool r4 = gu_rows == 4 || (gu_rows != 2 && (unsigned long long)(out_dim / 32) * n_used * n_tok >= 2ull * kCUs);
     return launch(std::string("rein_moe_gate_up_swiglu_q8_") + fmt_tag(fmt) + (r4 ? "_r4" : ""), out_dim / 32, n_used, n_tok, r4 ? 512 : 1024, 0, s, a);
 }
@@ -1469,7 +1582,7 @@ int rein_moe_down_combine(int fmt, const void* slab, const int32_t* ids, const f
     const unsigned lanes = half ? 32 : 64;
     unsigned threads = ((n_used * lanes + 63) / 64) * 64;
     if (threads > 512) threads = 512;
-    unsigned rows = env_u("REIN_MOE_DC_ROWS", 0);
+    unsigned rows = opt_u(O_MOE_DC_ROWS, 0);
     if (rows != 2 && rows != 4 && rows != 8) {
         rows = 8;
         while (rows > 2 && (unsigned long long)((out_dim + rows - 1) / rows) * n_tok < 4ull * kCUs) rows /= 2;
@@ -1585,20 +1698,20 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     // mostly empty tile pays its full matrix work -- and are ahead up to 1.6 entries per expert: 128 experts top-8
     // at 1 / 4 / 16 / 24 tokens 16 / 33 / 89 / 125 us against 48 / 61 / 126 / 141 for the pipeline below, at 28
     // tokens 141 against 143, at 32 tokens 160 against 145.  Same integer dots, fp32 sums in the decode kernels' order.
-    const bool chain = 5ull * ne <= 8ull * sh.n_expert && sh.expert_ff % 32 == 0 && env_u("REIN_MOE_CHAIN", 1) != 0;
+    const bool chain = 5ull * ne <= 8ull * sh.n_expert && sh.expert_ff % 32 == 0 && opt_u(O_MOE_CHAIN, 1) != 0;
     if (chain) {
         const unsigned ns_h = sh.hidden / 32, ns_f = sh.expert_ff / 32;
         // Where the one-wavefront router applies it shares a launch: for one or two tokens the gate / up launch
         // routes and quantizes its token itself (every workgroup again: 15.9 / 23.8 us against 17.3 / 25.4), beyond
         // that router and quantizer run as one small launch in front (16 tokens: 105 us against 111)
-        const bool wave = sh.n_expert <= 256 && sh.n_used <= 64 && sh.n_used <= sh.n_expert && env_u("REIN_TOPK_WAVE", 1) != 0;
+        const bool wave = sh.n_expert <= 256 && sh.n_used <= 64 && sh.n_used <= sh.n_expert && opt_u(O_TOPK_WAVE, 1) != 0;
         const bool routed = wave && sh.n_tok <= 2 && ns_h * 40u <= 48u * 1024u;
         if (routed) {
             void* xq_exp = base + w.xq_exp;
             const unsigned bpe = (unsigned)bpe_gu;
             void* a[] = {(void*)&gate_exps, (void*)&up_exps, (void*)&logits, (void*)&x, (void*)&ids, (void*)&weights, (void*)&xq_exp,
                          (void*)&sh.hidden, (void*)&sh.expert_ff, (void*)&bpe, (void*)&sh.n_expert, (void*)&sh.n_used};
-            const unsigned gu_rows = env_u("REIN_MOE_GU_ROWS", 0);
+            const unsigned gu_rows = opt_u(O_MOE_GU_ROWS, 0);
             const bool r4 = gu_rows == 4 || (gu_rows != 2 && (unsigned long long)(sh.expert_ff / 32) * sh.n_used * sh.n_tok >= 2ull * kCUs);
             if (int rc = launch(std::string("rein_moe_route_gate_up_swiglu_q8_") + fmt_tag(sh.gate_up_fmt) + (r4 ? "_r4" : ""), sh.expert_ff / 32,
                                 sh.n_used, sh.n_tok, r4 ? 512 : 1024, ns_h * 40u, s, a)) return rc;
@@ -1648,7 +1761,7 @@ int rein_moe_ffn(const rein_moe_shape* shp, const float* x, const float* logits,
     // gate and up projections, SwiGLU and the down projection's BlockQ8 rows in one launch;
     // REIN_MOE_FUSED=0 takes the two-output GEMM and swiglu_q8_f32 instead (the same bytes)
     const unsigned long long fused_grid = 8ull * (((ne + bn - 1) / bn + sh.n_expert + 7) / 8) * ((sh.expert_ff + 63) / 64);
-    if (sh.expert_ff % 32 == 0 && fused_grid <= 0x7FFFFFFFull && env_u("REIN_MOE_FUSED", 1) != 0) {
+    if (sh.expert_ff % 32 == 0 && fused_grid <= 0x7FFFFFFFull && opt_u(O_MOE_FUSED, 1) != 0) {
         if (int rc = rein_moe_grouped_swiglu_q8(sh.gate_up_fmt, gate_exps, up_exps, (unsigned)bpe_gu, eoff, toff, sh.n_expert,
                                                 base + w.g_in, base + w.xq_exp, sh.hidden, sh.expert_ff, ne, s)) return rc;
     } else {

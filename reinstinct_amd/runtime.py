@@ -98,6 +98,11 @@ def mmq_xq8_ws(fmt, w, xq, y, in_dim, out_dim, p_rows, workspace, workspace_byte
                               _s(stream)))
 
 
+def noalloc_prepare():
+    """rein_noalloc_prepare: place the fixed scratch array on the current device; outside any capture."""
+    check(lib.rein_noalloc_prepare())
+
+
 def mmq_xq8_noalloc(fmt, w, xq, y, in_dim, out_dim, p_rows, stream=None):
     """mmq_xq8_ws on the library's fixed 8 MiB device array: allocates nothing"""
     check(lib.rein_mmq_xq8_noalloc(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _s(stream)))

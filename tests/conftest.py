@@ -23,3 +23,26 @@ def _release_device_uploads(request):
         from reinstinct_amd import hip
         hip.synchronize()
         helpers.release_uploads()
+
+
+@pytest.fixture
+def options():
+    """Library options (rein_set_option) for one test: what the test sets goes back to its former
+    state afterwards."""
+    from reinstinct_amd import _lib
+
+    class Options:
+        def __init__(self):
+            self.before = {}
+
+        def set(self, name, value):
+            self.before.setdefault(name, _lib.get_option(name))
+            _lib.set_option(name, value)
+
+        def unset(self, name):
+            self.set(name, None)
+
+    o = Options()
+    yield o
+    for name, value in o.before.items():
+        _lib.set_option(name, value)

@@ -95,18 +95,20 @@ def rel_l2(a, b):
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
 
 
-def assert_close_f32(got, want, rel=1e-3, abs_=1e-4, what=""):
-    """fp32 output bar: |got-want| <= abs*max(1, rms(want)) + rel*|want| element-wise.
+def assert_close_f32(got, want, rel=1e-3, abs_=1e-4, what="", strict=False):
+    """fp32 output bar, element-wise.
 
-    The absolute part is stated for outputs of unit scale (weights ~N(0,0.02),
-    activations ~N(0,1) give rms(y) ~ 1).  The random-byte weights of the
-    reference's GPU tests (kernels.rs:3026-3061) give sums of terms of magnitude
-    ~40 and rms(y) in the hundreds; there the order of the fp32 additions alone
-    moves an element by 1e-4, so the absolute part scales with rms(want)."""
+    strict=True: |got-want| <= abs + rel*|want|, the bar as stated (1e-3 relative / 1e-4 absolute).  Every
+    test on the BASELINE recipe (weights ~N(0,0.02) quantized per format, activations ~N(0,1)) uses it.
+
+    strict=False: |got-want| <= abs*max(1, rms(want)) + rel*|want|.  Only for the random-byte weights of
+    the reference's GPU tests (kernels.rs:3026-3061): they give sums of terms of magnitude ~40 and rms(y)
+    in the hundreds, where the order of the fp32 additions alone moves an element by 1e-4, so the absolute
+    part scales with rms(want)."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
     err = np.abs(got - want)
-    scale = max(1.0, float(np.sqrt(np.mean(want * want)))) if want.size else 1.0
+    scale = 1.0 if strict or not want.size else max(1.0, float(np.sqrt(np.mean(want * want))))
     tol = abs_ * scale + rel * np.abs(want)
     bad = ~(err <= tol)
     if bad.any():

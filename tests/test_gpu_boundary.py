@@ -132,10 +132,10 @@ def test_reference_named_moe_prefill_chain(fmt, in_dim, bn):
     del d_slab, d_ids, d_x                                   # alive until the launches above have finished
 
 
-def test_library_grouped_launch_on_the_reference_named_kernel(monkeypatch):
+def test_library_grouped_launch_on_the_reference_named_kernel(options):
     # rein_moe_grouped_gemm falls back to the reference-named, grid-striding kernel when the
     # tile bound exceeds grid.y; the switch below forces that launch at a small size
-    monkeypatch.setenv("REIN_GROUPED_STRIDED", "1")
+    options.set("REIN_GROUPED_STRIDED", "1")
     fmt, in_dim, out_dim, n_expert, n_tok, n_used = rein.Q6_K, 768, 264, 5, 40, 2
     n = n_tok * n_used
     rng = np.random.default_rng(77)
@@ -161,10 +161,10 @@ def test_library_grouped_launch_on_the_reference_named_kernel(monkeypatch):
 
 # ---- the dot4 batched kernels at the row counts the library sends elsewhere ------------
 @pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS, rein.IQ3_S])
-def test_dot4_batched_kernels_3_to_8_rows(fmt, monkeypatch):
+def test_dot4_batched_kernels_3_to_8_rows(fmt, options):
     # rein_mv_<fmt>_r*_b4 / _b8: with both switches out of reach every row count stays on v_dot4
-    monkeypatch.setenv("REIN_SKINNY_FROM", "99")
-    monkeypatch.setenv("REIN_QUAD_FROM", "99")
+    options.set("REIN_SKINNY_FROM", "99")
+    options.set("REIN_QUAD_FROM", "99")
     in_dim, out_dim = 1024, 391
     raw = random_raw_weights(fmt, in_dim, out_dim, 40 + fmt)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
@@ -206,7 +206,7 @@ def test_config0_q4k_4096_by_4096():
     assert np.array_equal(xq, orc.quantize_q8(x))
     want = orc.matvec_q8(orc.Q4_K, packed, in_dim, out_dim, xq, 1)
     got = dy.to_host(np.float32)[None, :]
-    assert_close_f32(got, want, what="configs[0] Q4_K 4096x4096")
+    assert_close_f32(got, want, what="configs[0] Q4_K 4096x4096", strict=True)
     dots = orc.block_dots(orc.Q4_K, packed, in_dim, out_dim, xq, 1)
     assert np.array_equal(dd.to_host(np.int32).reshape(dots.shape), dots)
     f32 = orc.matvec_f32(x[0], orc.dequantize_to_f32(orc.Q4_K, raw, in_dim * out_dim).reshape(out_dim, in_dim))

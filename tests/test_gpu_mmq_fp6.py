@@ -12,7 +12,7 @@ import pytest
 
 import reinstinct_amd as rein
 from reinstinct_amd import hip, quant, runtime
-from reinstinct_amd._lib import ReinError, init
+from reinstinct_amd._lib import ReinError, init, set_option
 from oracle import orc
 from helpers import assert_close_f32, random_raw_weights
 
@@ -24,10 +24,10 @@ def gpu():
     init()
     hip.set_device(0)
     # the library keeps small GEMMs on the int8 launch; these tests are about the fp6 one
-    os.environ["REIN_MMQ6_FROM"] = "17"
+    set_option("REIN_MMQ6_FROM", "17")
     yield
     hip.synchronize()
-    os.environ.pop("REIN_MMQ6_FROM", None)
+    set_option("REIN_MMQ6_FROM", None)
 
 
 from helpers import dev  # noqa: E402  (uploads that stay alive until the test's last launch has finished)
@@ -101,12 +101,13 @@ def test_every_token_split_gives_the_same_bits():
     try:
         for n4, n2 in ((2, 1), (1, 3), (0, 5), (0, 0), (2, 0)):
             print(f"mmq6 split n4 {n4} n2 {n2}", flush=True)
-            os.environ["REIN_MMQ6_N4"], os.environ["REIN_MMQ6_N2"] = str(n4), str(n2)
+            set_option("REIN_MMQ6_N4", str(n4))
+            set_option("REIN_MMQ6_N2", str(n2))
             assert runtime.mmq_tile_plan_ws(rein.Q4_K, out_dim, p_rows) == (n4, n2)
             outs[(n4, n2)] = run_ws(dw, dq, in_dim, out_dim, p_rows).view(np.uint32)
     finally:
-        os.environ.pop("REIN_MMQ6_N4", None)
-        os.environ.pop("REIN_MMQ6_N2", None)
+        set_option("REIN_MMQ6_N4", None)
+        set_option("REIN_MMQ6_N2", None)
     first = next(iter(outs.values()))
     for k, v in outs.items():
         assert np.array_equal(v, first), f"split {k} differs"
@@ -123,9 +124,9 @@ def test_workspace_contract():
     # tiles of the int8 split-tail launch); up to 16 rows nothing uses one
     assert runtime.mmq_workspace_min_bytes(rein.Q6_K, in_dim, p_rows) == 0
     assert runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, 16) == 0
-    os.environ["REIN_MMQ6_FROM"] = "320"
+    set_option("REIN_MMQ6_FROM", "320")
     assert runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, 256) == 0 and runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, 320) > 0
-    os.environ["REIN_MMQ6_FROM"] = "17"
+    set_option("REIN_MMQ6_FROM", "17")
     ws = hip.DeviceBuf(need)
     dy = dev(np.zeros(p_rows * out_dim, np.float32))
     with pytest.raises(ReinError):                           # too small: refused, nothing launched
@@ -167,7 +168,7 @@ def test_two_launches_and_a_reused_workspace_agree():
 # contraction, their partial tiles summed in range order by whichever workgroup completes the tile
 def run_split_tail(dw, dq, in_dim, out_dim, p_rows, grid):
     ws_bytes = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, p_rows)
-    os.environ["REIN_MMQ6_SK_GRID"] = str(grid)
+    set_option("REIN_MMQ6_SK_GRID", str(grid))
     try:
         assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, p_rows, ws_bytes) == 2, "shape does not take the split-tail launch"
         ws = hip.DeviceBuf(ws_bytes)
@@ -178,7 +179,7 @@ def run_split_tail(dw, dq, in_dim, out_dim, p_rows, grid):
             hip.synchronize()
             outs.append(dy.to_host(np.float32).reshape(p_rows, out_dim).copy())
     finally:
-        os.environ.pop("REIN_MMQ6_SK_GRID", None)
+        set_option("REIN_MMQ6_SK_GRID", None)
     return outs
 
 
@@ -223,7 +224,7 @@ def test_split_tail_needs_the_full_workspace():
 def test_workspace_launches_at_the_benchmark_shape():
     # 5120 x 17408 at 512 tokens (one whole round + 32 tiles split eight ways) and 2048 tokens (mixed launch):
     # every element against the int8 launch, sampled tokens against the oracle; the default row threshold applies
-    os.environ.pop("REIN_MMQ6_FROM", None)
+    set_option("REIN_MMQ6_FROM", None)
     try:
         in_dim, out_dim = 5120, 17408
         w = (np.random.default_rng(31).standard_normal((512, in_dim)) * 0.02).astype(np.float32)
@@ -247,4 +248,4 @@ def test_workspace_launches_at_the_benchmark_shape():
             want = orc.matvec_q8(rein.Q4_K, packed, in_dim, out_dim, np.ascontiguousarray(xq[toks]).reshape(-1), len(toks))
             assert_close_f32(got[toks], want, what=f"workspace launch vs oracle, M {m}")
     finally:
-        os.environ["REIN_MMQ6_FROM"] = "17"
+        set_option("REIN_MMQ6_FROM", "17")

@@ -13,7 +13,7 @@ import pytest
 
 import reinstinct_amd as rein
 from reinstinct_amd import hip, quant, runtime
-from reinstinct_amd._lib import init
+from reinstinct_amd._lib import init, set_option
 from oracle import orc
 from helpers import assert_close_f32, dev, random_raw_weights
 
@@ -26,20 +26,20 @@ KNOBS = ("REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM
 def gpu():
     init()
     hip.set_device(0)
-    os.environ["REIN_MMQ6"] = "0"                    # Q4_K on the int8 tile too
+    set_option("REIN_MMQ6", "0")                    # Q4_K on the int8 tile too
     yield
     hip.synchronize()
     for k in KNOBS + ("REIN_MMQ6",):
-        os.environ.pop(k, None)
+        set_option(k, None)
 
 
 @pytest.fixture(autouse=True)
 def clean_knobs():
     for k in KNOBS:
-        os.environ.pop(k, None)
+        set_option(k, None)
     yield
     for k in KNOBS:
-        os.environ.pop(k, None)
+        set_option(k, None)
 
 
 def weights(fmt, in_dim, out_dim, seed):
@@ -83,10 +83,10 @@ CASES = [
 @pytest.mark.parametrize("p_rows,in_dim,out_dim,grid,split,tm", CASES)
 def test_split_tail_matches_oracle_and_repeats(fmt, p_rows, in_dim, out_dim, grid, split, tm):
     print(f"int8 split-tail fmt {fmt} P {p_rows} K {in_dim} N {out_dim} grid {grid} split {split} tm {tm}", flush=True)
-    if grid: os.environ["REIN_MMQ_SK_GRID"] = str(grid)
-    else: os.environ["REIN_MMQ_SK"] = "2"
-    if split: os.environ["REIN_MMQ_SK_SPLIT"] = str(split)
-    if tm: os.environ["REIN_MMQ_SK_TM"] = str(tm)
+    if grid: set_option("REIN_MMQ_SK_GRID", str(grid))
+    else: set_option("REIN_MMQ_SK", "2")
+    if split: set_option("REIN_MMQ_SK_SPLIT", str(split))
+    if tm: set_option("REIN_MMQ_SK_TM", str(tm))
     packed = weights(fmt, in_dim, out_dim, seed=p_rows + out_dim)
     x = np.random.default_rng(in_dim).standard_normal((p_rows, in_dim)).astype(np.float32)
     dw, dq = dev(packed), quantized(x)
@@ -100,8 +100,8 @@ def test_split_tail_matches_oracle_and_repeats(fmt, p_rows, in_dim, out_dim, gri
 def test_split_tail_with_a_ragged_last_chunk(fmt, in_dim):
     # contractions that are not whole 256-weight chunks: the last range ends inside a chunk
     p_rows, out_dim = 50, 200
-    os.environ["REIN_MMQ_SK_GRID"] = "8"
-    os.environ["REIN_MMQ_SK_SPLIT"] = "2"
+    set_option("REIN_MMQ_SK_GRID", "8")
+    set_option("REIN_MMQ_SK_SPLIT", "2")
     packed = weights(fmt, in_dim, out_dim, seed=in_dim)
     x = np.random.default_rng(3).standard_normal((p_rows, in_dim)).astype(np.float32)
     dw, dq = dev(packed), quantized(x)

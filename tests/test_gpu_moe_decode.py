@@ -200,13 +200,13 @@ def test_moe_decode_ffn_chain_config4_shapes():
 # ------------------------------------------------------------------ the two fused launches
 @pytest.mark.parametrize("rows", [0, 2, 4])
 @pytest.mark.parametrize("in_dim,out_dim,n_tok", [(2048, 768, 1), (2048, 96, 3), (256, 32, 2), (1024, 768, 3)])
-def test_gate_up_swiglu_q8_equals_the_two_launches(in_dim, out_dim, n_tok, rows, monkeypatch):
+def test_gate_up_swiglu_q8_equals_the_two_launches(in_dim, out_dim, n_tok, rows, options):
     # gate + up + SwiGLU + quantize in one launch: byte for byte what the fused matvec
     # followed by quantize_q8 writes, and that chain is what the oracle is compared with above;
     # with the library's choice of rows per wavefront (0; the last shape is large enough for four)
     # and with two and four forced
     if rows:
-        monkeypatch.setenv("REIN_MOE_GU_ROWS", str(rows))
+        options.set("REIN_MOE_GU_ROWS", str(rows))
     fmt, n_expert, n_used = rein.Q4_K, 10, 8
     rng = np.random.default_rng(in_dim * 7 + out_dim)
     gate, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=17)
@@ -236,11 +236,11 @@ def test_gate_up_swiglu_q8_equals_the_two_launches(in_dim, out_dim, n_tok, rows,
 @pytest.mark.parametrize("rows", [0, 4])
 @pytest.mark.parametrize("fmt", [rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.Q5_1])
 @pytest.mark.parametrize("in_dim,out_dim,n_tok", [(2048, 768, 1), (1024, 96, 3), (768, 768, 3)])
-def test_gate_up_swiglu_q8_other_formats(fmt, in_dim, out_dim, n_tok, rows, monkeypatch):
+def test_gate_up_swiglu_q8_other_formats(fmt, in_dim, out_dim, n_tok, rows, options):
     # the fused launch for the expert formats the reference has no fused kernel for: byte for byte what two
     # expert matvecs (gate, up) followed by swiglu_q8 write
     if rows:
-        monkeypatch.setenv("REIN_MOE_GU_ROWS", str(rows))
+        options.set("REIN_MOE_GU_ROWS", str(rows))
     n_expert, n_used = 10, 8
     rng = np.random.default_rng(in_dim * 3 + out_dim + fmt)
     gate, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=fmt * 10 + 1, pad16=True)
@@ -269,14 +269,14 @@ def test_gate_up_swiglu_q8_other_formats(fmt, in_dim, out_dim, n_tok, rows, monk
 @pytest.mark.parametrize("rows", [0, 2, 4, 8])
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("in_dim,out_dim,n_tok", [(768, 2048, 1), (768, 56, 2), (768, 43, 1), (2048, 64, 1), (1280, 37, 2)])
-def test_down_combine_equals_the_two_launches(fmt, in_dim, out_dim, n_tok, rows, monkeypatch):
+def test_down_combine_equals_the_two_launches(fmt, in_dim, out_dim, n_tok, rows, options):
     # down projection + weighted combine in one launch: bit for bit the two-launch result
     # (both team widths: up to 32 sub-blocks half-wavefronts, 2048 the full wavefront; the odd
     # row counts end on a workgroup that owns fewer rows than the others -- their slabs are padded to
     # the 16-byte stride the library asks for); with the library's own choice of rows per workgroup
     # (0) and with each of 2, 4 and 8 forced
     if rows:
-        monkeypatch.setenv("REIN_MOE_DC_ROWS", str(rows))
+        options.set("REIN_MOE_DC_ROWS", str(rows))
     n_expert, n_used = 12, 8
     rng = np.random.default_rng(in_dim * 5 + out_dim + fmt)
     slab, bpe = expert_slabs(fmt, in_dim, out_dim, n_expert, seed=fmt * 100 + 77, pad16=True)

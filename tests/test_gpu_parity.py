@@ -238,9 +238,9 @@ def test_mmq_parity(fmt, p_rows):
 @pytest.mark.parametrize("p_rows,in_dim,out_dim,ks", [
     (8, 2048, 77, 1), (8, 2048, 77, 3), (7, 2048, 77, 8), (16, 1280, 45, 2), (9, 1280, 45, 5),
     (3, 768, 130, 0), (13, 5120, 64, 16)])
-def test_skinny_mmq_parity(fmt, p_rows, in_dim, out_dim, ks, monkeypatch):
-    monkeypatch.setenv("REIN_SKINNY_KS", str(ks))
-    monkeypatch.setenv("REIN_SKINNY_FROM", "1")
+def test_skinny_mmq_parity(fmt, p_rows, in_dim, out_dim, ks, options):
+    options.set("REIN_SKINNY_KS", str(ks))
+    options.set("REIN_SKINNY_FROM", "1")
     raw, packed = make_weights(fmt, in_dim, out_dim, seed=1000 + fmt + p_rows)
     x = np.random.default_rng(p_rows + ks).standard_normal((p_rows, in_dim)).astype(np.float32)
     dq = gpu_quantize(x)
@@ -253,10 +253,10 @@ def test_skinny_mmq_parity(fmt, p_rows, in_dim, out_dim, ks, monkeypatch):
 
 @pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])       # the formats with 32-element blocks on disk
 @pytest.mark.parametrize("n_sub,p_rows", [(11, 8), (9, 5), (15, 16), (8, 2), (7, 8)])
-def test_skinny_mmq_ragged_chunks(fmt, n_sub, p_rows, monkeypatch):
+def test_skinny_mmq_ragged_chunks(fmt, n_sub, p_rows, options):
     # in_dim only a multiple of 32: the last chunk has 1..7 sub-blocks; 7 sub-blocks in
     # all (in_dim < 256) is below what the skinny kernel takes and falls back
-    monkeypatch.setenv("REIN_SKINNY_FROM", "1")
+    options.set("REIN_SKINNY_FROM", "1")
     in_dim, out_dim = 32 * n_sub, 50
     raw, packed = make_weights(fmt, in_dim, out_dim, seed=5 + n_sub)
     x = np.random.default_rng(8).standard_normal((p_rows, in_dim)).astype(np.float32)
@@ -288,17 +288,17 @@ def test_mmq_odd_sub_block_count(fmt):
 # tokens, including a ragged last tile of either size and a split that leaves no small tile.
 @pytest.mark.parametrize("fmt", ALL)
 @pytest.mark.parametrize("p_rows,n64", [(200, 1), (200, 3), (128, 2), (100, 0), (91, 1)])
-def test_mmq_mixed_tiles_parity(fmt, p_rows, n64, monkeypatch):
+def test_mmq_mixed_tiles_parity(fmt, p_rows, n64, options):
     in_dim, out_dim = 1024, 300
     raw, packed = make_weights(fmt, in_dim, out_dim, seed=0x3131 + fmt)
     x = Lcg(0x0BADCAFE + p_rows).acts(p_rows * in_dim).reshape(p_rows, in_dim)
     dq = gpu_quantize(x)
     dw = dev(packed)
-    monkeypatch.setenv("REIN_MMQ_TM", "32")
+    options.set("REIN_MMQ_TM", "32")
     d32 = dev(np.full(p_rows * out_dim, np.nan, np.float32))
     runtime.mmq_xq8(fmt, dw, dq, d32, in_dim, out_dim, p_rows)
-    monkeypatch.delenv("REIN_MMQ_TM")
-    monkeypatch.setenv("REIN_MMQ_N64", str(n64))
+    options.unset("REIN_MMQ_TM")
+    options.set("REIN_MMQ_N64", str(n64))
     dy = dev(np.full(p_rows * out_dim, np.nan, np.float32))
     runtime.mmq_xq8(fmt, dw, dq, dy, in_dim, out_dim, p_rows)
     hip.synchronize()
@@ -366,7 +366,7 @@ def test_moe_topk_parity():
     assert np.array_equal(d_ids.to_host(np.int32).reshape(ids.shape), ids)
 
 
-def test_moe_topk_wave_kernel_equals_the_workgroup_kernel(monkeypatch):
+def test_moe_topk_wave_kernel_equals_the_workgroup_kernel(options):
     # up to 256 experts the router runs one wavefront per token; it must give the ids and the weight bits of the
     # workgroup kernel (REIN_TOPK_WAVE=0): random logits, ties, NaN and -inf entries, every tail of the 4-token group
     rng = np.random.default_rng(77)
@@ -387,7 +387,7 @@ def test_moe_topk_wave_kernel_equals_the_workgroup_kernel(monkeypatch):
         d_logits = dev(logits)
         got = []
         for wave in ("1", "0"):
-            monkeypatch.setenv("REIN_TOPK_WAVE", wave)
+            options.set("REIN_TOPK_WAVE", wave)
             d_ids = dev(np.full(n_tok * n_used, -7, np.int32))
             d_w = dev(np.full(n_tok * n_used, np.nan, np.float32))
             runtime.moe_topk(d_logits, n_tok, n_expert, n_used, d_ids, d_w)
@@ -407,11 +407,11 @@ def gpu_sort(ids, n_expert, bn):
 
 
 @pytest.mark.parametrize("split", [False, True])
-def test_moe_sort_invariants(split, monkeypatch):
+def test_moe_sort_invariants(split, options):
     # both forms of the sort: one workgroup (small routing tables) and the reference's
     # zero / histogram / scan / scatter launches
     if split:
-        monkeypatch.setenv("REIN_MOE_SORT_SPLIT", "1")
+        options.set("REIN_MOE_SORT_SPLIT", "1")
     rng = np.random.default_rng(1)
     for n_tok, n_used, n_expert, bn in [(512, 8, 128, 32), (7, 2, 200, 16), (300, 4, 3, 32)]:
         ids = rng.integers(0, n_expert, (n_tok, n_used)).astype(np.int32)
@@ -592,7 +592,7 @@ def test_moe_ffn_end_to_end_small():
 @pytest.mark.parametrize("gu_fmt", [rein.Q4_K, rein.Q6_K, rein.Q8_0])
 @pytest.mark.parametrize("n_tok,n_expert,n_used,hidden", [(1, 16, 4, 512), (2, 128, 8, 512), (1, 200, 3, 768), (2, 9, 9, 1280),
                                                           (3, 64, 4, 512), (8, 32, 4, 768), (16, 64, 4, 512), (25, 64, 4, 512)])
-def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hidden, gu_fmt, monkeypatch):
+def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hidden, gu_fmt, options):
     # up to 1.6 routing entries per expert on average: rein_moe_ffn runs the two decode launches instead of
     # sort + grouped GEMMs; against the CPU chain, and against its own pipeline (REIN_MOE_CHAIN=0)
     ff = 256
@@ -608,7 +608,7 @@ def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hi
     dx, dl, dg, du, dd, ds = dev(x), dev(logits), dev(gate), dev(up), dev(down), dev(ones)
     outs = []
     for chain in ("1", "0"):
-        monkeypatch.setenv("REIN_MOE_CHAIN", chain)
+        options.set("REIN_MOE_CHAIN", chain)
         d_out = dev(np.full(n_tok * hidden, np.nan, np.float32))
         runtime.moe_ffn(sh, dx, dl, dg, du, dd, ds, ws, d_out)
         hip.synchronize()
@@ -627,9 +627,45 @@ def test_moe_ffn_few_tokens_takes_the_decode_kernels(n_tok, n_expert, n_used, hi
     assert rel_l2(outs[0], outs[1]) < 2e-3
     # the router and the quantizer share a launch there (one and two tokens: the gate / up launch itself, more: one
     # small launch in front); as separate launches (REIN_TOPK_WAVE=0) the bits are the same
-    monkeypatch.setenv("REIN_MOE_CHAIN", "1")
-    monkeypatch.setenv("REIN_TOPK_WAVE", "0")
+    options.set("REIN_MOE_CHAIN", "1")
+    options.set("REIN_TOPK_WAVE", "0")
     d_out = dev(np.full(n_tok * hidden, np.nan, np.float32))
     runtime.moe_ffn(sh, dx, dl, dg, du, dd, ds, ws, d_out)
     hip.synchronize()
     assert np.array_equal(d_out.to_host(np.uint32).reshape(n_tok, hidden), outs[0].view(np.uint32))
+
+
+@pytest.mark.parametrize("n_expert,n_used,n_tok", [(128, 8, 25), (128, 8, 26), (64, 4, 25), (64, 4, 26), (128, 8, 1), (128, 8, 2),
+                                                   (128, 8, 3)])
+def test_moe_ffn_default_choice_either_side_of_the_few_token_threshold(n_expert, n_used, n_tok):
+    # with no option set rein_moe_ffn runs the decode launches while 5 n_tok n_used <= 8 n_expert (25 tokens at 128
+    # experts top-8 and at 64 top-4) and the sorted pipeline from the next token on; one and two tokens route inside
+    # the gate / up launch, three and more in a small launch in front.  The fp32 additions of a token's row differ
+    # between the two forms (expert order against slot order), so the sum's bits depend on how many tokens share
+    # the call: each side of the edge is held against the oracle at the same bar.
+    hidden, ff = 512, 256
+    chain = 5 * n_tok * n_used <= 8 * n_expert
+    assert chain == (n_tok <= 25)
+    rng = np.random.default_rng(1000 * n_expert + n_tok)
+    x = rng.standard_normal((n_tok, hidden)).astype(np.float32)
+    logits = rng.standard_normal((n_tok, n_expert)).astype(np.float32)
+    gate = np.concatenate([make_weights(rein.Q4_K, hidden, ff, 300 + e, True)[1] for e in range(n_expert)])
+    up = np.concatenate([make_weights(rein.Q4_K, hidden, ff, 400 + e, True)[1] for e in range(n_expert)])
+    down = np.concatenate([make_weights(rein.Q6_K, ff, hidden, 500 + e, True)[1] for e in range(n_expert)])
+    scale = (1.0 + 0.25 * rng.standard_normal(n_expert)).astype(np.float32)
+    sh = runtime.moe_shape(n_tok, hidden, n_expert, n_used, ff, rein.Q4_K, rein.Q6_K)
+    ws = hip.DeviceBuf(runtime.moe_workspace_bytes(sh))
+    d_out = dev(np.full(n_tok * hidden, np.nan, np.float32))
+    runtime.moe_ffn(sh, dev(x), dev(logits), dev(gate), dev(up), dev(down), dev(scale), ws, d_out)
+    hip.synchronize()
+    got = d_out.to_host(np.float32).reshape(n_tok, hidden)
+    ids, wts = orc.moe_topk(logits, n_used)
+    perm, eoff, _ = orc.moe_sort(ids, n_expert, 32)
+    gin = orc.moe_gather_xq(orc.quantize_q8(x), perm, hidden // 32, n_used)
+    bpe_gu, bpe_dn = orc.repacked_len(orc.Q4_K, hidden, ff), orc.repacked_len(orc.Q6_K, ff, hidden)
+    eg = orc.grouped_gemm(orc.Q4_K, gate, bpe_gu, eoff, gin, hidden, ff)
+    eu = orc.grouped_gemm(orc.Q4_K, up, bpe_gu, eoff, gin, hidden, ff)
+    gout = orc.grouped_gemm(orc.Q6_K, down, bpe_dn, eoff, orc.quantize_q8(orc.swiglu_mul(eg, eu)), ff, hidden)
+    want = orc.moe_combine(orc.moe_scatter_rows(gout, perm, hidden).reshape(n_tok, n_used, hidden), ids, wts, scale)
+    assert rel_l2(got, want) < 2e-3
+    assert_close_f32(got, want, rel=2e-2, abs_=2e-3, what=f"moe_ffn default choice, {n_tok} tokens x {n_expert} experts")

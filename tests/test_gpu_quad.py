@@ -40,8 +40,8 @@ def run(fmt, packed, xq, in_dim, out_dim, n_rows):
 
 @pytest.mark.parametrize("fmt", DENSE)
 @pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (256, 64), (5120, 130), (4096, 33)])
-def test_quad_matvec_parity(fmt, in_dim, out_dim, monkeypatch):
-    monkeypatch.setenv("REIN_QUAD_FROM", "1")
+def test_quad_matvec_parity(fmt, in_dim, out_dim, options):
+    options.set("REIN_QUAD_FROM", "1")
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + in_dim)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     for n_rows in range(1, 9):
@@ -54,8 +54,8 @@ def test_quad_matvec_parity(fmt, in_dim, out_dim, monkeypatch):
 
 @pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])       # 32-weight blocks: any multiple of 32
 @pytest.mark.parametrize("in_dim", [32, 96, 352, 544, 1056])
-def test_quad_matvec_ragged_contraction(fmt, in_dim, monkeypatch):
-    monkeypatch.setenv("REIN_QUAD_FROM", "1")
+def test_quad_matvec_ragged_contraction(fmt, in_dim, options):
+    options.set("REIN_QUAD_FROM", "1")
     out_dim = 37
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=in_dim)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
@@ -82,7 +82,7 @@ def bits(a):
 
 
 @pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q8_0, rein.Q4_0])
-def test_mid_width_matrices_take_these_kernels_at_3_and_4_rows(fmt, monkeypatch):
+def test_mid_width_matrices_take_these_kernels_at_3_and_4_rows(fmt, options):
     # 8192..20480 output rows: the library's own choice for the formats that otherwise run the skinny MMQ;
     # the same bits as with the kernels forced, and the oracle's values
     in_dim, out_dim = 2304, 8200
@@ -93,14 +93,14 @@ def test_mid_width_matrices_take_these_kernels_at_3_and_4_rows(fmt, monkeypatch)
         xq = orc.quantize_q8(np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32))
         got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
         assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what=f"fmt {fmt} rows {n_rows}")
-        monkeypatch.setenv("REIN_QUAD_FROM", "1")
+        options.set("REIN_QUAD_FROM", "1")
         forced = run(fmt, packed, xq, in_dim, out_dim, n_rows)
-        monkeypatch.delenv("REIN_QUAD_FROM")
+        options.unset("REIN_QUAD_FROM")
         assert np.array_equal(bits(got), bits(forced)), "the default launch is not the 4x4x4 kernel"
 
 
 @pytest.mark.parametrize("fmt", DENSE)
-def test_small_matrices_stay_on_dot4(fmt, monkeypatch):
+def test_small_matrices_stay_on_dot4(fmt, options):
     # up to 2^24 weights at 3-4 rows and 6 * 2^20 at 5-8 the library keeps the dot4 kernels: the same bits as
     # with both matrix-core families switched off, and the oracle's values
     in_dim, out_dim = 2048, 1536
@@ -111,9 +111,9 @@ def test_small_matrices_stay_on_dot4(fmt, monkeypatch):
         xq = orc.quantize_q8(np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32))
         got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
         assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what=f"fmt {fmt} rows {n_rows}")
-        monkeypatch.setenv("REIN_QUAD_FROM", "99")
-        monkeypatch.setenv("REIN_SKINNY_FROM", "99")
+        options.set("REIN_QUAD_FROM", "99")
+        options.set("REIN_SKINNY_FROM", "99")
         forced = run(fmt, packed, xq, in_dim, out_dim, n_rows)
-        monkeypatch.delenv("REIN_QUAD_FROM")
-        monkeypatch.delenv("REIN_SKINNY_FROM")
+        options.unset("REIN_QUAD_FROM")
+        options.unset("REIN_SKINNY_FROM")
         assert np.array_equal(bits(got), bits(forced)), "the default launch is not a dot4 kernel"

@@ -107,7 +107,7 @@ def gaussian_slab(fmt, in_dim, out_dim, n_expert, seed):
     return np.concatenate(out)
 
 
-def test_moe_ffn_on_random_shapes(monkeypatch):
+def test_moe_ffn_on_random_shapes(options):
     rng = np.random.default_rng(4)
     for case in range(40):
         gu = EXPERT[rng.integers(4)] if rng.random() < 0.4 else rein.Q4_K
@@ -117,8 +117,8 @@ def test_moe_ffn_on_random_shapes(monkeypatch):
         n_used = int(rng.integers(1, min(8, n_expert) + 1))
         n_tok = int(rng.choice([1, 2, int(rng.integers(3, 17)), int(rng.integers(17, 80)), int(rng.integers(80, 260))]))
         fused, strided = str(int(rng.integers(2))), str(int(rng.random() < 0.2))
-        monkeypatch.setenv("REIN_MOE_FUSED", fused)
-        monkeypatch.setenv("REIN_GROUPED_STRIDED", strided)
+        options.set("REIN_MOE_FUSED", fused)
+        options.set("REIN_GROUPED_STRIDED", strided)
         print(f"moe case {case}: gate/up {gu} down {dn} hidden {hidden} ff {ff} experts {n_expert} top-{n_used} tokens {n_tok} "
               f"fused {fused} strided {strided}", flush=True)
         x = rng.standard_normal((n_tok, hidden)).astype(np.float32)

@@ -168,3 +168,42 @@ def test_moe_workspace_layout():
         + ne * 2048 * 4
     assert need <= n <= need + 14 * 256
     assert runtime.moe_gemm_bn() == 32
+
+
+def test_options_table():
+    # rein_set_option / rein_get_option / rein_reset_options: the library's launch switches live in one table
+    # that the environment seeds once; names are enumerable, unknown names and malformed values are refused
+    from reinstinct_amd import _lib
+    lib = _lib.load()
+    names = [lib.rein_option_name(i).decode() for i in range(lib.rein_option_count())]
+    assert len(names) == len(set(names)) >= 20 and all(n.startswith("REIN_") for n in names)
+    assert lib.rein_option_name(-1) is None and lib.rein_option_name(len(names)) is None
+    _lib.reset_options()
+    for n in names:
+        assert _lib.get_option(n) is None
+    _lib.set_option("REIN_MMQ6_FROM", 17)
+    assert _lib.get_option("REIN_MMQ6_FROM") == 17
+    # the table, not the environment, is what the entry points read: a later change of the environment is not seen
+    import os
+    os.environ["REIN_MMQ6_FROM"] = "999"
+    try:
+        assert _lib.get_option("REIN_MMQ6_FROM") == 17
+        # 17 rows now have an fp6 workspace form; back to the default threshold they have none
+        assert lib.rein_mmq_workspace_min_bytes(12, 512, 20) > 0
+        _lib.set_option("REIN_MMQ6_FROM", None)
+        assert _lib.get_option("REIN_MMQ6_FROM") is None
+        assert lib.rein_mmq_workspace_min_bytes(12, 512, 20) == 0
+    finally:
+        os.environ.pop("REIN_MMQ6_FROM", None)
+    _lib.set_option("REIN_MV_ROWS", "4")
+    _lib.reset_options()
+    assert _lib.get_option("REIN_MV_ROWS") is None
+    for bad_name in ("REIN_NO_SUCH_OPTION", ""):
+        with pytest.raises(_lib.ReinError) as err:
+            _lib.set_option(bad_name, 1)
+        assert err.value.code == -8
+    for bad_value in ("-1", "abc", "12x", "4294967296"):
+        with pytest.raises(_lib.ReinError) as err:
+            _lib.set_option("REIN_MV_ROWS", bad_value)
+        assert err.value.code == -3
+    assert _lib.get_option("REIN_MV_ROWS") is None

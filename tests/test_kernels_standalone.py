@@ -1,7 +1,15 @@
 """Every kernel source compiles on its own with the command line the reference's kernel
 cache uses (src/runtime/mod.rs:195-245: `hipcc --genco --offload-arch=<arch> -O3 -std=c++17
--I<dir> <file> -o <hsaco>`), so a host that builds kernels one file at a time at run time can
-point its kernel directory here.  Compile only (hipcc cross-compiles without a GPU)."""
+-I<dir> <file> -o <hsaco>`): the sources carry no dependence on a build system, and each file
+exports the reference's symbol names.
+
+This is a COMPILE-ONLY check (hipcc cross-compiles without a GPU); nothing built here is ever run.
+The supported build -- the one every GPU test, the smoke and the benchmark load -- is the single
+code object the Makefile in reinstinct_amd/csrc produces, with
+`-Xclang -target-feature -Xclang -packed-fp32-ops -fhip-fp32-correctly-rounded-divide-sqrt`:
+the first keeps the compiler from forming packed fp32 instructions, the second is part of the
+bit-level definition of quantize_q8.  A host that compiles these files itself at run time must
+pass the same flags; a code object built with the bare command above is untested."""
 import concurrent.futures
 import glob
 import os

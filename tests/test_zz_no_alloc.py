@@ -52,6 +52,54 @@ def test_no_alloc_entry_matches_the_workspace_entry_twice_in_a_row():
     assert run_pair(rein.Q4_K, 512, *big, seed=5) > 0
 
 
+def test_no_alloc_entry_under_stream_capture_and_without_touching_device_memory():
+    # rein_noalloc_prepare places the array outside any capture; after it a call may be recorded into a graph,
+    # the replays give the bits of the eager call, and the free device memory the runtime reports does not move
+    init()
+    hip.set_device(0)
+    runtime.noalloc_prepare()
+    fmt, p_rows, in_dim, out_dim = rein.Q4_K, 512, 2304, 14336
+    assert runtime.mmq_workspace_min_bytes(fmt, in_dim, p_rows) > 0
+    raw = random_raw_weights(fmt, in_dim, out_dim, 9)
+    dw = dev(quant.repack_for_matvec(fmt, raw, in_dim, out_dim))
+    x = np.random.default_rng(9).standard_normal((p_rows, in_dim)).astype(np.float32)
+    d_x, dq = dev(x), hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
+    runtime.quantize_q8(d_x, dq, in_dim, p_rows)
+    d_eager = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    d_graph = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    stream = hip.Stream()
+    runtime.mmq_xq8_noalloc(fmt, dw, dq, d_eager, in_dim, out_dim, p_rows, stream)      # warm-up, and the eager result
+    stream.synchronize()
+    hip.synchronize()
+    eager = d_eager.to_host(np.uint32)
+    free_before = hip.mem_info()[0]
+    print("no-alloc entry: capture", flush=True)
+    stream.begin_capture()
+    runtime.mmq_xq8_noalloc(fmt, dw, dq, d_graph, in_dim, out_dim, p_rows, stream)
+    graph = stream.end_capture()
+    exe = graph.instantiate()
+    zero = np.zeros(p_rows * out_dim, np.float32)
+    for replay in range(3):
+        d_graph.copy_from_host(zero)
+        hip.synchronize()
+        exe.launch(stream)
+        stream.synchronize()
+        assert np.array_equal(d_graph.to_host(np.uint32), eager), f"replay {replay} differs from the eager call"
+        # eager work between the replays
+        runtime.mmq_xq8_noalloc(fmt, dw, dq, d_eager, in_dim, out_dim, p_rows, stream)
+        stream.synchronize()
+        assert np.array_equal(d_eager.to_host(np.uint32), eager)
+    del exe, graph
+    hip.synchronize()
+    free_mid = hip.mem_info()[0]
+    for _ in range(8):
+        runtime.mmq_xq8_noalloc(fmt, dw, dq, d_eager, in_dim, out_dim, p_rows, stream)
+    stream.synchronize()
+    free_after = hip.mem_info()[0]
+    assert free_after == free_mid, f"free device memory moved across eight calls: {free_mid} -> {free_after}"
+    assert free_mid >= free_before - (4 << 20), "the graph objects aside, nothing may have been allocated"
+
+
 def test_no_alloc_entry_refuses_what_the_fixed_array_cannot_hold():
     init()
     hip.set_device(0)
