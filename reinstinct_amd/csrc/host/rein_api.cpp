@@ -232,6 +232,10 @@ int launch_skinny(int fmt, const void* w, const void* xq, float* y, unsigned in_
         }
         if (cost < best) { best = cost; ks = k; }
     }
+    // Measured correction for the two-wavefronts-per-SIMD kernels (Q5_K, Q6_K) at 5-8 rows against many row
+    // tiles: four wavefronts per tile, i.e. two tiles per CU at a time, beat the model's two (Q5_K 5120 -> 34816
+    // at 8 rows: 46.6 -> 41.0 us, Q6_K 58.8 -> 52.8; 2 / 4 / 8 wavefronts: 46.6 / 41.0 / 56.5)
+    if (occ == 2 && nv == 4 && tiles >= 1024 && ks < 4 && ks_max >= 4) ks = 4;
     const unsigned forced = opt_u(O_SKINNY_KS, 0);
     if (forced >= 1 && forced <= ks_max) ks = forced;
     const std::string name = std::string("rein_mmqs_") + fmt_tag(fmt) + "_v" + std::to_string(nv);
