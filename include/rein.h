@@ -516,7 +516,12 @@ size_t rein_moe_workspace_bytes(const rein_moe_shape *shape);
  * (5 n_tok n_used <= 8 n_expert) the same result comes from the decode
  * kernels instead (top-k -> quantize -> rein_moe_gate_up_swiglu_q8 -> rein_moe_down_combine, the
  * launches of qwen35.rs:3071-3167 fused in pairs): no sort, one expert read per entry; for one
- * and two tokens the gate / up launch also routes and quantizes, so the FFN is two launches. */
+ * and two tokens the gate / up launch also routes and quantizes, so the FFN is two launches.
+ * The two forms add a token's eight expert rows, and the terms inside each row, in different
+ * orders (slot order in the decode form, expert-sorted tiles in the pipeline): the fp32 bits
+ * of a token's output row therefore depend on how many tokens share the call (25 against 26
+ * at 128 experts top-8), within the path's 1e-3 / 1e-4 tolerance of either order.  The option
+ * REIN_MOE_CHAIN = 0 keeps every call on the pipeline. */
 int rein_moe_ffn(const rein_moe_shape *shape, const float *x, const float *logits,
                  const void *gate_exps, const void *up_exps, const void *down_exps,
                  const float *down_exps_s, void *workspace, float *out, rein_stream_t s);
