@@ -745,8 +745,8 @@ def main():
                       "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                    "frac": round(tops / INT8_PEAK_TOPS, 4),
                                    "kernel": mmq_kernel_name(rein.Q4_K, 5120, 17408, 512),
-                                   "counters_recorded": {"mfma_busy_frac_of_simd_cycles": 0.337, "valu_issue_frac": 0.487,
-                                                         "hbm_fetch_bytes": 148.7e6, "input_bytes": 57.1e6,
+                                   "counters_recorded": {"mfma_busy_frac_of_simd_cycles": 0.331, "valu_issue_frac": 0.479,
+                                                         "hbm_fetch_bytes": 148.6e6, "input_bytes": 57.1e6,
                                                          "source": "rocprofv3 --pmc runs of this file, profiles/rein_mmq6_q4k_sk_pp512.txt; "
                                                                    "not read in this run"}}}
         del mm
