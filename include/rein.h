@@ -350,11 +350,13 @@ int rein_mmq_xq8_ws(int fmt, const void *w, const void *xq, float *y, unsigned i
 /* rein_mmq_xq8_ws without the workspace argument and without any allocation, for callers that
  * cannot allocate device memory: code under graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  It has no counterpart in the reference.  The workspace is a fixed array of
- * 8 MiB in device memory that every GPU the process uses holds until the process ends
- * (librein_scratch.so, loaded from the directory of librein.so on the first call).  Shapes whose
- * rein_mmq_workspace_min_bytes exceeds 8 MiB are refused with REIN_E_TOO_LARGE (at in_dim 5120
- * that is above 768 rows); shapes that need no workspace run rein_mmq_xq8.  All calls on one
- * GPU share the array: calls that overlap on one GPU (two streams, two threads) race.
+ * 48 MiB in device memory that every GPU the process uses holds until the process ends
+ * (librein_scratch.so, loaded from the directory of librein.so on the first call); the call
+ * launches what rein_mmq_xq8_ws launches for a workspace of that size, the split-tail forms
+ * included (rein_mmq_form_ws tells which).  Shapes whose rein_mmq_workspace_min_bytes exceeds
+ * 48 MiB are refused with REIN_E_TOO_LARGE (at in_dim 5120 that is above 4608 rows; the
+ * split-tail form of the fp6 launch fits to 1536 rows).  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two threads) race.
  * "Allocates nothing" holds once the array's address is known on the current device: the first
  * look loads librein_scratch.so and asks the runtime for the symbol's address, which makes the
  * runtime place (and zero) the array on that device.  That step must not fall into a stream

@@ -1169,11 +1169,19 @@ int rein_noalloc_prepare(void)
     size_t bytes = 0;
     if (int rc = static_scratch(&ptr, &bytes)) return rc;
     // the kernels the entry point can launch: their handles are looked up now, not under a capture
-    static const char* const names[] = {"rein_mmq6_prep", "rein_mmq6_q4k_mix", "rein_mmq_q4k_t32", "rein_mmq_q4k_t64", "rein_mmq_q4k_mix"};
+    static const char* const names[] = {"rein_mmq6_prep", "rein_mmq6_q4k_mix", "rein_mmq6_q4k_sk", "rein_mmq6_tail_sum",
+                                        "rein_mmq_tail_sum_t32", "rein_mmq_tail_sum_t64"};
     for (const char* n : names) {
         hipFunction_t f;
         if (int rc = get_fn(n, &f)) return rc;
     }
+    static const int fmts[] = {REIN_TYPE_Q4_0, REIN_TYPE_Q4_K, REIN_TYPE_Q5_K, REIN_TYPE_Q6_K, REIN_TYPE_Q8_0, REIN_TYPE_IQ4_XS};
+    static const char* const forms[] = {"_t32", "_t64", "_mix", "_sk", "_sk32"};
+    for (int fmt : fmts)
+        for (const char* form : forms) {
+            hipFunction_t f;
+            if (int rc = get_fn(std::string("rein_mmq_") + fmt_tag(fmt) + form, &f)) return rc;
+        }
     return 0;
 }
 
@@ -1181,9 +1189,9 @@ int rein_mmq_xq8_noalloc(int fmt, const void* w, const void* xq, float* y, unsig
                          unsigned p_rows, rein_stream_t s)
 {
     if (int rc = need_runtime()) return rc;
-    // the smallest workspace form: the activation image alone (the 8 MiB array has no room for partial tiles)
+    // rein_mmq_xq8_ws on the fixed array: whichever launch that entry point picks for a workspace of the array's
+    // size (split-tail forms included where their partial tiles fit behind the activation image)
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
-    if (need == 0) return rein_mmq_xq8(fmt, w, xq, y, in_dim, out_dim, p_rows, s);      // that launch has no scratch
     void* ptr = nullptr;
     size_t bytes = 0;
     if (int rc = static_scratch(&ptr, &bytes)) return rc;

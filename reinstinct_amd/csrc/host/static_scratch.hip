@@ -13,7 +13,8 @@
 
 #include <mutex>
 
-#define REIN_STATIC_SCRATCH_BYTES (8u << 20)       // 8 MiB per GPU
+#define REIN_STATIC_SCRATCH_BYTES (48u << 20)      // 48 MiB per GPU: the activation image and the partial tiles of a
+                                                   // split-tail launch at 512 tokens x 5120, with room to 1500 tokens
 #define REIN_MAX_DEVICES 64
 
 static __device__ __align__(256) unsigned char scratch[REIN_STATIC_SCRATCH_BYTES];

@@ -104,7 +104,7 @@ def noalloc_prepare():
 
 
 def mmq_xq8_noalloc(fmt, w, xq, y, in_dim, out_dim, p_rows, stream=None):
-    """mmq_xq8_ws on the library's fixed 8 MiB device array: allocates nothing"""
+    """mmq_xq8_ws on the library's fixed 48 MiB device array: allocates nothing"""
     check(lib.rein_mmq_xq8_noalloc(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, p_rows, _s(stream)))
 
 

@@ -1,7 +1,7 @@
 """The entry point that allocates nothing (rein_mmq_xq8_noalloc) against the entry point it is a
-variant of (rein_mmq_xq8_ws with a caller's workspace of the size the fixed array is used at: the
-activation image, rein_mmq_workspace_min_bytes): the same bits, on two calls in a row, the second
-with a smaller input; shapes beyond the fixed array are refused."""
+variant of (rein_mmq_xq8_ws with a caller's workspace of the fixed array's size, 48 MiB): the same
+bits, on two calls in a row, the second with a smaller input, through every launch form a workspace
+of that size selects; shapes beyond the fixed array are refused."""
 import numpy as np
 import pytest
 
@@ -12,6 +12,8 @@ from helpers import dev, random_raw_weights
 
 pytestmark = pytest.mark.gpu
 
+SCRATCH_BYTES = 48 << 20        # the stated size of the library's fixed array
+
 
 def run_pair(fmt, p_rows, in_dim, out_dim, seed):
     print(f"no-alloc entry: fmt {fmt} P {p_rows} K {in_dim} N {out_dim}", flush=True)
@@ -20,46 +22,50 @@ def run_pair(fmt, p_rows, in_dim, out_dim, seed):
     x = np.random.default_rng(seed).standard_normal((p_rows, in_dim)).astype(np.float32)
     d_x, dq = dev(x), hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
     runtime.quantize_q8(d_x, dq, in_dim, p_rows)
-    need = runtime.mmq_workspace_min_bytes(fmt, in_dim, p_rows)
-    ws = hip.DeviceBuf(max(need, 16))
+    ws = hip.DeviceBuf(SCRATCH_BYTES)
     d_ref = dev(np.full(p_rows * out_dim, np.nan, np.float32))
-    runtime.mmq_xq8_ws(fmt, dw, dq, d_ref, in_dim, out_dim, p_rows, ws if need else None, need)
+    runtime.mmq_xq8_ws(fmt, dw, dq, d_ref, in_dim, out_dim, p_rows, ws, SCRATCH_BYTES)
     d_got = dev(np.full(p_rows * out_dim, np.nan, np.float32))
     runtime.mmq_xq8_noalloc(fmt, dw, dq, d_got, in_dim, out_dim, p_rows)
     hip.synchronize()
     ref, got = d_ref.to_host(np.uint32), d_got.to_host(np.uint32)
     assert not np.isnan(d_got.to_host(np.float32)).any()
     assert np.array_equal(got, ref), f"no-alloc entry differs at P {p_rows} K {in_dim} N {out_dim}"
-    return need
+    return runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, SCRATCH_BYTES)
 
 
 def test_no_alloc_entry_matches_the_workspace_entry_twice_in_a_row():
     init()
     hip.set_device(0)
-    # Q4_K from 320 rows up, three 32-token tiles per resident workgroup (here 112 row blocks x 16 and x 14 token
-    # tiles) and 2 M N K of 2.8e10 and more runs out of the fixed array; the second call is smaller than the first
+    # launch forms of rein_mmq_form_ws: 1 the mixed fp6 launch (activation image only), 2 the fp6 split-tail launch
+    # (image + one partial tile per workgroup), 3 the int8 split-tail launch, 0 the plain launch without scratch.
+    # The second call of each pair is smaller than the first and finds the first one's contents in the array.
     big = (2304, 14336)
-    assert run_pair(rein.Q4_K, 512, *big, seed=1) > 0
-    assert runtime.mmq_form_ws(rein.Q4_K, *big, 512, runtime.mmq_workspace_min_bytes(rein.Q4_K, big[0], 512)) == 1
-    assert run_pair(rein.Q4_K, 448, *big, seed=2) > 0
-    assert runtime.mmq_form_ws(rein.Q4_K, *big, 448, runtime.mmq_workspace_min_bytes(rein.Q4_K, big[0], 448)) == 1
-    # launches that use no scratch go straight through: other formats, few rows, GEMMs too small for the fp6 launch
+    assert run_pair(rein.Q4_K, 512, *big, seed=1) == 1
+    assert run_pair(rein.Q4_K, 448, *big, seed=2) == 1
+    tail = (5120, 6144)
+    assert run_pair(rein.Q4_K, 512, *tail, seed=7) == 2
+    assert run_pair(rein.Q4_K, 480, 4096, 8192, seed=8) == 2
+    assert run_pair(rein.Q6_K, 384, 4096, 12288, seed=9) == 3
+    assert run_pair(rein.Q4_K, 448, 2048, 264, seed=6) == 3
     assert run_pair(rein.Q6_K, 64, 512, 136, seed=3) == 0
     assert run_pair(rein.Q4_K, 40, 512, 136, seed=4) == 0
-    assert run_pair(rein.Q4_K, 448, 2048, 264, seed=6) > 0
-    assert runtime.mmq_form_ws(rein.Q4_K, 2048, 264, 448, runtime.mmq_workspace_min_bytes(rein.Q4_K, 2048, 448)) == 0
-    # and once more the larger shape, after the smaller ones
-    assert run_pair(rein.Q4_K, 512, *big, seed=5) > 0
+    # and once more the first shapes, after the others
+    assert run_pair(rein.Q4_K, 512, *tail, seed=10) == 2
+    assert run_pair(rein.Q4_K, 512, *big, seed=5) == 1
 
 
-def test_no_alloc_entry_under_stream_capture_and_without_touching_device_memory():
+@pytest.mark.parametrize("shape, form", [((512, 2304, 14336), 1), ((512, 5120, 6144), 2), ((448, 2048, 264), 3)])
+def test_no_alloc_entry_under_stream_capture_and_without_touching_device_memory(shape, form):
     # rein_noalloc_prepare places the array outside any capture; after it a call may be recorded into a graph,
     # the replays give the bits of the eager call, and the free device memory the runtime reports does not move
     init()
     hip.set_device(0)
     runtime.noalloc_prepare()
-    fmt, p_rows, in_dim, out_dim = rein.Q4_K, 512, 2304, 14336
+    fmt, (p_rows, in_dim, out_dim) = rein.Q4_K, shape
     assert runtime.mmq_workspace_min_bytes(fmt, in_dim, p_rows) > 0
+    assert runtime.mmq_form_ws(fmt, in_dim, out_dim, p_rows, SCRATCH_BYTES) == form
+    print(f"no-alloc entry under capture: P {p_rows} K {in_dim} N {out_dim} form {form}", flush=True)
     raw = random_raw_weights(fmt, in_dim, out_dim, 9)
     dw = dev(quant.repack_for_matvec(fmt, raw, in_dim, out_dim))
     x = np.random.default_rng(9).standard_normal((p_rows, in_dim)).astype(np.float32)
@@ -103,8 +109,8 @@ def test_no_alloc_entry_under_stream_capture_and_without_touching_device_memory(
 def test_no_alloc_entry_refuses_what_the_fixed_array_cannot_hold():
     init()
     hip.set_device(0)
-    p_rows, in_dim, out_dim = 1024, 5120, 128
-    assert runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, p_rows) > (8 << 20)
+    p_rows, in_dim, out_dim = 4864, 5120, 128
+    assert runtime.mmq_workspace_min_bytes(rein.Q4_K, in_dim, p_rows) > SCRATCH_BYTES
     raw = random_raw_weights(rein.Q4_K, in_dim, out_dim, 6)
     dw = dev(quant.repack_for_matvec(rein.Q4_K, raw, in_dim, out_dim))
     dq = hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
