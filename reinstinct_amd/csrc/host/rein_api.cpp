@@ -139,8 +139,8 @@ int check_ptr(const char* who, const void* p, size_t align, const char* what)
 // rein_set_option changes an entry, so the launch an entry point chooses depends on its arguments
 // and on this table alone.  Entries are single atomic words: setting one while another thread
 // launches is safe, the launch sees the old or the new value.
-enum Opt : int { O_MV_ROWS, O_MV_WPB, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
-const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
+enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
+const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
 constexpr uint64_t kOptSet = 1ull << 63;
 std::atomic<uint64_t> g_opts[O_COUNT];          // zero = unset
 std::once_flag g_opts_env_once;
@@ -306,6 +306,91 @@ bool small_for_matrix_cores(int fmt, unsigned in_dim, unsigned out_dim, unsigned
     return out_dim <= 2048 || (!quad_family && weights <= (1ull << 24));
 }
 
+// LDS-staged dot4 matvec (rein_mvl_*, kernels/matvec_lds.h), 2..4 activation rows: the rows of a
+// workgroup's activations live in LDS, B x (in_dim / 32) x 40 bytes of it.
+constexpr size_t kLdsPerCu = 160u * 1024u;
+size_t mvl_lds_bytes(unsigned in_dim, unsigned n_rows) { return (size_t)(n_rows <= 2 ? 2 : 4) * (in_dim / 32) * 40; }
+
+// Launch geometry, from a sweep over R 1/2/4, 4-16 wavefronts per workgroup and 1-4 resident workgroups
+// per CU on 15 shapes (Q4_K and Q6_K, 2 and 4 rows).  Up to 16 wavefronts per workgroup share one
+// copy of the activations.
+//   * A matrix whose row groups all fit the machine at once (at most two workgroups of 16 wavefronts per
+//     CU) is dealt out evenly, each wavefront one row group: 5120 rows are 512 workgroups of ten
+//     wavefronts at one row per wavefront, 256 of ten at two.  R is the smallest rows-per-wavefront for
+//     which that works and the copies fit the CU's LDS (Q6_K starts at two from in_dim 8192: 14336 -> 4096
+//     at 4 rows 17.8 us against 19.2, 18944 -> 3584 23.0 against 25.2).
+//   * Wider matrices run persistent: up to four workgroups per CU of four (2 rows) or eight (3-4 rows)
+//     wavefronts at two rows per wavefront, striding over the row groups, each trip requesting the
+//     next row group's first one.
+// us, Q4_K, this geometry against the best other one: 5120 -> 5120 at 4 rows 7.89 (8.12); 17408 -> 5120
+// 13.72 (14.28) and 18.84 (22.6); 14336 -> 4096 9.49 (10.04) and 12.40 (12.75); 5120 -> 34816 at 2 rows
+// 22.26 (22.61); 5120 -> 17408 13.22 (13.29); 8192 -> 28672 at 4 rows 33.03 (33.99).
+void mvl_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, unsigned* r_out, unsigned* wpb_out, unsigned* grid_out)
+{
+    const unsigned copies = (unsigned)std::min<size_t>(4, kLdsPerCu / mvl_lds_bytes(in_dim, n_rows));
+    unsigned r = 0, wpb = 0, grid = 0;
+    for (unsigned rr = fmt == REIN_TYPE_Q6_K && in_dim >= 8192 ? 2 : 1; rr <= 2 && r == 0; rr *= 2) {
+        const unsigned groups = (out_dim + rr - 1) / rr;
+        const unsigned c = (groups + kCUs * 16 - 1) / (kCUs * 16);
+        if (c > 2) break;                    // too wide for one row group per wavefront: persistent
+        if (c > copies) continue;            // the CU's LDS holds fewer copies: more rows per wavefront
+        r = rr;
+        wpb = (groups + kCUs * c - 1) / (kCUs * c);
+        grid = (groups + wpb - 1) / wpb;
+    }
+    if (r == 0) {
+        r = 2;
+        wpb = n_rows <= 2 ? 4 : 8;
+        while (copies * wpb < 16) wpb *= 2;
+        const unsigned groups = (out_dim + 1) / 2;
+        grid = std::min(kCUs * copies, (groups + wpb - 1) / wpb);
+    }
+    const unsigned r_forced = opt_u(O_MV_ROWS, 0), wpb_forced = opt_u(O_MV_WPB, 0);
+    if (r_forced == 1 || r_forced == 2 || r_forced == 4 || (wpb_forced >= 1 && wpb_forced <= 16)) {
+        if (r_forced == 1 || r_forced == 2 || r_forced == 4) r = r_forced;
+        if (wpb_forced >= 1 && wpb_forced <= 16) wpb = wpb_forced;
+        grid = ((out_dim + r - 1) / r + wpb - 1) / wpb;
+    }
+    *r_out = r; *wpb_out = wpb; *grid_out = grid;
+}
+
+// Whether a batched decode of 2..4 rows runs on the LDS-staged kernel.  From one run of the library's choice
+// among the other three families against this kernel, six formats x 16 shapes x 2 / 3 / 4 rows (ratio of the two
+// times; the kernel's outputs are those of the dot4 family bit for bit):
+//   3-4 rows  ahead for every format when the matrix has at most 6144 rows or a contraction of 8192 and more,
+//             from 2^24 weights: 5120 -> 5120 1.07-1.24, 17408 -> 5120 1.18-1.29, 4096 -> 4096 1.28-1.47,
+//             14336 -> 4096 1.22-1.57, 18944 -> 3584 1.15-1.58, 8192 -> 8192 1.00-1.11, 28672 -> 8192 1.07-1.25,
+//             8192 -> 28672 1.17-1.59.  Behind on short contractions against many rows (5120 -> 34816 0.76-1.05,
+//             5120 -> 17408 0.77-1.08, 3584 -> 18944 0.77-1.01, 5120 -> 7168 0.84-1.02), where the skinny MMQ and
+//             the 4x4x4 kernel stream best, and on small matrices (2048 -> 2048 0.86-1.04).
+//   2 rows    ahead for every format at contractions of 8192 and more from 2^25 weights (17408 -> 5120 0.98-1.11,
+//             14336 -> 4096 0.97-1.24, 8192 -> 8192 1.03-1.16, 28672 -> 8192 1.12-1.28, 18944 -> 3584 1.10-1.63,
+//             8192 -> 28672 1.10-1.34); on shorter contractions only Q4_K, Q4_0 and Q5_K against 14336 rows and
+//             more (5120 -> 34816 1.13 / 1.08 / 1.06, 5120 -> 17408 1.17 / 1.14 / 1.09, 3584 -> 18944 1.16 / 1.13 /
+//             1.05, 4096 -> 14336 1.04 / 1.08 / 1.03; Q6_K 0.91-1.10, IQ4_XS 0.97-1.06, Q8_0 0.95-1.08 there).
+bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    if (n_rows < 2 || n_rows > 4 || mvl_lds_bytes(in_dim, n_rows) > kLdsPerCu) return false;
+    if (opt_is_set(O_MV_LDS)) return opt_u(O_MV_LDS, 0) != 0;
+    if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
+    const unsigned long long weights = (unsigned long long)in_dim * out_dim;
+    if (n_rows >= 3) return weights >= (1ull << 24) && (out_dim <= 6144 || in_dim >= 8192);
+    if (weights < (1ull << 25)) return false;
+    if (in_dim >= 8192) return true;
+    return out_dim >= 14336 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K);
+}
+
+int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                      unsigned n_rows, rein_stream_t s)
+{
+    unsigned r, wpb, grid;
+    mvl_geometry(fmt, in_dim, out_dim, n_rows, &r, &wpb, &grid);
+    const unsigned b = n_rows <= 2 ? 2 : 4;
+    const std::string name = std::string("rein_mvl_") + fmt_tag(fmt) + "_r" + std::to_string(r) + "_b" + std::to_string(b);
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+    return launch(name, grid, 1, 1, wpb * 64, (unsigned)mvl_lds_bytes(in_dim, n_rows), s, args);
+}
+
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
                   unsigned out_dim, unsigned n_rows, rein_stream_t s)
 {
@@ -315,6 +400,7 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    if (use_mvl(fmt, in_dim, out_dim, n_rows)) return launch_matvec_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const bool small = small_for_matrix_cores(fmt, in_dim, out_dim, n_rows);
     if (!small && use_quad(fmt, out_dim, n_rows)) {
         // four output rows per wavefront, four wavefronts per workgroup

@@ -1,0 +1,127 @@
+"""The batched decode matvec that stages the activation rows in LDS (rein_mvl_*, 2..4 rows) against
+the oracle and, bit for bit, against the dot4 family whose arithmetic it repeats: every dense
+format, output row counts that do not divide into workgroups, ragged contractions, each launch
+geometry (one row group per wavefront, and persistent wavefronts that stride over row groups),
+forced rows per wavefront and workgroup sizes, and the shapes the library sends there by itself.
+REIN_MV_LDS forces the kernel on (1) or off (0)."""
+import numpy as np
+import pytest
+
+import reinstinct_amd as rein
+from reinstinct_amd import hip, quant, runtime
+from reinstinct_amd._lib import init
+from oracle import orc
+from helpers import assert_close_f32, dev, random_raw_weights
+
+pytestmark = pytest.mark.gpu
+
+DENSE = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS, rein.IQ3_S]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def gpu():
+    init()
+    hip.set_device(0)
+    yield
+    hip.synchronize()
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def run(fmt, packed, xq, in_dim, out_dim, n_rows):
+    dw, dq = dev(packed), dev(xq)
+    dy = dev(np.full(n_rows * out_dim, np.nan, np.float32))
+    runtime.matvec_batched_xq8(fmt, dw, dq, dy, in_dim, out_dim, n_rows)
+    hip.synchronize()
+    return dy.to_host(np.float32).reshape(n_rows, out_dim)
+
+
+def run_lds(options, fmt, packed, xq, in_dim, out_dim, n_rows):
+    options.set("REIN_MV_LDS", "1")
+    got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    options.unset("REIN_MV_LDS")
+    return got
+
+
+def run_dot4(options, fmt, packed, xq, in_dim, out_dim, n_rows):
+    for name, value in (("REIN_MV_LDS", "0"), ("REIN_SKINNY_FROM", "99"), ("REIN_QUAD_FROM", "99")):
+        options.set(name, value)
+    got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    for name in ("REIN_MV_LDS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM"):
+        options.unset(name)
+    return got
+
+
+def check(options, fmt, in_dim, out_dim, rows=(2, 3, 4), seed=0):
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + in_dim + seed)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in rows:
+        print("lds matvec", fmt, in_dim, out_dim, n_rows, flush=True)
+        xq = orc.quantize_q8(np.random.default_rng(n_rows + seed).standard_normal((n_rows, in_dim)).astype(np.float32))
+        got = run_lds(options, fmt, packed, xq, in_dim, out_dim, n_rows)
+        want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
+        assert_close_f32(got, want, what=f"lds fmt {fmt} {in_dim}->{out_dim} rows {n_rows}")
+        same = run_dot4(options, fmt, packed, xq, in_dim, out_dim, n_rows)
+        assert np.array_equal(bits(got), bits(same)), f"not the dot4 family's bits: fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
+
+
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (256, 64), (5120, 130), (4096, 33), (2304, 4099)])
+def test_lds_matvec_parity(fmt, in_dim, out_dim, options):
+    check(options, fmt, in_dim, out_dim)
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])       # 32-weight blocks: any multiple of 32
+@pytest.mark.parametrize("in_dim", [32, 96, 352, 544, 1056, 2080, 4128])
+def test_lds_matvec_ragged_contraction(fmt, in_dim, options):
+    check(options, fmt, in_dim, 37)
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q6_K, rein.Q8_0])
+@pytest.mark.parametrize("in_dim,out_dim", [(512, 9001), (256, 40003), (768, 16500)])
+def test_lds_matvec_persistent_wavefronts_stride_over_row_groups(fmt, in_dim, out_dim, options):
+    # more than 8192 rows: at most four workgroups per CU, each wavefront takes several row groups in turn
+    check(options, fmt, in_dim, out_dim)
+
+
+@pytest.mark.parametrize("rows_per_wave", [1, 2, 4])
+@pytest.mark.parametrize("waves", [1, 5, 16])
+def test_lds_matvec_forced_geometry(rows_per_wave, waves, options):
+    options.set("REIN_MV_ROWS", str(rows_per_wave))
+    options.set("REIN_MV_WPB", str(waves))
+    fmt, in_dim, out_dim = rein.Q4_K, 1280, 1031
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=waves)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in (2, 4):
+        xq = orc.quantize_q8(np.random.default_rng(n_rows).standard_normal((n_rows, in_dim)).astype(np.float32))
+        got = run_lds(options, fmt, packed, xq, in_dim, out_dim, n_rows)
+        assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what=f"R {rows_per_wave} W {waves}")
+
+
+def test_lds_matvec_largest_contraction_and_fallback_beyond_it(options):
+    # four rows x 32768 values fill the CU's 160 KB of LDS exactly; one superblock more and the forced option
+    # steps aside for the other families
+    fmt, out_dim = rein.Q4_K, 70
+    for in_dim in (32768, 33024):
+        raw = random_raw_weights(fmt, in_dim, out_dim, seed=in_dim)
+        packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+        xq = orc.quantize_q8(np.random.default_rng(1).standard_normal((4, in_dim)).astype(np.float32))
+        got = run_lds(options, fmt, packed, xq, in_dim, out_dim, 4)
+        assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, 4), what=f"K {in_dim}")
+
+
+@pytest.mark.parametrize("fmt,n_rows", [(rein.Q4_K, 3), (rein.Q6_K, 4), (rein.Q8_0, 3), (rein.IQ4_XS, 4)])
+def test_default_dispatch_takes_the_lds_kernel_for_narrow_matrices(fmt, n_rows, options):
+    # 3-4 rows, at most 6144 output rows, from 2^24 weights: the library's own choice -- the same bits as forced
+    in_dim, out_dim = 5120, 4100
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
+    got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what="default dispatch")
+    assert np.array_equal(bits(got), bits(run_lds(options, fmt, packed, xq, in_dim, out_dim, n_rows)))
+    # five rows and more stay with the matrix-core families
+    xq8 = orc.quantize_q8(np.random.default_rng(8).standard_normal((8, in_dim)).astype(np.float32))
+    assert_close_f32(run(fmt, packed, xq8, in_dim, out_dim, 8), orc.matvec_q8(fmt, packed, in_dim, out_dim, xq8, 8), what="8 rows")
