@@ -92,7 +92,8 @@ int rein_is_loaded(void);
  * Names (rein_option_name enumerates them): REIN_MV_ROWS, REIN_MV_WPB (decode matvec rows per
  * wavefront 1/2/4, wavefronts per workgroup 1/2/4; 1..16 for the LDS-staged kernel), REIN_MV_LDS
  * (batched decode of 2..4 rows on the kernel that stages the activation rows in LDS: 0 never,
- * 1 whenever the rows fit), REIN_SKINNY_FROM, REIN_SKINNY_KS,
+ * 1 whenever the rows fit), REIN_QUAD_LDS (the same for the 4x4x4 kernel, 3..8 rows),
+ * REIN_SKINNY_FROM, REIN_SKINNY_KS,
  * REIN_QUAD_FROM (batched decode: row count from which the skinny MMQ / the 4x4x4 kernel run,
  * wavefronts per row tile), REIN_GROUPED_STRIDED (1: the reference-named strided grouped
  * kernel), REIN_MMQ_TM, REIN_MMQ_N64 (int8 GEMM tile: 32 forces 32-token tiles; 64-token tiles

@@ -139,8 +139,8 @@ int check_ptr(const char* who, const void* p, size_t align, const char* what)
 // rein_set_option changes an entry, so the launch an entry point chooses depends on its arguments
 // and on this table alone.  Entries are single atomic words: setting one while another thread
 // launches is safe, the launch sees the old or the new value.
-enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
-const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
+enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
+const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
 constexpr uint64_t kOptSet = 1ull << 63;
 std::atomic<uint64_t> g_opts[O_COUNT];          // zero = unset
 std::once_flag g_opts_env_once;
@@ -367,7 +367,8 @@ void mvl_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, u
 //             14336 -> 4096 0.97-1.24, 8192 -> 8192 1.03-1.16, 28672 -> 8192 1.12-1.28, 18944 -> 3584 1.10-1.63,
 //             8192 -> 28672 1.10-1.34); on shorter contractions only Q4_K, Q4_0 and Q5_K against 14336 rows and
 //             more (5120 -> 34816 1.13 / 1.08 / 1.06, 5120 -> 17408 1.17 / 1.14 / 1.09, 3584 -> 18944 1.16 / 1.13 /
-//             1.05, 4096 -> 14336 1.04 / 1.08 / 1.03; Q6_K 0.91-1.10, IQ4_XS 0.97-1.06, Q8_0 0.95-1.08 there).
+//             1.05, 4096 -> 14336 1.04 / 1.08 / 1.03) and IQ3_S (1.05-1.14); Q6_K 0.91-1.10, IQ4_XS 0.97-1.06, Q8_0
+//             0.95-1.08 there.
 bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     if (n_rows < 2 || n_rows > 4 || mvl_lds_bytes(in_dim, n_rows) > kLdsPerCu) return false;
@@ -377,7 +378,7 @@ bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
     if (n_rows >= 3) return weights >= (1ull << 24) && (out_dim <= 6144 || in_dim >= 8192);
     if (weights < (1ull << 25)) return false;
     if (in_dim >= 8192) return true;
-    return out_dim >= 14336 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K);
+    return out_dim >= 14336 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S);
 }
 
 int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
@@ -391,6 +392,61 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
     return launch(name, grid, 1, 1, wpb * 64, (unsigned)mvl_lds_bytes(in_dim, n_rows), s, args);
 }
 
+// The 4x4x4 kernel with the activation rows staged in LDS (rein_mvql_*, kernels/matvec_quad.h), 3..8 rows.
+// Geometry from a sweep over 4-16 wavefronts per workgroup, 1-4 resident workgroups per CU and one row group
+// per wavefront or persistent wavefronts (Q4_K, Q6_K, Q5_K, Q8_0 on six shapes): up to 16384 rows 256
+// workgroups with one group of four rows per wavefront (5120 rows: five wavefronts, 14336: fourteen); beyond,
+// 512 workgroups of eight wavefronts that stride over the row groups.
+struct QuadLdsGeometry { unsigned wpb, grid; size_t lds; };
+QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    const unsigned n_sub = in_dim / 32, stride = n_sub + ((20u - (n_sub & 15u)) & 15u), t = n_rows <= 4 ? 4 : 8;
+    const unsigned parts = fmt == REIN_TYPE_Q8_0 ? 3 : 2;               // 16-byte parts of Fmt<FMT>::Raw
+    const unsigned groups = (out_dim + 3) / 4;
+    QuadLdsGeometry g;
+    g.wpb = std::min(16u, (groups + kCUs - 1) / kCUs);
+    g.grid = (groups + g.wpb - 1) / g.wpb;
+    if (groups > kCUs * 16) { g.wpb = 8; g.grid = 2 * kCUs; }
+    const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
+    if (wpb_forced >= 1 && wpb_forced <= 16) { g.wpb = wpb_forced; g.grid = (groups + g.wpb - 1) / g.wpb; }
+    g.lds = (size_t)t * stride * 40 + (size_t)g.wpb * parts * 76 * 16;
+    return g;
+}
+
+// Whether a batched decode of 3..8 rows runs on it.  One run of the library's other choice against this kernel, seven
+// formats x 16 shapes x 3 / 4 / 5 / 6 / 8 rows (ratio of the two times), from 2^24 weights (below, 0.52-0.99):
+//   5-8 rows  Q6_K, Q5_K, IQ4_XS (the formats of the 4x4x4 kernel): level or ahead everywhere -- 5120 -> 5120 1.05-1.18,
+//             5120 -> 34816 1.02-1.25, 4096 -> 14336 1.31-1.47, 8192 -> 8192 1.04-1.16, 2048 -> 16384 1.30-1.45,
+//             14336 -> 4096 1.01-1.15.  Q4_K, Q8_0, Q4_0, IQ3_S (skinny MMQ otherwise): ahead between 8192 and 20480
+//             rows (8192 -> 8192 1.11-1.23, 4096 -> 14336 1.21-1.36, 5120 -> 17408 1.05-1.16, 2048 -> 16384 1.20-1.35),
+//             behind or level outside (5120 -> 5120 0.96-1.02, 14336 -> 4096 0.84-0.95, 5120 -> 34816 0.95-1.08,
+//             8192 -> 28672 0.92-1.20).
+//   3-4 rows  after the LDS-staged dot4 kernel has had its pick (narrow matrices and long contractions): ahead against
+//             14336 rows and more for Q5_K 1.03-1.18, Q8_0 0.99-1.17, IQ3_S 1.08-1.51, Q4_K 0.98-1.18; mixed for
+//             Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
+// Contractions whose rows do not fit the LDS (eight rows from in_dim 16384) keep the other kernels.
+bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    if (n_rows < 3 || n_rows > 8 || mvql_geometry(fmt, in_dim, out_dim, n_rows).lds > kLdsPerCu) return false;
+    if (opt_is_set(O_QUAD_LDS)) return opt_u(O_QUAD_LDS, 0) != 0;
+    if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
+    if ((unsigned long long)in_dim * out_dim < (1ull << 24)) return false;
+    if (n_rows >= 5) {
+        if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS) return true;
+        return out_dim >= 8192 && out_dim <= 20480;
+    }
+    return out_dim >= 14336 && (fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K);
+}
+
+int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
+                    unsigned n_rows, rein_stream_t s)
+{
+    const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
+    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+    return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
+}
+
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
                   unsigned out_dim, unsigned n_rows, rein_stream_t s)
 {
@@ -401,6 +457,7 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
     if (use_mvl(fmt, in_dim, out_dim, n_rows)) return launch_matvec_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (use_mvql(fmt, in_dim, out_dim, n_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const bool small = small_for_matrix_cores(fmt, in_dim, out_dim, n_rows);
     if (!small && use_quad(fmt, out_dim, n_rows)) {
         // four output rows per wavefront, four wavefronts per workgroup

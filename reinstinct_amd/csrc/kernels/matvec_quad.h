@@ -228,3 +228,147 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
     {                                                                                             \
         rein_matvec_quad_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows);                        \
     }
+
+// ---- the same kernel with the activation rows staged in LDS once per workgroup ----------------------
+// In the kernel above a lane fetches one BlockQ8 per group of four activation rows and trip from memory
+// (40-byte records at a 40-byte stride) and hands it to the lane that needs it through LDS, like the
+// weights: at eight rows that is five times the weight bytes through the vector cache, plus six LDS
+// stores per trip.  Here the workgroup (up to 16 wavefronts) copies the 4*NT activation rows into LDS
+// once, as planes (quants 0..15, quants 16..31, {d, xsum}) whose row stride is 4 mod 16 entries, so that
+// the compute-side lane (block b, row j) reads its operand at (4t + j) * stride + sub-block directly and a
+// quarter-wave pass covers 64 different banks.  Only the weights still take the trip through the
+// wavefront's private LDS image.  A trip requests the next trip's weights (or the first trip of the
+// wavefront's next row group) before it computes.  Same arithmetic in the same order as the kernel above.
+// Launch: block = 64 x W threads (W <= 16), dynamic shared memory =
+//   4*NT * stride * 40 + W * kParts * 76 * 16 bytes, stride = n_sub + ((20 - n_sub % 16) % 16),
+// any grid (wavefronts stride over the row groups).
+template <int FMT, int NT>
+__device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
+                                                          float* __restrict__ y, unsigned in_dim, unsigned out_dim,
+                                                          unsigned n_rows)
+{
+    using F = Fmt<FMT>;
+    using Raw = typename F::Raw;
+    constexpr bool kTwo = F::kDotParts == 2;
+    constexpr int kParts = QuadRawBits<FMT>::kParts;
+    constexpr unsigned T = 4u * NT;
+    extern __shared__ uint4 rein_mvql_lds[];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wpb = blockDim.x >> 6;
+    const unsigned j = lane & 3u, blk = lane >> 2;
+    const unsigned lr = lane >> 4, ls = lane & 15u;
+    const unsigned put = lane + 4u * lr;
+    const unsigned get = 16u * j + blk + 4u * j;
+    const unsigned n_sub = in_dim >> 5;
+    // row stride of the activation planes: 4 mod 16 entries, so that the four activation rows of a
+    // quarter-wave pass (blocks 0..3, j = 0..3) read 64 different banks
+    const unsigned stride = n_sub + ((20u - (n_sub & 15u)) & 15u);
+    uint4* xlo = rein_mvql_lds;
+    uint4* xhi = xlo + T * stride;
+    uint2* xhd = reinterpret_cast<uint2*>(xhi + T * stride);
+    uint4* stage = reinterpret_cast<uint4*>(xhd + T * stride) + wave * (kParts * 76u);
+    const F fmt(w, n_sub, out_dim);
+    const unsigned n_groups = (out_dim + 3u) / 4u;
+    const XSums no_xs = {0, 0};
+
+    unsigned g = blockIdx.x * wpb + wave;
+    Raw rq;
+    {
+        const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
+        rq = fmt.load(row, min(ls, n_sub - 1u));
+    }
+    for (unsigned e = threadIdx.x; e < T * n_sub; e += blockDim.x) {
+        const unsigned t = e / n_sub, sb = e - t * n_sub;
+        const BlockQ8 v = xq[(size_t)min(t, n_rows - 1u) * n_sub + sb];
+        xlo[t * stride + sb] = make_uint4((unsigned)v.qs[0], (unsigned)v.qs[1], (unsigned)v.qs[2], (unsigned)v.qs[3]);
+        xhi[t * stride + sb] = make_uint4((unsigned)v.qs[4], (unsigned)v.qs[5], (unsigned)v.qs[6], (unsigned)v.qs[7]);
+        xhd[t * stride + sb] = make_uint2(__builtin_bit_cast(unsigned, v.d), __builtin_bit_cast(unsigned, v.xsum));
+    }
+    __syncthreads();
+
+    for (; g < n_groups; g += gridDim.x * wpb) {
+        float acc[NT][4];
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+
+        for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) {
+            const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(rq);
+#pragma unroll
+            for (int i = 0; i < kParts; i++) stage[i * 76 + put] = bits.p[i];
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                const bool last = sb0 + 16u >= n_sub;
+                const unsigned ng = last ? min(g + gridDim.x * wpb, n_groups - 1u) : g;
+                const unsigned nrow = min(ng * 4u + lr, out_dim - 1u);
+                rq = fmt.load(nrow, min((last ? 0u : sb0 + 16u) + ls, n_sub - 1u));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            QuadRawBits<FMT> mine;
+#pragma unroll
+            for (int i = 0; i < kParts; i++) mine.p[i] = stage[i * 76 + get];
+            Raw my;
+            __builtin_memcpy(&my, &mine, sizeof(my));
+            SubW sw;
+            F::unpack(my, sw);
+            const bool live = sb0 + blk < n_sub;
+            const unsigned sbx = min(sb0 + blk, n_sub - 1u);
+            int a[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) a[k] = rein_fold_offset<FMT>(sw.w[k]);
+            float s0[4], s1[4];
+            s0[0] = rein_quad_bcast<0>(sw.s0); s0[1] = rein_quad_bcast<1>(sw.s0);
+            s0[2] = rein_quad_bcast<2>(sw.s0); s0[3] = rein_quad_bcast<3>(sw.s0);
+            s1[0] = rein_quad_bcast<0>(sw.s1); s1[1] = rein_quad_bcast<1>(sw.s1);
+            s1[2] = rein_quad_bcast<2>(sw.s1); s1[3] = rein_quad_bcast<3>(sw.s1);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const unsigned at = (4u * t + j) * stride + sbx;
+                const uint4 lo = xlo[at], hi = xhi[at];
+                const uint2 hd = xhd[at];
+                const bool on = live && 4u * t + j < n_rows;
+                const float dx = on ? __builtin_bit_cast(float, hd.x) : 0.0f;
+                const float xsum = on ? __builtin_bit_cast(float, hd.y) : 0.0f;
+                const int q[8] = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+                rein_quad_v4i d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};
+#pragma unroll
+                for (int k = 0; k < 4; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
+                if (kTwo) {
+#pragma unroll
+                    for (int k = 4; k < 8; k++) d1 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d1, 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int k = 4; k < 8; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    SubW sc;
+                    sc.s0 = s0[r];
+                    sc.s1 = s1[r];
+                    acc[t][r] += F::term(sc, d0[r], d1[r], dx, xsum, no_xs);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float v = acc[t][r];
+                v += __shfl_xor(v, 4);
+                v += __shfl_xor(v, 8);
+                v += __shfl_xor(v, 16);
+                v += __shfl_xor(v, 32);
+                const unsigned tok = 4u * t + j, orow = g * 4u + r;
+                if (blk == 0u && tok < n_rows && orow < out_dim) y[(size_t)tok * out_dim + orow] = v;
+            }
+    }
+}
+
+// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows), n_rows <= 4 * NT
+#define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT)                                                \
+    extern "C" __global__ __launch_bounds__(1024) void name(                                      \
+        const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y,    \
+        unsigned int in_dim, unsigned int out_dim, unsigned int n_rows)                           \
+    {                                                                                             \
+        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows);                    \
+    }

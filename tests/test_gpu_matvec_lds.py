@@ -1,9 +1,10 @@
-"""The batched decode matvec that stages the activation rows in LDS (rein_mvl_*, 2..4 rows) against
-the oracle and, bit for bit, against the dot4 family whose arithmetic it repeats: every dense
-format, output row counts that do not divide into workgroups, ragged contractions, each launch
-geometry (one row group per wavefront, and persistent wavefronts that stride over row groups),
-forced rows per wavefront and workgroup sizes, and the shapes the library sends there by itself.
-REIN_MV_LDS forces the kernel on (1) or off (0)."""
+"""The two batched decode kernels that stage the activation rows in LDS -- the dot4 form (rein_mvl_*,
+2..4 rows) and the 4x4x4 matrix-instruction form (rein_mvql_*, 3..8 rows) -- against the oracle and,
+bit for bit, against the family whose arithmetic each repeats: every dense format, output row
+counts that do not divide into workgroups, ragged contractions, each launch geometry (one row group
+per wavefront, and persistent wavefronts that stride over row groups), forced rows per wavefront
+and workgroup sizes, and the shapes the library sends there by itself.  REIN_MV_LDS and
+REIN_QUAD_LDS force the kernels on (1) or off (0)."""
 import numpy as np
 import pytest
 
@@ -125,3 +126,83 @@ def test_default_dispatch_takes_the_lds_kernel_for_narrow_matrices(fmt, n_rows, 
     # five rows and more stay with the matrix-core families
     xq8 = orc.quantize_q8(np.random.default_rng(8).standard_normal((8, in_dim)).astype(np.float32))
     assert_close_f32(run(fmt, packed, xq8, in_dim, out_dim, 8), orc.matvec_q8(fmt, packed, in_dim, out_dim, xq8, 8), what="8 rows")
+
+
+# ---- the 4x4x4 matrix-instruction form --------------------------------------------------------------
+
+def run_opts(options, pairs, fmt, packed, xq, in_dim, out_dim, n_rows):
+    for name, value in pairs:
+        options.set(name, value)
+    got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    for name, _ in pairs:
+        options.unset(name)
+    return got
+
+
+def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0):
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + in_dim + seed)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in rows:
+        print("lds quad", fmt, in_dim, out_dim, n_rows, flush=True)
+        xq = orc.quantize_q8(np.random.default_rng(n_rows + seed).standard_normal((n_rows, in_dim)).astype(np.float32))
+        got = run_opts(options, [("REIN_QUAD_LDS", "1"), ("REIN_MV_LDS", "0")], fmt, packed, xq, in_dim, out_dim, n_rows)
+        want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
+        assert_close_f32(got, want, what=f"lds quad fmt {fmt} {in_dim}->{out_dim} rows {n_rows}")
+        same = run_opts(options, [("REIN_QUAD_FROM", "1"), ("REIN_QUAD_LDS", "0"), ("REIN_MV_LDS", "0")], fmt, packed, xq,
+                        in_dim, out_dim, n_rows)
+        if fmt == rein.Q6_K and n_rows <= 4:
+            # the compiler contracts the two-scale term of this one instantiation differently: last-bit differences
+            assert np.allclose(got, same, rtol=0.0, atol=2e-6 * float(np.abs(same).max())), f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
+        else:
+            assert np.array_equal(bits(got), bits(same)), f"not the 4x4x4 family's bits: fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
+
+
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (256, 64), (5120, 130), (4096, 33), (2304, 4099)])
+def test_lds_quad_parity(fmt, in_dim, out_dim, options):
+    check_quad_lds(options, fmt, in_dim, out_dim)
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])
+@pytest.mark.parametrize("in_dim", [32, 96, 352, 544, 1056, 2080])
+def test_lds_quad_ragged_contraction(fmt, in_dim, options):
+    check_quad_lds(options, fmt, in_dim, 37, rows=(3, 4, 7))
+
+
+@pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q6_K, rein.Q8_0])
+@pytest.mark.parametrize("in_dim,out_dim", [(256, 70003), (512, 16500)])
+def test_lds_quad_persistent_and_widest_workgroups(fmt, in_dim, out_dim, options):
+    # 70003 rows: 512 workgroups of eight wavefronts stride over 17501 row groups; 16500: sixteen wavefronts per workgroup
+    check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 8))
+
+
+@pytest.mark.parametrize("waves", [1, 3, 16])
+def test_lds_quad_forced_workgroup_size(waves, options):
+    options.set("REIN_MV_WPB", str(waves))
+    check_quad_lds(options, rein.Q5_K, 1280, 1031, rows=(4, 5))
+
+
+def test_lds_quad_fallback_when_the_rows_do_not_fit(options):
+    # eight rows x 16384 values and the wavefronts' weight images exceed 160 KB: the forced option steps aside
+    fmt, in_dim, out_dim = rein.Q4_K, 16384, 70
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=2)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    for n_rows in (4, 8):
+        xq = orc.quantize_q8(np.random.default_rng(1).standard_normal((n_rows, in_dim)).astype(np.float32))
+        got = run_opts(options, [("REIN_QUAD_LDS", "1"), ("REIN_MV_LDS", "0")], fmt, packed, xq, in_dim, out_dim, n_rows)
+        assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what=f"K {in_dim} rows {n_rows}")
+
+
+@pytest.mark.parametrize("fmt,in_dim,out_dim,n_rows", [(rein.Q6_K, 5120, 4100, 8), (rein.IQ4_XS, 5120, 4100, 6),
+                                                      (rein.Q4_K, 2048, 8200, 5), (rein.Q8_0, 1024, 16388, 8),
+                                                      (rein.Q5_K, 1280, 14340, 3)])
+def test_default_dispatch_takes_the_lds_quad_kernel(fmt, in_dim, out_dim, n_rows, options):
+    # 5-8 rows: Q6_K / Q5_K / IQ4_XS everywhere, the other formats between 8192 and 20480 rows; 3-4 rows: Q5_K,
+    # Q8_0, IQ3_S and Q4_K against 14336 rows and more (from 2^24 weights)
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
+    packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
+    got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what="default dispatch")
+    forced = run_opts(options, [("REIN_QUAD_LDS", "1"), ("REIN_MV_LDS", "0")], fmt, packed, xq, in_dim, out_dim, n_rows)
+    assert np.array_equal(bits(got), bits(forced)), "the default launch is not the LDS-staged 4x4x4 kernel"

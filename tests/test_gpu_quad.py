@@ -65,17 +65,21 @@ def test_quad_matvec_ragged_contraction(fmt, in_dim, options):
         assert_close_f32(run(fmt, packed, xq, in_dim, out_dim, n_rows), want, what=f"quad ragged {in_dim}")
 
 
-@pytest.mark.parametrize("fmt,n_rows", [(rein.Q6_K, 3), (rein.Q6_K, 8), (rein.Q5_K, 4), (rein.IQ4_XS, 3), (rein.IQ4_XS, 6)])
-def test_default_dispatch_at_benchmark_width(fmt, n_rows):
+@pytest.mark.parametrize("fmt,n_rows", [(rein.Q6_K, 3), (rein.Q6_K, 4), (rein.Q5_K, 4), (rein.IQ4_XS, 3)])
+def test_default_dispatch_at_benchmark_width(fmt, n_rows, options):
     # the row counts the library sends to these kernels by itself, at the K of the decode shapes (a matrix
     # large enough that the library does not keep it on dot4, and with more than 6144 rows, below which 3-4
-    # rows go to the LDS-staged dot4 kernel)
+    # rows go to the LDS-staged dot4 kernel; five rows and more go to the LDS-staged form of these kernels)
     in_dim, out_dim = 5120, 6404
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
     want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
-    assert_close_f32(run(fmt, packed, xq, in_dim, out_dim, n_rows), want, what="default dispatch")
+    got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    assert_close_f32(got, want, what="default dispatch")
+    options.set("REIN_QUAD_FROM", "1")
+    forced = run(fmt, packed, xq, in_dim, out_dim, n_rows)
+    assert np.array_equal(np.ascontiguousarray(got).view(np.uint32), np.ascontiguousarray(forced).view(np.uint32))
 
 
 def bits(a):
