@@ -397,19 +397,35 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
 // per wavefront or persistent wavefronts (Q4_K, Q6_K, Q5_K, Q8_0 on six shapes): up to 16384 rows 256
 // workgroups with one group of four rows per wavefront (5120 rows: five wavefronts, 14336: fourteen); beyond,
 // 512 workgroups of eight wavefronts that stride over the row groups.
-struct QuadLdsGeometry { unsigned wpb, grid; size_t lds; };
+struct QuadLdsGeometry { unsigned wpb, grid, phase_sub; size_t lds; };       // lds == 0: no launch fits
 QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    const unsigned n_sub = in_dim / 32, stride = n_sub + ((20u - (n_sub & 15u)) & 15u), t = n_rows <= 4 ? 4 : 8;
+    const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : 8;
     const unsigned parts = fmt == REIN_TYPE_Q8_0 ? 3 : 2;               // 16-byte parts of Fmt<FMT>::Raw
     const unsigned groups = (out_dim + 3) / 4;
     QuadLdsGeometry g;
     g.wpb = std::min(16u, (groups + kCUs - 1) / kCUs);
     g.grid = (groups + g.wpb - 1) / g.wpb;
-    if (groups > kCUs * 16) { g.wpb = 8; g.grid = 2 * kCUs; }
+    const bool persistent = groups > kCUs * 16;
+    if (persistent) { g.wpb = 8; g.grid = 2 * kCUs; }
     const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
     if (wpb_forced >= 1 && wpb_forced <= 16) { g.wpb = wpb_forced; g.grid = (groups + g.wpb - 1) / g.wpb; }
-    g.lds = (size_t)t * stride * 40 + (size_t)g.wpb * parts * 76 * 16;
+    const auto bytes = [&](unsigned n_stage) {
+        const unsigned stride = n_stage + ((20u - (n_stage & 15u)) & 15u);
+        return (size_t)t * stride * 40 + (size_t)g.wpb * parts * 76 * 16;
+    };
+    g.phase_sub = n_sub;
+    g.lds = bytes(n_sub);
+    if (g.lds > kLdsPerCu) {
+        // The rows do not fit: stage the contraction in phases.  That form keeps a wavefront's partial sums in
+        // registers across the phases, so it needs one row group per wavefront at most.
+        g.lds = 0;
+        if ((unsigned long long)g.grid * g.wpb >= groups)
+            for (unsigned phases = 2; phases <= 8 && g.lds == 0; phases++) {
+                const unsigned per = (((n_sub + phases - 1) / phases) + 15u) & ~15u;
+                if (bytes(per) <= kLdsPerCu) { g.phase_sub = per; g.lds = bytes(per); }
+            }
+    }
     return g;
 }
 
@@ -420,20 +436,23 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
 //             14336 -> 4096 1.01-1.15.  Q4_K, Q8_0, Q4_0, IQ3_S (skinny MMQ otherwise): ahead between 8192 and 20480
 //             rows (8192 -> 8192 1.11-1.23, 4096 -> 14336 1.21-1.36, 5120 -> 17408 1.05-1.16, 2048 -> 16384 1.20-1.35),
 //             behind or level outside (5120 -> 5120 0.96-1.02, 14336 -> 4096 0.84-0.95, 5120 -> 34816 0.95-1.08,
-//             8192 -> 28672 0.92-1.20).
+//             8192 -> 28672 0.92-1.20).  Contractions staged in phases (eight rows from in_dim 16384): Q6_K 1.05-1.14,
+//             Q5_K 1.00-1.11, IQ4_XS 0.99-1.08 on 17408 -> 5120, 14336 -> 4096, 28672 -> 8192, 18944 -> 3584; the
+//             other formats 0.71-0.98 there and stay on the skinny MMQ.
 //   3-4 rows  after the LDS-staged dot4 kernel has had its pick (narrow matrices and long contractions): ahead against
 //             14336 rows and more for Q5_K 1.03-1.18, Q8_0 0.99-1.17, IQ3_S 1.08-1.51, Q4_K 0.98-1.18; mixed for
 //             Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
-// Contractions whose rows do not fit the LDS (eight rows from in_dim 16384) keep the other kernels.
 bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    if (n_rows < 3 || n_rows > 8 || mvql_geometry(fmt, in_dim, out_dim, n_rows).lds > kLdsPerCu) return false;
+    if (n_rows < 3 || n_rows > 8) return false;
+    const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
+    if (g.lds == 0) return false;
     if (opt_is_set(O_QUAD_LDS)) return opt_u(O_QUAD_LDS, 0) != 0;
     if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
     if ((unsigned long long)in_dim * out_dim < (1ull << 24)) return false;
     if (n_rows >= 5) {
         if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS) return true;
-        return out_dim >= 8192 && out_dim <= 20480;
+        return out_dim >= 8192 && out_dim <= 20480 && g.phase_sub >= in_dim / 32;
     }
     return out_dim >= 14336 && (fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K);
 }
@@ -443,7 +462,7 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
 {
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
     const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
-    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub};
     return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
 }
 

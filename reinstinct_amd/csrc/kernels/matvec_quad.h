@@ -239,13 +239,19 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
 // quarter-wave pass covers 64 different banks.  Only the weights still take the trip through the
 // wavefront's private LDS image.  A trip requests the next trip's weights (or the first trip of the
 // wavefront's next row group) before it computes.  Same arithmetic in the same order as the kernel above.
+//
+// A contraction whose rows do not fit the LDS is staged in phases of `phase_sub` sub-blocks (a multiple
+// of 16): every wavefront then owns at most ONE row group (the launch has at least as many wavefronts as
+// row groups), keeps its partial sums in registers across the phases, and the workgroup re-stages between
+// two barriers that every wavefront reaches, with or without a row group.  phase_sub >= in_dim / 32 is the
+// single-phase form, in which wavefronts may stride over several row groups.
 // Launch: block = 64 x W threads (W <= 16), dynamic shared memory =
-//   4*NT * stride * 40 + W * kParts * 76 * 16 bytes, stride = n_sub + ((20 - n_sub % 16) % 16),
-// any grid (wavefronts stride over the row groups).
+//   4*NT * stride * 40 + W * kParts * 76 * 16 bytes, stride = n + ((20 - n % 16) % 16) for
+//   n = min(in_dim / 32, phase_sub).
 template <int FMT, int NT>
 __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
                                                           float* __restrict__ y, unsigned in_dim, unsigned out_dim,
-                                                          unsigned n_rows)
+                                                          unsigned n_rows, unsigned phase_sub)
 {
     using F = Fmt<FMT>;
     using Raw = typename F::Raw;
@@ -259,96 +265,91 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
     const unsigned put = lane + 4u * lr;
     const unsigned get = 16u * j + blk + 4u * j;
     const unsigned n_sub = in_dim >> 5;
-    // row stride of the activation planes: 4 mod 16 entries, so that the four activation rows of a
-    // quarter-wave pass (blocks 0..3, j = 0..3) read 64 different banks
-    const unsigned stride = n_sub + ((20u - (n_sub & 15u)) & 15u);
+    const unsigned n_stage = min(n_sub, phase_sub);                   // sub-blocks staged at a time
+    const unsigned stride = n_stage + ((20u - (n_stage & 15u)) & 15u);
     uint4* xlo = rein_mvql_lds;
     uint4* xhi = xlo + T * stride;
     uint2* xhd = reinterpret_cast<uint2*>(xhi + T * stride);
     uint4* stage = reinterpret_cast<uint4*>(xhd + T * stride) + wave * (kParts * 76u);
     const F fmt(w, n_sub, out_dim);
     const unsigned n_groups = (out_dim + 3u) / 4u;
+    const unsigned step = gridDim.x * wpb;
     const XSums no_xs = {0, 0};
 
-    unsigned g = blockIdx.x * wpb + wave;
+    // sub-blocks [first, first + count) of every activation row -> planes
+    auto stage_x = [&](unsigned first, unsigned count) {
+        for (unsigned e = threadIdx.x; e < T * count; e += blockDim.x) {
+            const unsigned t = e / count, sb = e - t * count;
+            const BlockQ8 v = xq[(size_t)min(t, n_rows - 1u) * n_sub + first + sb];
+            xlo[t * stride + sb] = make_uint4((unsigned)v.qs[0], (unsigned)v.qs[1], (unsigned)v.qs[2], (unsigned)v.qs[3]);
+            xhi[t * stride + sb] = make_uint4((unsigned)v.qs[4], (unsigned)v.qs[5], (unsigned)v.qs[6], (unsigned)v.qs[7]);
+            xhd[t * stride + sb] = make_uint2(__builtin_bit_cast(unsigned, v.d), __builtin_bit_cast(unsigned, v.xsum));
+        }
+    };
+
     Raw rq;
-    {
-        const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
-        rq = fmt.load(row, min(ls, n_sub - 1u));
-    }
-    for (unsigned e = threadIdx.x; e < T * n_sub; e += blockDim.x) {
-        const unsigned t = e / n_sub, sb = e - t * n_sub;
-        const BlockQ8 v = xq[(size_t)min(t, n_rows - 1u) * n_sub + sb];
-        xlo[t * stride + sb] = make_uint4((unsigned)v.qs[0], (unsigned)v.qs[1], (unsigned)v.qs[2], (unsigned)v.qs[3]);
-        xhi[t * stride + sb] = make_uint4((unsigned)v.qs[4], (unsigned)v.qs[5], (unsigned)v.qs[6], (unsigned)v.qs[7]);
-        xhd[t * stride + sb] = make_uint2(__builtin_bit_cast(unsigned, v.d), __builtin_bit_cast(unsigned, v.xsum));
-    }
-    __syncthreads();
-
-    for (; g < n_groups; g += gridDim.x * wpb) {
-        float acc[NT][4];
+    // one trip of row group g: 16 sub-blocks from sb0, whose activations sit at plane index x0 + block
+    auto trip = [&](unsigned g, unsigned sb0, unsigned x0, float (&acc)[NT][4]) {
+        const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(rq);
 #pragma unroll
-        for (int t = 0; t < NT; t++)
+        for (int i = 0; i < kParts; i++) stage[i * 76 + put] = bits.p[i];
+        // the load registers are free again: the next trip (of this row group, or the first of the wavefront's
+        // next one) is requested now, pinned between scheduling barriers as in the kernel above
+        __builtin_amdgcn_sched_barrier(0);
+        {
+            const bool last = sb0 + 16u >= n_sub;
+            const unsigned ng = last ? min(g + step, n_groups - 1u) : g;
+            const unsigned nrow = min(ng * 4u + lr, out_dim - 1u);
+            rq = fmt.load(nrow, min((last ? 0u : sb0 + 16u) + ls, n_sub - 1u));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        QuadRawBits<FMT> mine;
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
-
-        for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) {
-            const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(rq);
+        for (int i = 0; i < kParts; i++) mine.p[i] = stage[i * 76 + get];
+        Raw my;
+        __builtin_memcpy(&my, &mine, sizeof(my));
+        SubW sw;
+        F::unpack(my, sw);
+        const bool live = sb0 + blk < n_sub;
+        const unsigned sbx = x0 + min(blk, n_sub - 1u - sb0);
+        int a[8];
 #pragma unroll
-            for (int i = 0; i < kParts; i++) stage[i * 76 + put] = bits.p[i];
-            __builtin_amdgcn_sched_barrier(0);
-            {
-                const bool last = sb0 + 16u >= n_sub;
-                const unsigned ng = last ? min(g + gridDim.x * wpb, n_groups - 1u) : g;
-                const unsigned nrow = min(ng * 4u + lr, out_dim - 1u);
-                rq = fmt.load(nrow, min((last ? 0u : sb0 + 16u) + ls, n_sub - 1u));
+        for (int k = 0; k < 8; k++) a[k] = rein_fold_offset<FMT>(sw.w[k]);
+        float s0[4], s1[4];
+        s0[0] = rein_quad_bcast<0>(sw.s0); s0[1] = rein_quad_bcast<1>(sw.s0);
+        s0[2] = rein_quad_bcast<2>(sw.s0); s0[3] = rein_quad_bcast<3>(sw.s0);
+        s1[0] = rein_quad_bcast<0>(sw.s1); s1[1] = rein_quad_bcast<1>(sw.s1);
+        s1[2] = rein_quad_bcast<2>(sw.s1); s1[3] = rein_quad_bcast<3>(sw.s1);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const unsigned at = (4u * t + j) * stride + sbx;
+            const uint4 lo = xlo[at], hi = xhi[at];
+            const uint2 hd = xhd[at];
+            const bool on = live && 4u * t + j < n_rows;
+            const float dx = on ? __builtin_bit_cast(float, hd.x) : 0.0f;
+            const float xsum = on ? __builtin_bit_cast(float, hd.y) : 0.0f;
+            const int q[8] = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+            rein_quad_v4i d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < 4; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
+            if (kTwo) {
+#pragma unroll
+                for (int k = 4; k < 8; k++) d1 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d1, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int k = 4; k < 8; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            QuadRawBits<FMT> mine;
 #pragma unroll
-            for (int i = 0; i < kParts; i++) mine.p[i] = stage[i * 76 + get];
-            Raw my;
-            __builtin_memcpy(&my, &mine, sizeof(my));
-            SubW sw;
-            F::unpack(my, sw);
-            const bool live = sb0 + blk < n_sub;
-            const unsigned sbx = min(sb0 + blk, n_sub - 1u);
-            int a[8];
-#pragma unroll
-            for (int k = 0; k < 8; k++) a[k] = rein_fold_offset<FMT>(sw.w[k]);
-            float s0[4], s1[4];
-            s0[0] = rein_quad_bcast<0>(sw.s0); s0[1] = rein_quad_bcast<1>(sw.s0);
-            s0[2] = rein_quad_bcast<2>(sw.s0); s0[3] = rein_quad_bcast<3>(sw.s0);
-            s1[0] = rein_quad_bcast<0>(sw.s1); s1[1] = rein_quad_bcast<1>(sw.s1);
-            s1[2] = rein_quad_bcast<2>(sw.s1); s1[3] = rein_quad_bcast<3>(sw.s1);
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                const unsigned at = (4u * t + j) * stride + sbx;
-                const uint4 lo = xlo[at], hi = xhi[at];
-                const uint2 hd = xhd[at];
-                const bool on = live && 4u * t + j < n_rows;
-                const float dx = on ? __builtin_bit_cast(float, hd.x) : 0.0f;
-                const float xsum = on ? __builtin_bit_cast(float, hd.y) : 0.0f;
-                const int q[8] = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-                rein_quad_v4i d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};
-#pragma unroll
-                for (int k = 0; k < 4; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
-                if (kTwo) {
-#pragma unroll
-                    for (int k = 4; k < 8; k++) d1 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d1, 0, 0, 0);
-                } else {
-#pragma unroll
-                    for (int k = 4; k < 8; k++) d0 = __builtin_amdgcn_mfma_i32_4x4x4i8(a[k], q[k], d0, 0, 0, 0);
-                }
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    SubW sc;
-                    sc.s0 = s0[r];
-                    sc.s1 = s1[r];
-                    acc[t][r] += F::term(sc, d0[r], d1[r], dx, xsum, no_xs);
-                }
+            for (int r = 0; r < 4; r++) {
+                SubW sc;
+                sc.s0 = s0[r];
+                sc.s1 = s1[r];
+                acc[t][r] += F::term(sc, d0[r], d1[r], dx, xsum, no_xs);
             }
         }
+    };
+    // sum over the 16 blocks (lane bits 2..5); lanes 0..3 (block 0) store
+    auto finish = [&](unsigned g, float (&acc)[NT][4]) {
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -361,14 +362,48 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
                 const unsigned tok = 4u * t + j, orow = g * 4u + r;
                 if (blk == 0u && tok < n_rows && orow < out_dim) y[(size_t)tok * out_dim + orow] = v;
             }
+    };
+
+    unsigned g = blockIdx.x * wpb + wave;
+    {   // the first trip's weights are on their way while the activations are staged
+        const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
+        rq = fmt.load(row, min(ls, n_sub - 1u));
+    }
+    float acc[NT][4];
+    if (phase_sub >= n_sub) {
+        stage_x(0u, n_sub);
+        __syncthreads();
+        for (; g < n_groups; g += step) {
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+            for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) trip(g, sb0, sb0, acc);
+            finish(g, acc);
+        }
+    } else {
+        const bool has = g < n_groups;                 // wave-uniform
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+        for (unsigned ph0 = 0; ph0 < n_sub; ph0 += phase_sub) {
+            const unsigned count = min(phase_sub, n_sub - ph0);
+            if (ph0 != 0u) __syncthreads();            // every wavefront is done with the previous phase's planes
+            stage_x(ph0, count);
+            __syncthreads();
+            if (has)
+                for (unsigned sb0 = ph0; sb0 < ph0 + count; sb0 += 16u) trip(g, sb0, sb0 - ph0, acc);
+        }
+        if (has) finish(g, acc);
     }
 }
 
-// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows), n_rows <= 4 * NT
+// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub), n_rows <= 4 * NT
 #define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT)                                                \
     extern "C" __global__ __launch_bounds__(1024) void name(                                      \
         const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y,    \
-        unsigned int in_dim, unsigned int out_dim, unsigned int n_rows)                           \
+        unsigned int in_dim, unsigned int out_dim, unsigned int n_rows, unsigned int phase_sub)   \
     {                                                                                             \
-        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows);                    \
+        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows, phase_sub);         \
     }
