@@ -139,8 +139,8 @@ int check_ptr(const char* who, const void* p, size_t align, const char* what)
 // rein_set_option changes an entry, so the launch an entry point chooses depends on its arguments
 // and on this table alone.  Entries are single atomic words: setting one while another thread
 // launches is safe, the launch sees the old or the new value.
-enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
-const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
+enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_QUAD_SLICES, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
+const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_QUAD_SLICES", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
 constexpr uint64_t kOptSet = 1ull << 63;
 std::atomic<uint64_t> g_opts[O_COUNT];          // zero = unset
 std::once_flag g_opts_env_once;
@@ -375,7 +375,12 @@ bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
     if (opt_is_set(O_MV_LDS)) return opt_u(O_MV_LDS, 0) != 0;
     if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
-    if (n_rows >= 3) return weights >= (1ull << 24) && (out_dim <= 6144 || in_dim >= 8192);
+    if (n_rows >= 3) {
+        // (up to 8192 rows and from 20 * 2^20 weights the 4x4x4 kernel with its contraction sliced over wavefronts is
+        // ahead of this one for every format but Q8_0 -- use_mvql)
+        if (fmt != REIN_TYPE_Q8_0 && out_dim <= 8192 && weights >= (20ull << 20) && opt_u(O_QUAD_LDS, 1) != 0) return false;
+        return weights >= (1ull << 24) && (out_dim <= 6144 || in_dim >= 8192);
+    }
     if (weights < (1ull << 25)) return false;
     if (in_dim >= 8192) return true;
     return out_dim >= 14336 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S);
@@ -397,19 +402,33 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
 // per wavefront or persistent wavefronts (Q4_K, Q6_K, Q5_K, Q8_0 on six shapes): up to 16384 rows 256
 // workgroups with one group of four rows per wavefront (5120 rows: five wavefronts, 14336: fourteen); beyond,
 // 512 workgroups of eight wavefronts that stride over the row groups.
-struct QuadLdsGeometry { unsigned wpb, grid, phase_sub; size_t lds; };       // lds == 0: no launch fits
+struct QuadLdsGeometry { unsigned wpb, grid, phase_sub, slices; size_t lds; };       // lds == 0: no launch fits
 QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : 8;
     const unsigned parts = fmt == REIN_TYPE_Q8_0 ? 3 : 2;               // 16-byte parts of Fmt<FMT>::Raw
     const unsigned groups = (out_dim + 3) / 4;
     QuadLdsGeometry g;
-    g.wpb = std::min(16u, (groups + kCUs - 1) / kCUs);
-    g.grid = (groups + g.wpb - 1) / g.wpb;
+    g.slices = 1;
+    unsigned gpb = std::min(16u, (groups + kCUs - 1) / kCUs);          // row groups per workgroup
     const bool persistent = groups > kCUs * 16;
-    if (persistent) { g.wpb = 8; g.grid = 2 * kCUs; }
     const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
-    if (wpb_forced >= 1 && wpb_forced <= 16) { g.wpb = wpb_forced; g.grid = (groups + g.wpb - 1) / g.wpb; }
+    if (wpb_forced >= 1 && wpb_forced <= 16) gpb = wpb_forced;
+    if (persistent && !(wpb_forced >= 1 && wpb_forced <= 16)) { g.wpb = 8; g.grid = 2 * kCUs; }
+    else {
+        // few row groups per CU: several wavefronts share a row group, each taking every slices-th trip
+        // (us, Q4_K at 8 rows, slices 1 / 2 / 3-4: 17408 -> 5120 28.7 / 21.1 / 19.9, 14336 -> 4096 22.5 / 16.1 / 14.6,
+        // 5120 -> 5120 10.5 / 8.8 / 9.0, 8192 -> 8192 16.8 / 15.1, 5120 -> 1024 12.0 / 8.4 / 6.9: one trip in flight per
+        // wavefront and five wavefronts per CU is a latency-bound launch): as many slices as give a workgroup 16
+        // wavefronts, each with two trips at least
+        const unsigned want = opt_u(O_QUAD_SLICES, 0);
+        const unsigned trips = (n_sub + 15) / 16;
+        g.slices = want >= 1 && want <= 8 ? want : std::min(8u, std::max(1u, trips / 2));
+        g.slices = std::max(1u, std::min(g.slices, 16u / gpb));
+        g.slices = std::min(g.slices, std::max(1u, trips));
+        g.wpb = gpb * g.slices;
+        g.grid = (groups + gpb - 1) / gpb;
+    }
     const auto bytes = [&](unsigned n_stage) {
         const unsigned stride = n_stage + ((20u - (n_stage & 15u)) & 15u);
         return (size_t)t * stride * 40 + (size_t)g.wpb * parts * 76 * 16;
@@ -418,30 +437,35 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
     g.lds = bytes(n_sub);
     if (g.lds > kLdsPerCu) {
         // The rows do not fit: stage the contraction in phases.  That form keeps a wavefront's partial sums in
-        // registers across the phases, so it needs one row group per wavefront at most.
+        // registers across the phases, so it needs one row group per wavefront at most; a phase is a whole number
+        // of rounds of the slices' trips.
         g.lds = 0;
-        if ((unsigned long long)g.grid * g.wpb >= groups)
+        const unsigned round = 16u * g.slices;
+        if (!persistent || (unsigned long long)g.grid * g.wpb >= groups)
             for (unsigned phases = 2; phases <= 8 && g.lds == 0; phases++) {
-                const unsigned per = (((n_sub + phases - 1) / phases) + 15u) & ~15u;
+                const unsigned per = (((n_sub + phases - 1) / phases) + round - 1) / round * round;
                 if (bytes(per) <= kLdsPerCu) { g.phase_sub = per; g.lds = bytes(per); }
             }
     }
     return g;
 }
 
-// Whether a batched decode of 3..8 rows runs on it.  One run of the library's other choice against this kernel, seven
-// formats x 16 shapes x 3 / 4 / 5 / 6 / 8 rows (ratio of the two times), from 2^24 weights (below, 0.52-0.99):
-//   5-8 rows  Q6_K, Q5_K, IQ4_XS (the formats of the 4x4x4 kernel): level or ahead everywhere -- 5120 -> 5120 1.05-1.18,
-//             5120 -> 34816 1.02-1.25, 4096 -> 14336 1.31-1.47, 8192 -> 8192 1.04-1.16, 2048 -> 16384 1.30-1.45,
-//             14336 -> 4096 1.01-1.15.  Q4_K, Q8_0, Q4_0, IQ3_S (skinny MMQ otherwise): ahead between 8192 and 20480
-//             rows (8192 -> 8192 1.11-1.23, 4096 -> 14336 1.21-1.36, 5120 -> 17408 1.05-1.16, 2048 -> 16384 1.20-1.35),
-//             behind or level outside (5120 -> 5120 0.96-1.02, 14336 -> 4096 0.84-0.95, 5120 -> 34816 0.95-1.08,
-//             8192 -> 28672 0.92-1.20).  Contractions staged in phases (eight rows from in_dim 16384): Q6_K 1.05-1.14,
-//             Q5_K 1.00-1.11, IQ4_XS 0.99-1.08 on 17408 -> 5120, 14336 -> 4096, 28672 -> 8192, 18944 -> 3584; the
-//             other formats 0.71-0.98 there and stay on the skinny MMQ.
-//   3-4 rows  after the LDS-staged dot4 kernel has had its pick (narrow matrices and long contractions): ahead against
-//             14336 rows and more for Q5_K 1.03-1.18, Q8_0 0.99-1.17, IQ3_S 1.08-1.51, Q4_K 0.98-1.18; mixed for
-//             Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
+// Whether a batched decode of 3..8 rows runs on it.  Runs of the library's other choice against this kernel, seven
+// formats x 16 shapes x 3 / 4 / 5 / 6 / 8 rows (ratio of the two times):
+//   5-8 rows  Q6_K, Q5_K, IQ4_XS (the formats of the 4x4x4 kernel): level or ahead everywhere from 5 * 2^20 weights --
+//             5120 -> 5120 1.05-1.18 (1.15-1.37 with slices), 5120 -> 34816 1.02-1.25, 4096 -> 14336 1.31-1.47, 8192 -> 8192
+//             1.04-1.16, 2048 -> 16384 1.30-1.45, 17408 -> 5120 1.39-1.40, 18944 -> 3584 1.47-1.57, 5120 -> 1024 1.0-1.47.
+//             Q4_K, Q8_0, Q4_0, IQ3_S (skinny MMQ otherwise): ahead up to 20480 rows -- 17408 -> 5120 1.21-1.37, 14336 ->
+//             4096 1.25-1.46, 18944 -> 3584 1.27-1.50, 5120 -> 5120 1.12-1.16, 4096 -> 4096 1.12-1.35, 5120 -> 1024
+//             1.20-1.51, 8192 -> 8192 1.00-1.23, 4096 -> 14336 1.21-1.36, 2048 -> 16384 1.20-1.35 -- except where the rows
+//             need phases against more than 6144 rows (28672 -> 8192 0.88-1.06); behind or level beyond 20480 rows
+//             (5120 -> 34816 0.95-1.08, 8192 -> 28672 0.92-1.20).
+//   3-4 rows  up to 8192 rows and from 20 * 2^20 weights ahead of the LDS-staged dot4 kernel for every format but Q8_0
+//             (0.95-1.02): Q4_K 5120 -> 5120 1.05-1.08, 17408 -> 5120 1.24-1.26, 14336 -> 4096 1.09, 28672 -> 8192
+//             1.15-1.18, 18944 -> 3584 1.17, 5120 -> 7168 1.18-1.20, 8192 -> 8192 0.96; Q4_0 1.08-1.33; Q6_K 1.07-1.22;
+//             Q5_K 1.05-1.27; IQ4_XS 1.01-1.17; IQ3_S 0.99-1.21; 4096 -> 4096 (2^24 weights) 0.86-0.97 and stays.
+//             Against 14336 rows and more, where neither of those applies: Q5_K 1.03-1.18, Q8_0 0.99-1.17, IQ3_S
+//             1.08-1.51, Q4_K 0.98-1.18; mixed for Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
 bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     if (n_rows < 3 || n_rows > 8) return false;
@@ -449,11 +473,15 @@ bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
     if (g.lds == 0) return false;
     if (opt_is_set(O_QUAD_LDS)) return opt_u(O_QUAD_LDS, 0) != 0;
     if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
-    if ((unsigned long long)in_dim * out_dim < (1ull << 24)) return false;
+    const unsigned long long weights = (unsigned long long)in_dim * out_dim;
     if (n_rows >= 5) {
+        if (weights < (5ull << 20)) return false;
         if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS) return true;
-        return out_dim >= 8192 && out_dim <= 20480 && g.phase_sub >= in_dim / 32;
+        const bool phased = g.phase_sub < in_dim / 32;
+        return out_dim <= 20480 && !(phased && out_dim > 6144);
     }
+    if (fmt != REIN_TYPE_Q8_0 && out_dim <= 8192 && weights >= (20ull << 20)) return true;
+    if (weights < (1ull << 24)) return false;
     return out_dim >= 14336 && (fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K);
 }
 
@@ -462,7 +490,7 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
 {
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
     const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
-    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub};
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub, (void*)&g.slices};
     return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
 }
 
@@ -475,6 +503,9 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    // (an option that forces one LDS-staged family on goes first)
+    const bool mvql_forced = opt_u(O_QUAD_LDS, 0) != 0 && opt_u(O_MV_LDS, 0) == 0;
+    if (mvql_forced && use_mvql(fmt, in_dim, out_dim, n_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     if (use_mvl(fmt, in_dim, out_dim, n_rows)) return launch_matvec_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     if (use_mvql(fmt, in_dim, out_dim, n_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const bool small = small_for_matrix_cores(fmt, in_dim, out_dim, n_rows);

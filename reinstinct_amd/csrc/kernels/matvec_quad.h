@@ -251,13 +251,14 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
 template <int FMT, int NT>
 __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
                                                           float* __restrict__ y, unsigned in_dim, unsigned out_dim,
-                                                          unsigned n_rows, unsigned phase_sub)
+                                                          unsigned n_rows, unsigned phase_sub, unsigned slices)
 {
     using F = Fmt<FMT>;
     using Raw = typename F::Raw;
     constexpr bool kTwo = F::kDotParts == 2;
     constexpr int kParts = QuadRawBits<FMT>::kParts;
     constexpr unsigned T = 4u * NT;
+    static_assert(kParts * 76 * 16 >= NT * 16 * 4, "a wavefront's partial sums go through its weight image");
     extern __shared__ uint4 rein_mvql_lds[];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wpb = blockDim.x >> 6;
     const unsigned j = lane & 3u, blk = lane >> 2;
@@ -288,8 +289,9 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
     };
 
     Raw rq;
-    // one trip of row group g: 16 sub-blocks from sb0, whose activations sit at plane index x0 + block
-    auto trip = [&](unsigned g, unsigned sb0, unsigned x0, float (&acc)[NT][4]) {
+    // one trip of row group g: 16 sub-blocks from sb0, whose activations sit at plane index x0 + block; the
+    // wavefront's next trip starts `ahead` sub-blocks further on
+    auto trip = [&](unsigned g, unsigned sb0, unsigned x0, unsigned ahead, float (&acc)[NT][4]) {
         const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(rq);
 #pragma unroll
         for (int i = 0; i < kParts; i++) stage[i * 76 + put] = bits.p[i];
@@ -297,10 +299,10 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
         // next one) is requested now, pinned between scheduling barriers as in the kernel above
         __builtin_amdgcn_sched_barrier(0);
         {
-            const bool last = sb0 + 16u >= n_sub;
+            const bool last = sb0 + ahead >= n_sub;
             const unsigned ng = last ? min(g + step, n_groups - 1u) : g;
             const unsigned nrow = min(ng * 4u + lr, out_dim - 1u);
-            rq = fmt.load(nrow, min((last ? 0u : sb0 + 16u) + ls, n_sub - 1u));
+            rq = fmt.load(nrow, min((last ? 0u : sb0 + ahead) + ls, n_sub - 1u));
         }
         __builtin_amdgcn_sched_barrier(0);
         QuadRawBits<FMT> mine;
@@ -364,46 +366,82 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
             }
     };
 
-    unsigned g = blockIdx.x * wpb + wave;
-    {   // the first trip's weights are on their way while the activations are staged
-        const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
-        rq = fmt.load(row, min(ls, n_sub - 1u));
-    }
     float acc[NT][4];
-    if (phase_sub >= n_sub) {
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+    if (phase_sub >= n_sub && slices <= 1u) {
+        unsigned g = blockIdx.x * wpb + wave;
+        {   // the first trip's weights are on their way while the activations are staged
+            const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
+            rq = fmt.load(row, min(ls, n_sub - 1u));
+        }
         stage_x(0u, n_sub);
         __syncthreads();
         for (; g < n_groups; g += step) {
+            for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) trip(g, sb0, sb0, 16u, acc);
+            finish(g, acc);
 #pragma unroll
             for (int t = 0; t < NT; t++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
-            for (unsigned sb0 = 0; sb0 < n_sub; sb0 += 16u) trip(g, sb0, sb0, acc);
-            finish(g, acc);
         }
     } else {
-        const bool has = g < n_groups;                 // wave-uniform
-#pragma unroll
-        for (int t = 0; t < NT; t++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+        // one (row group, slice) per wavefront: wavefront w of the workgroup takes row group w / slices and every
+        // slices-th trip of it, from trip w % slices on
+        const unsigned gpb = wpb / slices;                       // row groups per workgroup
+        const unsigned slice = wave % slices;
+        const unsigned g = blockIdx.x * gpb + wave / slices;
+        const bool has = wave < gpb * slices && g < n_groups;    // wave-uniform
+        const unsigned ahead = 16u * slices;
+        {
+            const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
+            rq = fmt.load(row, min(16u * slice + ls, n_sub - 1u));
+        }
         for (unsigned ph0 = 0; ph0 < n_sub; ph0 += phase_sub) {
             const unsigned count = min(phase_sub, n_sub - ph0);
             if (ph0 != 0u) __syncthreads();            // every wavefront is done with the previous phase's planes
             stage_x(ph0, count);
             __syncthreads();
             if (has)
-                for (unsigned sb0 = ph0; sb0 < ph0 + count; sb0 += 16u) trip(g, sb0, sb0 - ph0, acc);
+                for (unsigned sb0 = ph0 + 16u * slice; sb0 < ph0 + count; sb0 += ahead) trip(g, sb0, sb0 - ph0, ahead, acc);
         }
-        if (has) finish(g, acc);
+        if (slices <= 1u) {
+            if (has) finish(g, acc);
+        } else {
+            // The slices' partial sums meet in LDS (each wavefront's weight image has room for its 16 x NT
+            // values) and are added in slice order by the first slice's wavefront: the result does not depend on timing.
+            float* part = reinterpret_cast<float*>(stage);
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float v = acc[t][r];
+                    v += __shfl_xor(v, 4);
+                    v += __shfl_xor(v, 8);
+                    v += __shfl_xor(v, 16);
+                    v += __shfl_xor(v, 32);
+                    if (blk == 0u) part[(t * 4 + r) * 4 + j] = v;
+                }
+            __syncthreads();
+            if (has && slice == 0u && lane < 16u * NT) {
+                float v = part[lane];
+                for (unsigned k = 1; k < slices; k++) v += part[k * (kParts * 76u * 4u) + lane];
+                const unsigned t = lane >> 4, r = (lane >> 2) & 3u, jj = lane & 3u;
+                const unsigned tok = 4u * t + jj, orow = g * 4u + r;
+                if (tok < n_rows && orow < out_dim) y[(size_t)tok * out_dim + orow] = v;
+            }
+        }
     }
 }
 
-// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub), n_rows <= 4 * NT
+// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub, slices), n_rows <= 4 * NT
 #define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT)                                                \
     extern "C" __global__ __launch_bounds__(1024) void name(                                      \
         const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y,    \
-        unsigned int in_dim, unsigned int out_dim, unsigned int n_rows, unsigned int phase_sub)   \
+        unsigned int in_dim, unsigned int out_dim, unsigned int n_rows, unsigned int phase_sub,   \
+        unsigned int slices)                                                                      \
     {                                                                                             \
-        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows, phase_sub);         \
+        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows, phase_sub, slices); \
     }

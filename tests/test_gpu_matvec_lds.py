@@ -113,19 +113,17 @@ def test_lds_matvec_largest_contraction_and_fallback_beyond_it(options):
         assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, 4), what=f"K {in_dim}")
 
 
-@pytest.mark.parametrize("fmt,n_rows", [(rein.Q4_K, 3), (rein.Q6_K, 4), (rein.Q8_0, 3), (rein.IQ4_XS, 4)])
-def test_default_dispatch_takes_the_lds_kernel_for_narrow_matrices(fmt, n_rows, options):
-    # 3-4 rows, at most 6144 output rows, from 2^24 weights: the library's own choice -- the same bits as forced
-    in_dim, out_dim = 5120, 4100
+@pytest.mark.parametrize("fmt,in_dim,out_dim,n_rows", [(rein.Q4_K, 4096, 4100, 3), (rein.Q6_K, 4096, 4100, 4), (rein.Q8_0, 5120, 4100, 3),
+                                                      (rein.Q8_0, 5120, 4100, 4), (rein.IQ4_XS, 4096, 4100, 4), (rein.Q5_K, 8192, 8200, 2)])
+def test_default_dispatch_takes_the_lds_kernel(fmt, in_dim, out_dim, n_rows, options):
+    # 3-4 rows, at most 6144 output rows, from 2^24 weights (Q8_0 at any size, the others up to 20 * 2^20 weights, beyond
+    # which the sliced 4x4x4 kernel takes over); 2 rows at contractions of 8192 and more: the same bits as forced
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
     got = run(fmt, packed, xq, in_dim, out_dim, n_rows)
     assert_close_f32(got, orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows), what="default dispatch")
     assert np.array_equal(bits(got), bits(run_lds(options, fmt, packed, xq, in_dim, out_dim, n_rows)))
-    # five rows and more stay with the matrix-core families
-    xq8 = orc.quantize_q8(np.random.default_rng(8).standard_normal((8, in_dim)).astype(np.float32))
-    assert_close_f32(run(fmt, packed, xq8, in_dim, out_dim, 8), orc.matvec_q8(fmt, packed, in_dim, out_dim, xq8, 8), what="8 rows")
 
 
 # ---- the 4x4x4 matrix-instruction form --------------------------------------------------------------
@@ -139,21 +137,27 @@ def run_opts(options, pairs, fmt, packed, xq, in_dim, out_dim, n_rows):
     return got
 
 
-def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0):
+def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0, slices="1"):
+    """slices: wavefronts that share a row group, each taking every slices-th trip of the contraction (None: the
+    library's own number).  One slice repeats the 4x4x4 family's arithmetic in its order; several add their partial
+    sums in slice order, which is another -- fixed -- order of the same terms."""
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + in_dim + seed)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    forced = [("REIN_QUAD_LDS", "1"), ("REIN_MV_LDS", "0")] + ([("REIN_QUAD_SLICES", slices)] if slices else [])
     for n_rows in rows:
-        print("lds quad", fmt, in_dim, out_dim, n_rows, flush=True)
+        print("lds quad", fmt, in_dim, out_dim, n_rows, "slices", slices, flush=True)
         xq = orc.quantize_q8(np.random.default_rng(n_rows + seed).standard_normal((n_rows, in_dim)).astype(np.float32))
-        got = run_opts(options, [("REIN_QUAD_LDS", "1"), ("REIN_MV_LDS", "0")], fmt, packed, xq, in_dim, out_dim, n_rows)
+        got = run_opts(options, forced, fmt, packed, xq, in_dim, out_dim, n_rows)
         want = orc.matvec_q8(fmt, packed, in_dim, out_dim, xq, n_rows)
-        assert_close_f32(got, want, what=f"lds quad fmt {fmt} {in_dim}->{out_dim} rows {n_rows}")
+        assert_close_f32(got, want, what=f"lds quad fmt {fmt} {in_dim}->{out_dim} rows {n_rows} slices {slices}")
+        again = run_opts(options, forced, fmt, packed, xq, in_dim, out_dim, n_rows)
+        assert np.array_equal(bits(got), bits(again)), "two runs of the same launch differ"
         same = run_opts(options, [("REIN_QUAD_FROM", "1"), ("REIN_QUAD_LDS", "0"), ("REIN_MV_LDS", "0")], fmt, packed, xq,
                         in_dim, out_dim, n_rows)
-        # the same operations in the same order; where the compiler contracts a format's two-product term differently in
-        # the two kernels (Q6_K) the last bits differ
-        assert np.allclose(got, same, rtol=0.0, atol=2e-6 * float(np.abs(same).max())), f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
-        if fmt != rein.Q6_K:
+        assert np.allclose(got, same, rtol=0.0, atol=4e-6 * float(np.abs(same).max())), f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
+        # one slice: the same operations in the same order; where the compiler contracts a format's two-product term
+        # differently in the two kernels (Q6_K) the last bits differ
+        if slices == "1" and fmt != rein.Q6_K:
             assert np.array_equal(bits(got), bits(same)), f"not the 4x4x4 family's bits: fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
 
 
@@ -161,6 +165,13 @@ def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0):
 @pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (256, 64), (5120, 130), (4096, 33), (2304, 4099)])
 def test_lds_quad_parity(fmt, in_dim, out_dim, options):
     check_quad_lds(options, fmt, in_dim, out_dim)
+
+
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (5120, 130), (2304, 4099), (7168, 1030)])
+@pytest.mark.parametrize("slices", [None, "2", "3", "8"])
+def test_lds_quad_contraction_sliced_over_wavefronts(fmt, in_dim, out_dim, slices, options):
+    check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 4, 5, 8), slices=slices)
 
 
 @pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])
@@ -188,14 +199,18 @@ def test_lds_quad_long_contractions_are_staged_in_phases(fmt, options):
     # registers in between; 32768 values: three phases; a ragged count of row groups leaves wavefronts without one
     for in_dim, out_dim, rows in ((17408, 70, (5, 8)), (32768, 21, (8,)), (16384, 130, (4, 7))):
         check_quad_lds(options, fmt, in_dim, out_dim, rows=rows, seed=1)
+    # phases and slices together: a phase is a whole number of rounds of the slices' trips
+    for slices in (None, "3", "5"):
+        check_quad_lds(options, fmt, 17408, 70, rows=(8,), seed=2, slices=slices)
 
 
 @pytest.mark.parametrize("fmt,in_dim,out_dim,n_rows", [(rein.Q6_K, 5120, 4100, 8), (rein.IQ4_XS, 5120, 4100, 6),
                                                       (rein.Q4_K, 2048, 8200, 5), (rein.Q8_0, 1024, 16388, 8),
-                                                      (rein.Q5_K, 1280, 14340, 3)])
+                                                      (rein.Q5_K, 1280, 14340, 3), (rein.Q4_K, 5120, 4100, 4),
+                                                      (rein.Q4_0, 5120, 1030, 7), (rein.IQ3_S, 17408, 1300, 8)])
 def test_default_dispatch_takes_the_lds_quad_kernel(fmt, in_dim, out_dim, n_rows, options):
-    # 5-8 rows: Q6_K / Q5_K / IQ4_XS everywhere, the other formats between 8192 and 20480 rows; 3-4 rows: Q5_K,
-    # Q8_0, IQ3_S and Q4_K against 14336 rows and more (from 2^24 weights)
+    # 5-8 rows: Q6_K / Q5_K / IQ4_XS everywhere, the other formats up to 20480 rows (from 5 * 2^20 weights); 3-4 rows:
+    # every format but Q8_0 up to 8192 rows from 20 * 2^20 weights, and Q5_K, Q8_0, IQ3_S, Q4_K against 14336 rows and more
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))

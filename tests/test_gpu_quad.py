@@ -67,10 +67,10 @@ def test_quad_matvec_ragged_contraction(fmt, in_dim, options):
 
 @pytest.mark.parametrize("fmt,n_rows", [(rein.Q6_K, 3), (rein.Q6_K, 4), (rein.Q5_K, 4), (rein.IQ4_XS, 3)])
 def test_default_dispatch_at_benchmark_width(fmt, n_rows, options):
-    # the row counts the library sends to these kernels by itself, at the K of the decode shapes (a matrix
-    # large enough that the library does not keep it on dot4, and with more than 6144 rows, below which 3-4
-    # rows go to the LDS-staged dot4 kernel; five rows and more go to the LDS-staged form of these kernels)
-    in_dim, out_dim = 5120, 6404
+    # the row counts the library sends to these kernels by itself: 3-4 rows against more than 8192 and fewer than
+    # 14336 rows from 2^24 weights (narrower matrices and longer contractions go to the LDS-staged kernels, as do five
+    # rows and more)
+    in_dim, out_dim = 2048, 9004
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
