@@ -405,7 +405,7 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
 struct QuadLdsGeometry { unsigned wpb, grid, phase_sub, slices; size_t lds; };       // lds == 0: no launch fits
 QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : 8;
+    const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : n_rows <= 8 ? 8 : 16;
     const unsigned parts = fmt == REIN_TYPE_Q8_0 ? 3 : 2;               // 16-byte parts of Fmt<FMT>::Raw
     const unsigned groups = (out_dim + 3) / 4;
     QuadLdsGeometry g;
@@ -450,7 +450,7 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
     return g;
 }
 
-// Whether a batched decode of 3..8 rows runs on it.  Runs of the library's other choice against this kernel, seven
+// Whether a batched decode of 3..16 rows runs on it.  Runs of the library's other choice against this kernel, seven
 // formats x 16 shapes x 3 / 4 / 5 / 6 / 8 rows (ratio of the two times):
 //   5-8 rows  Q6_K, Q5_K, IQ4_XS (the formats of the 4x4x4 kernel): level or ahead everywhere from 5 * 2^20 weights --
 //             5120 -> 5120 1.05-1.18 (1.15-1.37 with slices), 5120 -> 34816 1.02-1.25, 4096 -> 14336 1.31-1.47, 8192 -> 8192
@@ -468,12 +468,24 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
 //             1.08-1.51, Q4_K 0.98-1.18; mixed for Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
 bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    if (n_rows < 3 || n_rows > 8) return false;
+    if (n_rows < 3 || n_rows > 16) return false;
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
     if (g.lds == 0) return false;
     if (opt_is_set(O_QUAD_LDS)) return opt_u(O_QUAD_LDS, 0) != 0;
     if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
+    if (n_rows > 8) {
+        // 9-16 rows (rein_mmq_xq8 sends them here), against the skinny MMQ at 12 and 16 rows: Q6_K and Q5_K ahead on
+        // narrow and on short-and-mid matrices (5120 -> 5120 1.27 / 1.13, 17408 -> 5120 1.29 / 1.17, 14336 -> 4096 1.30 /
+        // 1.19, 18944 -> 3584 1.32 / 1.20, 4096 -> 14336 1.15, 2048 -> 16384 1.32 / 1.12, 8192 -> 8192 1.04-1.10, 5120 ->
+        // 1024 1.9 / 1.6), the other formats by 1.00-1.22 against at most 4096 rows with a long contraction and 1.28-1.42
+        // at 5120 -> 1024; everything behind against many rows (5120 -> 34816 0.72-0.93, 5120 -> 17408 0.69-0.85,
+        // 28672 -> 8192 0.69-0.92, 5120 -> 7168 0.83-1.01)
+        if (weights < (1ull << 22)) return false;
+        if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K)
+            return out_dim <= 6144 || (in_dim <= 4096 && out_dim <= 16384) || (in_dim <= 8192 && out_dim <= 8192);
+        return weights >= (5ull << 20) && out_dim <= 4096 && (in_dim >= 14336 || out_dim <= 1536);
+    }
     if (n_rows >= 5) {
         if (weights < (5ull << 20)) return false;
         if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS) return true;
@@ -489,7 +501,7 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
                     unsigned n_rows, rein_stream_t s)
 {
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
-    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
+    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : "_t16");
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub, (void*)&g.slices};
     return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
 }
@@ -940,6 +952,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
+    if (p_rows > 8 && p_rows <= 16 && use_mvql(fmt, in_dim, out_dim, p_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // Token tiles: 32 tokens (rein_mmq_<fmt>_t32, three workgroups per CU) or the mixed launch
     // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).

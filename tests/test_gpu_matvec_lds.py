@@ -34,7 +34,10 @@ def bits(a):
 def run(fmt, packed, xq, in_dim, out_dim, n_rows):
     dw, dq = dev(packed), dev(xq)
     dy = dev(np.full(n_rows * out_dim, np.nan, np.float32))
-    runtime.matvec_batched_xq8(fmt, dw, dq, dy, in_dim, out_dim, n_rows)
+    if n_rows <= 8:
+        runtime.matvec_batched_xq8(fmt, dw, dq, dy, in_dim, out_dim, n_rows)
+    else:
+        runtime.mmq_xq8(fmt, dw, dq, dy, in_dim, out_dim, n_rows)           # 9..16 rows arrive through this entry point
     hip.synchronize()
     return dy.to_host(np.float32).reshape(n_rows, out_dim)
 
@@ -157,7 +160,8 @@ def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0, slic
         assert np.allclose(got, same, rtol=0.0, atol=4e-6 * float(np.abs(same).max())), f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
         # one slice: the same operations in the same order; where the compiler contracts a format's two-product term
         # differently in the two kernels (Q6_K) the last bits differ
-        if slices == "1" and fmt != rein.Q6_K:
+        # (nine rows and more have no other 4x4x4 kernel: the comparison launch is the skinny MMQ)
+        if slices == "1" and fmt != rein.Q6_K and n_rows <= 8:
             assert np.array_equal(bits(got), bits(same)), f"not the 4x4x4 family's bits: fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
 
 
@@ -187,6 +191,14 @@ def test_lds_quad_persistent_and_widest_workgroups(fmt, in_dim, out_dim, options
     check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 8))
 
 
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (5120, 130), (2304, 4099), (17408, 70)])
+@pytest.mark.parametrize("slices", ["1", None])
+def test_lds_quad_nine_to_sixteen_rows(fmt, in_dim, out_dim, slices, options):
+    # rein_mvql_<fmt>_t16 behind rein_mmq_xq8 (the skinny MMQ otherwise); 16 rows x 17408 values take four phases
+    check_quad_lds(options, fmt, in_dim, out_dim, rows=(9, 12, 16), slices=slices)
+
+
 @pytest.mark.parametrize("waves", [1, 3, 16])
 def test_lds_quad_forced_workgroup_size(waves, options):
     options.set("REIN_MV_WPB", str(waves))
@@ -207,10 +219,13 @@ def test_lds_quad_long_contractions_are_staged_in_phases(fmt, options):
 @pytest.mark.parametrize("fmt,in_dim,out_dim,n_rows", [(rein.Q6_K, 5120, 4100, 8), (rein.IQ4_XS, 5120, 4100, 6),
                                                       (rein.Q4_K, 2048, 8200, 5), (rein.Q8_0, 1024, 16388, 8),
                                                       (rein.Q5_K, 1280, 14340, 3), (rein.Q4_K, 5120, 4100, 4),
-                                                      (rein.Q4_0, 5120, 1030, 7), (rein.IQ3_S, 17408, 1300, 8)])
+                                                      (rein.Q4_0, 5120, 1030, 7), (rein.IQ3_S, 17408, 1300, 8),
+                                                      (rein.Q6_K, 2048, 2100, 12), (rein.Q5_K, 4096, 9000, 16),
+                                                      (rein.Q4_K, 14336, 1030, 9)])
 def test_default_dispatch_takes_the_lds_quad_kernel(fmt, in_dim, out_dim, n_rows, options):
     # 5-8 rows: Q6_K / Q5_K / IQ4_XS everywhere, the other formats up to 20480 rows (from 5 * 2^20 weights); 3-4 rows:
-    # every format but Q8_0 up to 8192 rows from 20 * 2^20 weights, and Q5_K, Q8_0, IQ3_S, Q4_K against 14336 rows and more
+    # every format but Q8_0 up to 8192 rows from 20 * 2^20 weights, and Q5_K, Q8_0, IQ3_S, Q4_K against 14336 rows and more;
+    # 9-16 rows: Q6_K / Q5_K on narrow and short-and-mid matrices, the others against few rows with a long contraction
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
