@@ -405,7 +405,7 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
 struct QuadLdsGeometry { unsigned wpb, grid, phase_sub, slices; size_t lds; };       // lds == 0: no launch fits
 QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : n_rows <= 8 ? 8 : 16;
+    const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : n_rows <= 8 ? 8 : n_rows <= 16 ? 16 : 32;
     const unsigned parts = fmt == REIN_TYPE_Q8_0 ? 3 : 2;               // 16-byte parts of Fmt<FMT>::Raw
     const unsigned groups = (out_dim + 3) / 4;
     QuadLdsGeometry g;
@@ -442,7 +442,7 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
         g.lds = 0;
         const unsigned round = 16u * g.slices;
         if (!persistent || (unsigned long long)g.grid * g.wpb >= groups)
-            for (unsigned phases = 2; phases <= 8 && g.lds == 0; phases++) {
+            for (unsigned phases = 2; phases <= 32 && g.lds == 0; phases++) {
                 const unsigned per = (((n_sub + phases - 1) / phases) + round - 1) / round * round;
                 if (bytes(per) <= kLdsPerCu) { g.phase_sub = per; g.lds = bytes(per); }
             }
@@ -450,7 +450,7 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
     return g;
 }
 
-// Whether a batched decode of 3..16 rows runs on it.  Runs of the library's other choice against this kernel, seven
+// Whether a batched decode of 3..32 rows runs on it.  Runs of the library's other choice against this kernel, seven
 // formats x 16 shapes x 3 / 4 / 5 / 6 / 8 rows (ratio of the two times):
 //   5-8 rows  Q6_K, Q5_K, IQ4_XS (the formats of the 4x4x4 kernel): level or ahead everywhere from 5 * 2^20 weights --
 //             5120 -> 5120 1.05-1.18 (1.15-1.37 with slices), 5120 -> 34816 1.02-1.25, 4096 -> 14336 1.31-1.47, 8192 -> 8192
@@ -468,12 +468,19 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
 //             1.08-1.51, Q4_K 0.98-1.18; mixed for Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
 bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
-    if (n_rows < 3 || n_rows > 16) return false;
+    if (n_rows < 3 || n_rows > 32) return false;
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
     if (g.lds == 0) return false;
     if (opt_is_set(O_QUAD_LDS)) return opt_u(O_QUAD_LDS, 0) != 0;
     if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
+    if (n_rows > 16)
+        // 17-32 rows, against the 32-token tile launch of rein_mmq_xq8, which hands out one workgroup per 128 rows (40
+        // workgroups for 5120 rows): ahead up to 8192 rows for every format -- 24 / 32 rows, us: Q4_K 5120 -> 5120 39 ->
+        // 23, 17408 -> 5120 127 -> 56, 14336 -> 4096 104 -> 40, 8192 -> 8192 70 -> 38, 28672 -> 8192 207 -> 111, 5120 -> 1024
+        // 38 -> 14; Q6_K 69 -> 50, 230 -> 127, 188 -> 91, 114 -> 92; beyond (4096 -> 14336 0.72-1.30, 2048 -> 16384
+        // 0.65-1.13) the tile launch has workgroups enough
+        return weights >= (1ull << 22) && out_dim <= 8192;
     if (n_rows > 8) {
         // 9-16 rows (rein_mmq_xq8 sends them here), against the skinny MMQ at 12 and 16 rows: Q6_K and Q5_K ahead on
         // narrow and on short-and-mid matrices (5120 -> 5120 1.27 / 1.13, 17408 -> 5120 1.29 / 1.17, 14336 -> 4096 1.30 /
@@ -501,7 +508,7 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
                     unsigned n_rows, rein_stream_t s)
 {
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
-    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : "_t16");
+    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" : "_t32");
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub, (void*)&g.slices};
     return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
 }
@@ -952,7 +959,7 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    if (p_rows > 8 && p_rows <= 16 && use_mvql(fmt, in_dim, out_dim, p_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (p_rows > 8 && p_rows <= 32 && use_mvql(fmt, in_dim, out_dim, p_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // Token tiles: 32 tokens (rein_mmq_<fmt>_t32, three workgroups per CU) or the mixed launch
     // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).

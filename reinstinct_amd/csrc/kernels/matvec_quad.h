@@ -425,12 +425,14 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
                     if (blk == 0u) part[(t * 4 + r) * 4 + j] = v;
                 }
             __syncthreads();
-            if (has && slice == 0u && lane < 16u * NT) {
-                float v = part[lane];
-                for (unsigned k = 1; k < slices; k++) v += part[k * (kParts * 76u * 4u) + lane];
-                const unsigned t = lane >> 4, r = (lane >> 2) & 3u, jj = lane & 3u;
-                const unsigned tok = 4u * t + jj, orow = g * 4u + r;
-                if (tok < n_rows && orow < out_dim) y[(size_t)tok * out_dim + orow] = v;
+            if (has && slice == 0u) {
+                for (unsigned e = lane; e < 16u * NT; e += 64u) {
+                    float v = part[e];
+                    for (unsigned k = 1; k < slices; k++) v += part[k * (kParts * 76u * 4u) + e];
+                    const unsigned t = e >> 4, r = (e >> 2) & 3u, jj = e & 3u;
+                    const unsigned tok = 4u * t + jj, orow = g * 4u + r;
+                    if (tok < n_rows && orow < out_dim) y[(size_t)tok * out_dim + orow] = v;
+                }
             }
         }
     }

@@ -199,6 +199,14 @@ def test_lds_quad_nine_to_sixteen_rows(fmt, in_dim, out_dim, slices, options):
     check_quad_lds(options, fmt, in_dim, out_dim, rows=(9, 12, 16), slices=slices)
 
 
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (5120, 130), (2304, 4099), (17408, 70)])
+@pytest.mark.parametrize("slices", ["1", None])
+def test_lds_quad_seventeen_to_thirty_two_rows(fmt, in_dim, out_dim, slices, options):
+    # rein_mvql_<fmt>_t32 behind rein_mmq_xq8 (the 32-token tile launch otherwise); 32 rows x 5120 values take two phases
+    check_quad_lds(options, fmt, in_dim, out_dim, rows=(17, 24, 32), slices=slices)
+
+
 @pytest.mark.parametrize("waves", [1, 3, 16])
 def test_lds_quad_forced_workgroup_size(waves, options):
     options.set("REIN_MV_WPB", str(waves))
@@ -221,11 +229,13 @@ def test_lds_quad_long_contractions_are_staged_in_phases(fmt, options):
                                                       (rein.Q5_K, 1280, 14340, 3), (rein.Q4_K, 5120, 4100, 4),
                                                       (rein.Q4_0, 5120, 1030, 7), (rein.IQ3_S, 17408, 1300, 8),
                                                       (rein.Q6_K, 2048, 2100, 12), (rein.Q5_K, 4096, 9000, 16),
-                                                      (rein.Q4_K, 14336, 1030, 9)])
+                                                      (rein.Q4_K, 14336, 1030, 9), (rein.Q8_0, 2048, 2100, 17),
+                                                      (rein.Q4_K, 5120, 1030, 32)])
 def test_default_dispatch_takes_the_lds_quad_kernel(fmt, in_dim, out_dim, n_rows, options):
     # 5-8 rows: Q6_K / Q5_K / IQ4_XS everywhere, the other formats up to 20480 rows (from 5 * 2^20 weights); 3-4 rows:
     # every format but Q8_0 up to 8192 rows from 20 * 2^20 weights, and Q5_K, Q8_0, IQ3_S, Q4_K against 14336 rows and more;
-    # 9-16 rows: Q6_K / Q5_K on narrow and short-and-mid matrices, the others against few rows with a long contraction
+    # 9-16 rows: Q6_K / Q5_K on narrow and short-and-mid matrices, the others against few rows with a long contraction;
+    # 17-32 rows: every format up to 8192 rows
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=n_rows)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     xq = orc.quantize_q8(np.random.default_rng(fmt).standard_normal((n_rows, in_dim)).astype(np.float32))
