@@ -7,6 +7,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <cstdio>
 #include <cstring>
 #include <mutex>
 #include <algorithm>
@@ -1390,11 +1391,20 @@ int rein_noalloc_prepare(void)
     }
     static const int fmts[] = {REIN_TYPE_Q4_0, REIN_TYPE_Q4_K, REIN_TYPE_Q5_K, REIN_TYPE_Q6_K, REIN_TYPE_Q8_0, REIN_TYPE_IQ4_XS};
     static const char* const forms[] = {"_t32", "_t64", "_mix", "_sk", "_sk32"};
-    for (int fmt : fmts)
+    // (up to 32 rows the entry point launches the few-row kernels)
+    static const char* const few[] = {"rein_mmqs_%s_v1", "rein_mmqs_%s_v2", "rein_mmqs_%s_v4", "rein_mmqs_%s_v8", "rein_mvql_%s_t16", "rein_mvql_%s_t32"};
+    for (int fmt : fmts) {
         for (const char* form : forms) {
             hipFunction_t f;
             if (int rc = get_fn(std::string("rein_mmq_") + fmt_tag(fmt) + form, &f)) return rc;
         }
+        for (const char* pattern : few) {
+            char name[64];
+            std::snprintf(name, sizeof(name), pattern, fmt_tag(fmt));
+            hipFunction_t f;
+            if (int rc = get_fn(name, &f)) return rc;
+        }
+    }
     return 0;
 }
 
