@@ -310,7 +310,10 @@ int rein_matvec_ondisk_xq8(int fmt, const void *w_blocks, const void *xq, float 
 int rein_matvec_q8_0_splitk(const void *w, const void *xq, float *y_partials, unsigned in_dim,
                             unsigned out_dim, unsigned n_split, rein_stream_t s);
 /* matmul_mmq_into without its quantize step (src/runtime/prefill.rs:512-567):
- * Y[p_rows][out_dim] = Xq . W^T on the int8 MFMA path. */
+ * Y[p_rows][out_dim] = Xq . W^T on the int8 MFMA path.  Few rows take the batched-decode
+ * kernels instead of token tiles: up to 8 rows what rein_matvec_batched_xq8 launches, up to 16
+ * the skinny MMQ or the LDS-staged 4x4x4 kernel, up to 32 rows against at most 8192 output
+ * rows that kernel as well (the tile launch would hand out one workgroup per 128 rows). */
 int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                  unsigned out_dim, unsigned p_rows, rein_stream_t s);
 /* The same product with a caller-provided workspace of rein_mmq_workspace_bytes(fmt, in_dim,

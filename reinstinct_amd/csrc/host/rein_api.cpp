@@ -960,7 +960,9 @@ int rein_mmq_xq8(int fmt, const void* w, const void* xq, float* y, unsigned in_d
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    if (p_rows > 8 && p_rows <= 32 && use_mvql(fmt, in_dim, out_dim, p_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    // few rows: the batched-decode kernels (up to eight rows the choice of rein_matvec_batched_xq8, the same outputs)
+    if (p_rows <= 8) return launch_matvec(who, fmt, w, xq, y, in_dim, out_dim, p_rows, s);
+    if (p_rows <= 32 && use_mvql(fmt, in_dim, out_dim, p_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     if (p_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, p_rows, s);
     // Token tiles: 32 tokens (rein_mmq_<fmt>_t32, three workgroups per CU) or the mixed launch
     // (rein_mmq_<fmt>_mix: n64 tiles of 64 tokens per row block, the rest in 32-token tiles).
