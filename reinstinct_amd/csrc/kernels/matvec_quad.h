@@ -1,5 +1,7 @@
-// Batched decode matvec on the small int8 matrix instruction: 3 to 8 activation rows for
-// the formats whose weight unpack is expensive (Q6_K, Q5_K, IQ4_XS).
+// Batched decode matvec on the small int8 matrix instruction: 3 to 8 activation rows (the
+// first kernel below; the library picks it for the formats whose weight unpack is expensive,
+// Q6_K, Q5_K, IQ4_XS) and 3 to 32 rows with the activation rows staged in LDS (the second
+// kernel, every format).
 //
 // On the dot4 matvec every activation row costs eight v_dot4_i32_i8 per weight sub-block
 // and lane, and the weight unpack is repeated per output row.  v_mfma_i32_4x4x4_16b_i8
@@ -244,10 +246,18 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
 // of 16): every wavefront then owns at most ONE row group (the launch has at least as many wavefronts as
 // row groups), keeps its partial sums in registers across the phases, and the workgroup re-stages between
 // two barriers that every wavefront reaches, with or without a row group.  phase_sub >= in_dim / 32 is the
-// single-phase form, in which wavefronts may stride over several row groups.
-// Launch: block = 64 x W threads (W <= 16), dynamic shared memory =
+// single-phase form, in which -- with slices == 1 -- wavefronts may stride over several row groups.
+//
+// A matrix with few rows has few row groups (5120 rows: 1280, five per CU), each with one trip of weights
+// in flight: a latency-bound launch.  With `slices` = S > 1 wavefront w of the workgroup takes row group
+// w / S and every S-th trip of its contraction, from trip w % S on; the S partial sums meet in LDS (in the
+// wavefronts' weight images) and the first slice's wavefront adds them in slice order, so the result does
+// not depend on timing (it differs in the last bits from the S = 1 order).  Again one row group per
+// wavefront at most; with phases, phase_sub is a multiple of 16 * S, so that a wavefront's next trip is
+// the same sub-blocks whether or not a phase boundary lies in between.
+// Launch: block = 64 x W threads (W <= 16, a multiple of S), dynamic shared memory =
 //   4*NT * stride * 40 + W * kParts * 76 * 16 bytes, stride = n + ((20 - n % 16) % 16) for
-//   n = min(in_dim / 32, phase_sub).
+//   n = min(in_dim / 32, phase_sub); grid >= ceil(row groups / (W / S)) unless single-phase with S = 1.
 template <int FMT, int NT>
 __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
                                                           float* __restrict__ y, unsigned in_dim, unsigned out_dim,
