@@ -140,8 +140,8 @@ int check_ptr(const char* who, const void* p, size_t align, const char* what)
 // rein_set_option changes an entry, so the launch an entry point chooses depends on its arguments
 // and on this table alone.  Entries are single atomic words: setting one while another thread
 // launches is safe, the launch sees the old or the new value.
-enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_QUAD_SLICES, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
-const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_QUAD_SLICES", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
+enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_QUAD_SLICES, O_QUAD_DEPTH, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
+const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_QUAD_SLICES", "REIN_QUAD_DEPTH", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
 constexpr uint64_t kOptSet = 1ull << 63;
 std::atomic<uint64_t> g_opts[O_COUNT];          // zero = unset
 std::once_flag g_opts_env_once;
@@ -466,7 +466,8 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
 //             1.15-1.18, 18944 -> 3584 1.17, 5120 -> 7168 1.18-1.20, 8192 -> 8192 0.96; Q4_0 1.08-1.33; Q6_K 1.07-1.22;
 //             Q5_K 1.05-1.27; IQ4_XS 1.01-1.17; IQ3_S 0.99-1.21; 4096 -> 4096 (2^24 weights) 0.86-0.97 and stays.
 //             Against 14336 rows and more, where neither of those applies: Q5_K 1.03-1.18, Q8_0 0.99-1.17, IQ3_S
-//             1.08-1.51, Q4_K 0.98-1.18; mixed for Q4_0 0.92-1.13, IQ4_XS 0.93-1.08, Q6_K 0.89-1.09, which stay.
+//             1.08-1.51, Q4_K 0.98-1.18, Q4_0 (with two trips in flight) 1.03-1.18; mixed for IQ4_XS 0.93-1.08 and Q6_K
+//             0.89-1.09, which stay.
 bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     if (n_rows < 3 || n_rows > 32) return false;
@@ -502,7 +503,8 @@ bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
     }
     if (fmt != REIN_TYPE_Q8_0 && out_dim <= 8192 && weights >= (20ull << 20)) return true;
     if (weights < (1ull << 24)) return false;
-    return out_dim >= 14336 && (fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K);
+    return out_dim >= 14336 && (fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K ||
+                                fmt == REIN_TYPE_Q4_0);
 }
 
 int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
@@ -510,7 +512,19 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
 {
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
     const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" : "_t32");
-    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub, (void*)&g.slices};
+    // Trips of weights in flight per wavefront where wavefronts stride over row groups or own a whole one (no slices,
+    // no phases): two for the formats with little arithmetic per sub-block at 3-4 rows -- two register sets taking
+    // turns -- (us, 5120 -> 34816 / 5120 -> 17408 / 3584 -> 18944 at 4 rows, one -> two: Q4_K 28.3 -> 26.0, 18.8 -> 17.3,
+    // 14.2 -> 13.0; Q4_0 27.4 -> 23.7, 18.9 -> 16.1, 14.4 -> 12.2; IQ3_S 27.8 -> 24.2, 18.7 -> 16.2; Q8_0 40.1 -> 37.5,
+    // 25.8 -> 23.0; Q5_K 33.0 -> 32.3, 21.2 -> 20.3) and for Q8_0 / Q4_0 / IQ3_S at 5-8 rows against 16384 rows and more
+    // (1.05-1.07 x); Q6_K and IQ4_XS lose 3-10 % to the registers it costs, Q4_K and Q5_K at 8 rows 1-4 %.
+    const bool light = fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q5_K;
+    unsigned depth = 1;
+    if (n_rows <= 4 && light) depth = 2;
+    else if (n_rows <= 8 && out_dim >= 16384 && (fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_IQ3_S)) depth = 2;
+    depth = opt_u(O_QUAD_DEPTH, depth);
+    void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub, (void*)&g.slices,
+                    (void*)&depth};
     return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
 }
 

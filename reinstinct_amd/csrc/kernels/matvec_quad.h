@@ -261,7 +261,7 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
 template <int FMT, int NT>
 __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq,
                                                           float* __restrict__ y, unsigned in_dim, unsigned out_dim,
-                                                          unsigned n_rows, unsigned phase_sub, unsigned slices)
+                                                          unsigned n_rows, unsigned phase_sub, unsigned slices, unsigned depth)
 {
     using F = Fmt<FMT>;
     using Raw = typename F::Raw;
@@ -301,18 +301,17 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
     Raw rq;
     // one trip of row group g: 16 sub-blocks from sb0, whose activations sit at plane index x0 + block; the
     // wavefront's next trip starts `ahead` sub-blocks further on
-    auto trip = [&](unsigned g, unsigned sb0, unsigned x0, unsigned ahead, float (&acc)[NT][4]) {
-        const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(rq);
+    // (the weights of the trip arrive in rqx; the same registers then take the request for sub-blocks psb.. of row group png)
+    auto trip_on = [&](Raw& rqx, unsigned sb0, unsigned x0, unsigned png, unsigned psb, float (&acc)[NT][4]) {
+        const QuadRawBits<FMT> bits = rein_quad_raw_bits<FMT>(rqx);
 #pragma unroll
         for (int i = 0; i < kParts; i++) stage[i * 76 + put] = bits.p[i];
-        // the load registers are free again: the next trip (of this row group, or the first of the wavefront's
-        // next one) is requested now, pinned between scheduling barriers as in the kernel above
+        // the load registers are free again: a later trip (of this row group, or of the wavefront's next one) is
+        // requested now, pinned between scheduling barriers as in the kernel above
         __builtin_amdgcn_sched_barrier(0);
         {
-            const bool last = sb0 + ahead >= n_sub;
-            const unsigned ng = last ? min(g + step, n_groups - 1u) : g;
-            const unsigned nrow = min(ng * 4u + lr, out_dim - 1u);
-            rq = fmt.load(nrow, min((last ? 0u : sb0 + ahead) + ls, n_sub - 1u));
+            const unsigned nrow = min(min(png, n_groups - 1u) * 4u + lr, out_dim - 1u);
+            rqx = fmt.load(nrow, min(psb + ls, n_sub - 1u));
         }
         __builtin_amdgcn_sched_barrier(0);
         QuadRawBits<FMT> mine;
@@ -360,6 +359,10 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
             }
         }
     };
+    auto trip = [&](unsigned g, unsigned sb0, unsigned x0, unsigned ahead, float (&acc)[NT][4]) {
+        const bool last = sb0 + ahead >= n_sub;
+        trip_on(rq, sb0, x0, last ? g + step : g, last ? 0u : sb0 + ahead, acc);
+    };
     // sum over the 16 blocks (lane bits 2..5); lanes 0..3 (block 0) store
     auto finish = [&](unsigned g, float (&acc)[NT][4]) {
 #pragma unroll
@@ -386,6 +389,38 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
         {   // the first trip's weights are on their way while the activations are staged
             const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
             rq = fmt.load(row, min(ls, n_sub - 1u));
+        }
+        if (depth >= 2u) {
+            // two trips of weights in flight per wavefront: two register sets take turns, each refilled with the trip
+            // after next as soon as its own has gone to LDS
+            struct Pos { unsigned g, sb0; };
+            auto nxt = [&](Pos p) { Pos q; const bool last = p.sb0 + 16u >= n_sub; q.g = last ? p.g + step : p.g; q.sb0 = last ? 0u : p.sb0 + 16u; return q; };
+            Pos p; p.g = g; p.sb0 = 0u;
+            Pos q = nxt(p), r2 = nxt(q);
+            Raw rq2;
+            {
+                const unsigned row = min(min(q.g, n_groups - 1u) * 4u + lr, out_dim - 1u);
+                rq2 = fmt.load(row, min(q.sb0 + ls, n_sub - 1u));
+            }
+            stage_x(0u, n_sub);
+            __syncthreads();
+            auto one = [&](Raw& rqx) {
+                trip_on(rqx, p.sb0, p.sb0, r2.g, r2.sb0, acc);
+                if (p.sb0 + 16u >= n_sub) {
+                    finish(p.g, acc);
+#pragma unroll
+                    for (int t = 0; t < NT; t++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+                }
+                p = q; q = r2; r2 = nxt(r2);
+            };
+            while (p.g < n_groups) {
+                one(rq);
+                if (!(p.g < n_groups)) break;
+                one(rq2);
+            }
+            return;
         }
         stage_x(0u, n_sub);
         __syncthreads();
@@ -448,12 +483,13 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
     }
 }
 
-// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub, slices), n_rows <= 4 * NT
+// name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub, slices, depth), n_rows <= 4 * NT
 #define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT)                                                \
     extern "C" __global__ __launch_bounds__(1024) void name(                                      \
         const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y,    \
         unsigned int in_dim, unsigned int out_dim, unsigned int n_rows, unsigned int phase_sub,   \
-        unsigned int slices)                                                                      \
+        unsigned int slices, unsigned int depth)                                                  \
     {                                                                                             \
-        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows, phase_sub, slices); \
+        rein_matvec_quad_lds_body<FMT, NT>(w, xq, y, in_dim, out_dim, n_rows, phase_sub, slices,  \
+                                           depth);                                                \
     }

@@ -207,6 +207,16 @@ def test_lds_quad_seventeen_to_thirty_two_rows(fmt, in_dim, out_dim, slices, opt
     check_quad_lds(options, fmt, in_dim, out_dim, rows=(17, 24, 32), slices=slices)
 
 
+@pytest.mark.parametrize("fmt", DENSE)
+@pytest.mark.parametrize("depth", ["1", "2"])
+def test_lds_quad_two_trips_in_flight(fmt, depth, options):
+    # two register sets taking turns (REIN_QUAD_DEPTH=2) give the bits of one: persistent wavefronts over an odd and an
+    # even number of trips per row group, one row group per wavefront, fewer row groups than wavefronts
+    options.set("REIN_QUAD_DEPTH", depth)
+    for in_dim, out_dim in ((256, 70003), (512, 16500), (2304, 4099), (1056 if fmt in (rein.Q4_0, rein.Q8_0) else 1280, 37), (512, 3)):
+        check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 4, 8))
+
+
 @pytest.mark.parametrize("waves", [1, 3, 16])
 def test_lds_quad_forced_workgroup_size(waves, options):
     options.set("REIN_MV_WPB", str(waves))
