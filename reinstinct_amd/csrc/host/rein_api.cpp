@@ -519,8 +519,12 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
     // 25.8 -> 23.0; Q5_K 33.0 -> 32.3, 21.2 -> 20.3) and for Q8_0 / Q4_0 / IQ3_S at 5-8 rows against 16384 rows and more
     // (1.05-1.07 x); Q6_K and IQ4_XS lose 3-10 % to the registers it costs, Q4_K and Q5_K at 8 rows 1-4 %.
     const bool light = fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q5_K;
+    // With slices or phases (narrow matrices) the second register set gains only where a wavefront has the CU nearly to
+    // itself: 5120 -> 1024 1.05-1.20 x for every format at 4 and 8 rows, 0.86-1.05 from 4096 rows on.
+    const bool strided = g.slices == 1 && g.phase_sub >= in_dim / 32;
     unsigned depth = 1;
-    if (n_rows <= 4 && light) depth = 2;
+    if (!strided) depth = out_dim <= 1536 ? 2 : 1;
+    else if (n_rows <= 4 && light) depth = 2;
     else if (n_rows <= 8 && out_dim >= 16384 && (fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_IQ3_S)) depth = 2;
     depth = opt_u(O_QUAD_DEPTH, depth);
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows, (void*)&g.phase_sub, (void*)&g.slices,

@@ -240,7 +240,8 @@ __device__ __forceinline__ void rein_matvec_quad_body(const uint8_t* __restrict_
 // the compute-side lane (block b, row j) reads its operand at (4t + j) * stride + sub-block directly and a
 // quarter-wave pass covers 64 different banks.  Only the weights still take the trip through the
 // wavefront's private LDS image.  A trip requests the next trip's weights (or the first trip of the
-// wavefront's next row group) before it computes.  Same arithmetic in the same order as the kernel above.
+// wavefront's next row group) before it computes.  Same arithmetic in the same order as the kernel above (the
+// compiler's choice of fused multiply-adds may differ between the two, so the last bits may).
 //
 // A contraction whose rows do not fit the LDS is staged in phases of `phase_sub` sub-blocks (a multiple
 // of 16): every wavefront then owns at most ONE row group (the launch has at least as many wavefronts as
@@ -440,17 +441,26 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
         const unsigned g = blockIdx.x * gpb + wave / slices;
         const bool has = wave < gpb * slices && g < n_groups;    // wave-uniform
         const unsigned ahead = 16u * slices;
+        const bool two = depth >= 2u;                            // two register sets of weights taking turns
+        Raw rq2;
         {
             const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
             rq = fmt.load(row, min(16u * slice + ls, n_sub - 1u));
+            if (two) rq2 = fmt.load(row, min(16u * slice + ahead + ls, n_sub - 1u));
         }
+        bool odd = false;
         for (unsigned ph0 = 0; ph0 < n_sub; ph0 += phase_sub) {
             const unsigned count = min(phase_sub, n_sub - ph0);
             if (ph0 != 0u) __syncthreads();            // every wavefront is done with the previous phase's planes
             stage_x(ph0, count);
             __syncthreads();
             if (has)
-                for (unsigned sb0 = ph0 + 16u * slice; sb0 < ph0 + count; sb0 += ahead) trip(g, sb0, sb0 - ph0, ahead, acc);
+                for (unsigned sb0 = ph0 + 16u * slice; sb0 < ph0 + count; sb0 += ahead) {
+                    if (!two) trip(g, sb0, sb0 - ph0, ahead, acc);
+                    else if (!odd) trip_on(rq, sb0, sb0 - ph0, g, sb0 + 2u * ahead, acc);
+                    else trip_on(rq2, sb0, sb0 - ph0, g, sb0 + 2u * ahead, acc);
+                    odd = !odd;
+                }
         }
         if (slices <= 1u) {
             if (has) finish(g, acc);

