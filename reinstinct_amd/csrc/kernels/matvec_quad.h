@@ -454,13 +454,15 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
             if (ph0 != 0u) __syncthreads();            // every wavefront is done with the previous phase's planes
             stage_x(ph0, count);
             __syncthreads();
-            if (has)
+            if (has && !two) {
+                for (unsigned sb0 = ph0 + 16u * slice; sb0 < ph0 + count; sb0 += ahead) trip(g, sb0, sb0 - ph0, ahead, acc);
+            } else if (has) {
                 for (unsigned sb0 = ph0 + 16u * slice; sb0 < ph0 + count; sb0 += ahead) {
-                    if (!two) trip(g, sb0, sb0 - ph0, ahead, acc);
-                    else if (!odd) trip_on(rq, sb0, sb0 - ph0, g, sb0 + 2u * ahead, acc);
+                    if (!odd) trip_on(rq, sb0, sb0 - ph0, g, sb0 + 2u * ahead, acc);
                     else trip_on(rq2, sb0, sb0 - ph0, g, sb0 + 2u * ahead, acc);
                     odd = !odd;
                 }
+            }
         }
         if (slices <= 1u) {
             if (has) finish(g, acc);
