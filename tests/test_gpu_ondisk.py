@@ -41,7 +41,8 @@ def gpu_quantize(x):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("in_dim,out_dim,gaussian", [(2048, 384, False), (5120, 1001, True), (256, 3, False), (4096, 64, True)])
+@pytest.mark.parametrize("in_dim,out_dim,gaussian", [(2048, 384, False), (5120, 1001, True), (256, 3, False), (4096, 64, True),
+                                                     (17408, 9, False), (768, 2051, False)])
 def test_ondisk_matvec_parity(fmt, in_dim, out_dim, gaussian):
     if gaussian:
         w = (np.random.default_rng(fmt + in_dim).standard_normal((out_dim, in_dim)) * 0.02).astype(np.float32)
@@ -66,6 +67,20 @@ def test_ondisk_matvec_parity(fmt, in_dim, out_dim, gaussian):
     runtime.matvec_xq8(fmt, dev(packed), dq, dy2, in_dim, out_dim)
     hip.synchronize()
     assert_close_f32(got, dy2.to_host(np.float32), rel=1e-5, abs_=1e-6, what="on-disk vs repacked kernel")
+
+
+@pytest.mark.parametrize("in_dim,out_dim", [(32, 1), (96, 5), (352, 7), (2080, 3), (4128, 130)])
+def test_ondisk_q8_0_rows_that_are_not_multiples_of_16_bytes(in_dim, out_dim):
+    # 34-byte blocks: rows start at 2-byte alignment and the matrix ends inside a 16-byte piece
+    fmt = rein.Q8_0
+    raw = random_raw_weights(fmt, in_dim, out_dim, seed=in_dim)
+    x = np.random.default_rng(in_dim).standard_normal((1, in_dim)).astype(np.float32)
+    dq = gpu_quantize(x)
+    dy = dev(np.full(out_dim, np.nan, np.float32))
+    runtime.matvec_ondisk_xq8(fmt, dev(raw), dq, dy, in_dim, out_dim)
+    hip.synchronize()
+    packed = orc.repack_for_matvec(fmt, raw, in_dim, out_dim)
+    assert_close_f32(dy.to_host(np.float32), orc.matvec_q8(fmt, packed, in_dim, out_dim, dq.to_host(np.uint8), 1)[0], what="Q8_0 ragged rows")
 
 
 @pytest.mark.parametrize("fmt", FMTS)
