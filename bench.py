@@ -622,7 +622,8 @@ def decode_sweep(stream, steps):
                 base = sl if base is None else base
                 g = c.bytes_per_launch / sl / 1e9
                 out.append({"fmt": FMT_NAME[f], "K": k, "N": n, "batch": b, "us": round(sl * 1e6, 2), "GBs": round(g, 0),
-                            "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 3), "vs_batch1": round(sl / base, 3)})
+                            "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 3), "vs_batch1": round(sl / base, 3),
+                            "kernel": runtime.matvec_kernel_name(f, k, n, b)})
                 log("decode sweep", out[-1])
                 del c
             del rot

@@ -298,6 +298,13 @@ int rein_matvec_xq8(int fmt, const void *w, const void *xq, float *y, unsigned i
  * 448-508): y[n_rows][out_dim], 1 <= n_rows <= 8; the weights are streamed once. */
 int rein_matvec_batched_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                             unsigned out_dim, unsigned n_rows, rein_stream_t s);
+/* Which kernel a product of few activation rows launches, given the shape and the option table
+ * (host logic only, nothing is launched): 1..8 rows as rein_matvec_xq8 / rein_matvec_batched_xq8
+ * dispatch them, 9..32 rows the few-row kernels behind rein_mmq_xq8, "" where that entry point
+ * launches token tiles.  The reference picks its kernels in qwen35.rs:2232-2280 by format alone;
+ * here the choice also depends on the shape, and this call makes it visible. */
+int rein_matvec_kernel_name(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, char *name,
+                            size_t name_len);
 /* The on-disk-layout matvec (src/runtime/qwen35.rs:2209-2229; kernels/matvec_q4_k_dp4a.cpp
  * and its Q5_K / Q6_K / Q8_0 siblings): `w_blocks` holds out_dim rows of GGUF blocks as
  * they are on disk (not repacked) -- the path a tied token_embd / output matrix takes.

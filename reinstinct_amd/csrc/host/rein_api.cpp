@@ -532,6 +532,49 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
     return launch(name, g.grid, 1, 1, g.wpb * 64, (unsigned)g.lds, s, args);
 }
 
+// Which kernel family a decode of 1..8 activation rows runs on.
+enum class MvFamily { Dot4, Dot4Lds, Skinny, Quad, QuadLds };
+MvFamily matvec_family(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    // (an option that forces one LDS-staged family on goes first)
+    const bool mvql_forced = opt_u(O_QUAD_LDS, 0) != 0 && opt_u(O_MV_LDS, 0) == 0;
+    if (mvql_forced && use_mvql(fmt, in_dim, out_dim, n_rows)) return MvFamily::QuadLds;
+    if (use_mvl(fmt, in_dim, out_dim, n_rows)) return MvFamily::Dot4Lds;
+    if (use_mvql(fmt, in_dim, out_dim, n_rows)) return MvFamily::QuadLds;
+    const bool small = small_for_matrix_cores(fmt, in_dim, out_dim, n_rows);
+    if (!small && use_quad(fmt, out_dim, n_rows)) return MvFamily::Quad;
+    // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
+    if (!small && n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return MvFamily::Skinny;
+    return MvFamily::Dot4;
+}
+
+// The kernel a few-row product launches: 1..8 rows as rein_matvec_batched_xq8 dispatches them, 9..32 rows the few-row
+// kernels behind rein_mmq_xq8 ("" where that entry point launches token tiles).
+std::string matvec_kernel_name(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    const std::string tag = fmt_tag(fmt);
+    const std::string t = n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" : "_t32";
+    if (n_rows > 8) {
+        if (n_rows <= 32 && use_mvql(fmt, in_dim, out_dim, n_rows)) return "rein_mvql_" + tag + t;
+        if (n_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return "rein_mmqs_" + tag + "_v8";
+        return "";
+    }
+    switch (matvec_family(fmt, in_dim, out_dim, n_rows)) {
+    case MvFamily::QuadLds: return "rein_mvql_" + tag + t;
+    case MvFamily::Quad:    return "rein_mvq_" + tag + t;
+    case MvFamily::Skinny:  return "rein_mmqs_" + tag + "_v" + std::to_string(n_rows <= 2 ? 1 : n_rows <= 4 ? 2 : 4);
+    case MvFamily::Dot4Lds: {
+        unsigned r, wpb, grid;
+        mvl_geometry(fmt, in_dim, out_dim, n_rows, &r, &wpb, &grid);
+        return "rein_mvl_" + tag + "_r" + std::to_string(r) + "_b" + std::to_string(n_rows <= 2 ? 2 : 4);
+    }
+    default: {
+        const unsigned b = batch_slot(n_rows);
+        return "rein_mv_" + tag + "_r" + std::to_string(pick_rows_per_wave(fmt, out_dim, b)) + "_b" + std::to_string(b);
+    }
+    }
+}
+
 int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float* y, unsigned in_dim,
                   unsigned out_dim, unsigned n_rows, rein_stream_t s)
 {
@@ -541,20 +584,16 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (int rc = check_ptr(who, w, 16, "w")) return rc;
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     if (int rc = check_ptr(who, y, 4, "y")) return rc;
-    // (an option that forces one LDS-staged family on goes first)
-    const bool mvql_forced = opt_u(O_QUAD_LDS, 0) != 0 && opt_u(O_MV_LDS, 0) == 0;
-    if (mvql_forced && use_mvql(fmt, in_dim, out_dim, n_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
-    if (use_mvl(fmt, in_dim, out_dim, n_rows)) return launch_matvec_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
-    if (use_mvql(fmt, in_dim, out_dim, n_rows)) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
-    const bool small = small_for_matrix_cores(fmt, in_dim, out_dim, n_rows);
-    if (!small && use_quad(fmt, out_dim, n_rows)) {
+    const MvFamily family = matvec_family(fmt, in_dim, out_dim, n_rows);
+    if (family == MvFamily::QuadLds) return launch_quad_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (family == MvFamily::Dot4Lds) return launch_matvec_lds(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (family == MvFamily::Quad) {
         // four output rows per wavefront, four wavefronts per workgroup
         const std::string name = std::string("rein_mvq_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : "_t8");
         void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
         return launch(name, ((out_dim + 3) / 4 + 3) / 4, 1, 1, 256, 0, s, args);
     }
-    // (the skinny kernel fetches a row's eight fp16 scales at once: in_dim >= 256)
-    if (!small && n_rows >= skinny_from_rows(fmt) && in_dim >= 256) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+    if (family == MvFamily::Skinny) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(fmt, out_dim, b);
     // Wavefronts per workgroup (they share nothing): four, or two where the finer grain deals the wavefronts more
@@ -864,6 +903,18 @@ int rein_matvec_batched_xq8(int fmt, const void* w, const void* xq, float* y, un
                             unsigned out_dim, unsigned n_rows, rein_stream_t s)
 {
     return launch_matvec("rein_matvec_batched_xq8", fmt, w, xq, y, in_dim, out_dim, n_rows, s);
+}
+
+int rein_matvec_kernel_name(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, char* name, size_t name_len)
+{
+    const char* who = "rein_matvec_kernel_name";
+    if (!name || name_len == 0) return fail(REIN_E_BAD_POINTER, std::string(who) + ": no room for the name");
+    if (int rc = check_shape(who, fmt, in_dim, out_dim, n_rows)) return rc;
+    if (int rc = check_dense_fmt(who, fmt)) return rc;
+    const std::string k = matvec_kernel_name(fmt, in_dim, out_dim, n_rows);
+    if (k.size() + 1 > name_len) return fail(REIN_E_TOO_LARGE, std::string(who) + ": the name needs " + std::to_string(k.size() + 1) + " bytes");
+    std::memcpy(name, k.c_str(), k.size() + 1);
+    return 0;
 }
 
 int rein_matvec_ondisk_xq8(int fmt, const void* w_blocks, const void* xq, float* y, unsigned in_dim,

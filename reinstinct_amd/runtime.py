@@ -61,6 +61,13 @@ def matvec_batched_xq8(fmt, w, xq, y, in_dim, out_dim, n_rows, stream=None):
     check(lib.rein_matvec_batched_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, n_rows, _s(stream)))
 
 
+def matvec_kernel_name(fmt, in_dim, out_dim, n_rows):
+    """the kernel a product of 1..32 activation rows launches for this shape ('' where rein_mmq_xq8 launches token tiles)"""
+    buf = C.create_string_buffer(64)
+    check(lib.rein_matvec_kernel_name(fmt, in_dim, out_dim, n_rows, buf, len(buf)))
+    return buf.value.decode()
+
+
 def matvec_ondisk_xq8(fmt, w_blocks, xq, y, in_dim, out_dim, stream=None):
     """the on-disk-layout dp4a matvec (src/runtime/qwen35.rs:2209-2229)"""
     check(lib.rein_matvec_ondisk_xq8(fmt, _p(w_blocks), _p(xq), _p(y), in_dim, out_dim, _s(stream)))

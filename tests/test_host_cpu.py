@@ -207,3 +207,55 @@ def test_options_table():
             _lib.set_option("REIN_MV_ROWS", bad_value)
         assert err.value.code == -3
     assert _lib.get_option("REIN_MV_ROWS") is None
+
+
+def test_matvec_kernel_name_follows_the_dispatch_rules():
+    # rein_matvec_kernel_name: host logic only -- which kernel 1..32 activation rows launch for a shape, by the rules
+    # beside use_mvl / use_mvql / use_quad in rein_api.cpp and the option table
+    import reinstinct_amd as rein
+    from reinstinct_amd import _lib
+    _lib.reset_options()
+    name = runtime.matvec_kernel_name
+    # one row: dot4, rows per wavefront by the width
+    assert name(rein.Q4_K, 5120, 5120, 1) == "rein_mv_q4k_r2_b1"
+    assert name(rein.Q4_K, 5120, 34816, 1) == "rein_mv_q4k_r4_b1"
+    # two rows: LDS-staged dot4 at long contractions and, for Q4_K, against many rows; dot4 otherwise
+    assert name(rein.Q4_K, 17408, 5120, 2) == "rein_mvl_q4k_r1_b2"
+    assert name(rein.Q4_K, 5120, 34816, 2) == "rein_mvl_q4k_r2_b2"
+    assert name(rein.Q6_K, 5120, 34816, 2) == "rein_mv_q6k_r2_b2"
+    assert name(rein.Q4_K, 5120, 5120, 2) == "rein_mv_q4k_r2_b2"
+    # three to four rows: the sliced 4x4x4 kernel on narrow matrices (not Q8_0), LDS-staged dot4 for Q8_0 and mid sizes
+    assert name(rein.Q4_K, 5120, 5120, 4) == "rein_mvql_q4k_t4"
+    assert name(rein.Q8_0, 5120, 5120, 3) == "rein_mvl_q8_0_r1_b4"
+    assert name(rein.Q4_K, 4096, 4096, 4) == "rein_mvl_q4k_r1_b4"
+    assert name(rein.Q4_K, 5120, 34816, 4) == "rein_mvql_q4k_t4"
+    assert name(rein.Q6_K, 5120, 34816, 4) == "rein_mvq_q6k_t4"
+    assert name(rein.Q4_K, 2048, 1536, 4) == "rein_mv_q4k_r1_b4"            # small matrices stay on dot4
+    # five to eight rows
+    assert name(rein.Q4_K, 17408, 5120, 8) == "rein_mvql_q4k_t8"
+    assert name(rein.Q4_K, 5120, 34816, 8) == "rein_mmqs_q4k_v4"
+    assert name(rein.Q6_K, 5120, 34816, 8) == "rein_mvql_q6k_t8"
+    # nine and more rows arrive through rein_mmq_xq8
+    assert name(rein.Q6_K, 5120, 5120, 12) == "rein_mvql_q6k_t16"
+    assert name(rein.Q4_K, 5120, 5120, 12) == "rein_mmqs_q4k_v8"
+    assert name(rein.Q4_K, 5120, 5120, 32) == "rein_mvql_q4k_t32"
+    assert name(rein.Q4_K, 5120, 34816, 32) == ""                             # token tiles
+    assert name(rein.Q4_K, 5120, 5120, 33) == ""
+    # options pin a family
+    try:
+        _lib.set_option("REIN_QUAD_LDS", 0)
+        assert name(rein.Q4_K, 5120, 5120, 4) == "rein_mvl_q4k_r1_b4"
+        assert name(rein.Q4_K, 17408, 5120, 8) == "rein_mmqs_q4k_v4"
+        _lib.set_option("REIN_MV_LDS", 0)
+        assert name(rein.Q4_K, 5120, 5120, 4) == "rein_mmqs_q4k_v2"
+        _lib.set_option("REIN_SKINNY_FROM", 99)
+        _lib.set_option("REIN_QUAD_FROM", 99)
+        assert name(rein.Q4_K, 5120, 5120, 4) == "rein_mv_q4k_r2_b4"
+        _lib.set_option("REIN_QUAD_FROM", 1)
+        assert name(rein.Q4_K, 5120, 5120, 4) == "rein_mvq_q4k_t4"
+    finally:
+        _lib.reset_options()
+    with pytest.raises(_lib.ReinError):
+        name(rein.Q4_K, 5120, 0, 1)
+    with pytest.raises(_lib.ReinError):
+        name(99, 5120, 5120, 1)
