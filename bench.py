@@ -489,6 +489,52 @@ def extras_decode_stream(stream):
     return res
 
 
+def extras_decode_layer_separate(stream):
+    """One decoder layer's matvecs at batch 1 when the model file keeps its projections as separate tensors, which is
+    how the reference launches them (src/runtime/qwen35.rs:2670-2705): Q 5120->5120, K and V 5120->1024 (V in Q6_K),
+    O 5120->5120, gate and up 5120->17408, down 17408->5120 -- seven launches -- against the same seven products in
+    four launches with rein_matvec_multi_xq8 (Q+K+V, O, gate+up, down).  Eight layers with their own weights in one
+    hipGraph, so every matvec streams from HBM."""
+    n_layers, hidden, ffn, kv = 8, 5120, 17408, 1024
+    spec = [("q", rein.Q4_K, hidden, hidden), ("k", rein.Q4_K, hidden, kv), ("v", rein.Q6_K, hidden, kv),
+            ("o", rein.Q4_K, hidden, hidden), ("gate", rein.Q4_K, hidden, ffn), ("up", rein.Q4_K, hidden, ffn),
+            ("down", rein.Q4_K, ffn, hidden)]
+    host = {nm: tiled_weights(f, k, n, seed=i) for i, (nm, f, k, n) in enumerate(spec)}
+    layers = [{nm: hip.DeviceBuf.from_host(host[nm]) for nm, _, _, _ in spec} for _ in range(n_layers)]
+    total = sum(h.nbytes for h in host.values())
+    fm = {nm: f for nm, f, _, _ in spec}
+    dq = {}
+    for k in (hidden, ffn):
+        dx = hip.DeviceBuf.from_host(np.random.default_rng(k).standard_normal((1, k)).astype(np.float32))
+        dq[k] = hip.DeviceBuf((k // 32) * 40)
+        runtime.quantize_q8(dx, dq[k], k, 1, stream)
+    ys = {nm: hip.DeviceBuf(n * 4) for nm, _, _, n in spec}
+
+    def seven():
+        for w in layers:
+            for nm, f, k, n in spec:
+                runtime.matvec_xq8(f, w[nm], dq[k], ys[nm], k, n, stream)
+
+    def four():
+        for w in layers:
+            runtime.matvec_multi_xq8([fm["q"], fm["k"], fm["v"]], [w["q"], w["k"], w["v"]], [ys["q"], ys["k"], ys["v"]],
+                                     [hidden, kv, kv], dq[hidden], hidden, stream)
+            runtime.matvec_xq8(fm["o"], w["o"], dq[hidden], ys["o"], hidden, hidden, stream)
+            runtime.matvec_multi_xq8([fm["gate"], fm["up"]], [w["gate"], w["up"]], [ys["gate"], ys["up"]], [ffn, ffn],
+                                     dq[hidden], hidden, stream)
+            runtime.matvec_xq8(fm["down"], w["down"], dq[ffn], ys["down"], ffn, hidden, stream)
+
+    a = time_graph(stream, seven, n_layers)
+    b = time_graph(stream, four, n_layers)
+    res = {"workload": "one decoder layer, projections kept as separate tensors (Q, K, V, O, gate, up, down; Q4_K, V in Q6_K), "
+                       "batch 1, 8 layers in one hipGraph",
+           "us_per_layer_7_launches": round(a * 1e6, 2), "us_per_layer_4_launches_multi": round(b * 1e6, 2),
+           "weight_MB_per_layer": round(total / 1e6, 1), "GBs_7_launches": round(total / a / 1e9, 0),
+           "GBs_4_launches_multi": round(total / b / 1e9, 0), "frac_hbm_peak_multi": round(total / b / 1e9 / HBM_PEAK_GBS, 4)}
+    log("decode layer, separate tensors", res)
+    return res
+
+
 def extras_decode_ffn(stream):
     """The FFN half of a dense decoder layer at batch 1 with the fused producers in place
     (hidden 5120, FFN 17408, Q4_K): add_rmsnorm_q8 -> gate+up matvec -> swiglu_q8 -> down matvec,
@@ -755,7 +801,8 @@ def main():
     if not args.no_configs:
         out["configs"] = {"decode_sweep_configs1": decode_sweep(stream, args.steps), "mmq_configs2": extras_mmq(stream), "mmq_short_prompts": extras_mmq_small(stream),
                           "moe_configs3": extras_moe(stream), "moe_configs3_one_token": extras_moe_decode(stream),
-                          "decode_stream_configs4": extras_decode_stream(stream)}
+                          "decode_stream_configs4": extras_decode_stream(stream),
+                          "decode_layer_separate_tensors": extras_decode_layer_separate(stream)}
 
     if args.sweep:
         sweep = []

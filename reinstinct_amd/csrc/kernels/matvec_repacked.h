@@ -29,15 +29,16 @@ struct XBlocks {
     int   q[B][8];
 };
 
+// The row groups first, first + step, ... of one matrix, walked by the calling wavefront.
 template <int FMT, int R, int B, int U = 1>
-__device__ __forceinline__ void rein_matvec_body(const uint8_t* __restrict__ w,
+__device__ __forceinline__ void rein_matvec_span(const uint8_t* __restrict__ w,
                                                  const BlockQ8* __restrict__ xq,
                                                  float* __restrict__ y,
-                                                 unsigned in_dim, unsigned out_dim, unsigned n_rows)
+                                                 unsigned in_dim, unsigned out_dim, unsigned n_rows,
+                                                 unsigned first, unsigned step)
 {
     using F = Fmt<FMT>;
     const unsigned lane  = threadIdx.x & 63u;
-    const unsigned wpb   = blockDim.x >> 6;
     const unsigned n_sub = in_dim >> 5;
     const F fmt(w, n_sub, out_dim);
 
@@ -45,7 +46,7 @@ __device__ __forceinline__ void rein_matvec_body(const uint8_t* __restrict__ w,
     const unsigned rmax = out_dim - 1;
     const unsigned bmax = n_rows - 1;
 
-    for (unsigned g = blockIdx.x * wpb + (threadIdx.x >> 6); g < n_groups; g += gridDim.x * wpb) {
+    for (unsigned g = first; g < n_groups; g += step) {
         const unsigned row0 = g * R;
         float acc[R][B];
 #pragma unroll
@@ -116,6 +117,17 @@ __device__ __forceinline__ void rein_matvec_body(const uint8_t* __restrict__ w,
                     y[(size_t)b * out_dim + row0 + r] = s;
             }
     }
+}
+
+// Every wavefront of the launch takes the row groups of its own index, striding by the launch's wavefront count.
+template <int FMT, int R, int B, int U = 1>
+__device__ __forceinline__ void rein_matvec_body(const uint8_t* __restrict__ w,
+                                                 const BlockQ8* __restrict__ xq,
+                                                 float* __restrict__ y,
+                                                 unsigned in_dim, unsigned out_dim, unsigned n_rows)
+{
+    const unsigned wpb = blockDim.x >> 6;
+    rein_matvec_span<FMT, R, B, U>(w, xq, y, in_dim, out_dim, n_rows, blockIdx.x * wpb + (threadIdx.x >> 6), gridDim.x * wpb);
 }
 
 // Per-block integer dots exactly as the matvec forms them, for the bit-exact

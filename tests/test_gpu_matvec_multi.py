@@ -1,0 +1,97 @@
+"""rein_matvec_multi_xq8: the decode step's consecutive matvecs on one activation row (Q / K / V, gate / up;
+src/runtime/qwen35.rs:2670-2672, 2702-2703) in one launch.  Every output is compared with the oracle and, bit for
+bit, with rein_matvec_xq8 on the same matrix: mixed formats, matrices of very different heights, row counts that
+do not divide by the rows per wavefront, each rows-per-wavefront kernel, and the argument checks."""
+import numpy as np
+import pytest
+
+import reinstinct_amd as rein
+from reinstinct_amd import hip, quant, runtime
+from reinstinct_amd._lib import ReinError, init
+from oracle import orc
+from helpers import assert_close_f32, dev, random_raw_weights
+
+pytestmark = pytest.mark.gpu
+
+DENSE = [rein.Q4_0, rein.Q8_0, rein.Q4_K, rein.Q5_K, rein.Q6_K, rein.IQ4_XS, rein.IQ3_S]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def gpu():
+    init()
+    hip.set_device(0)
+    yield
+    hip.synchronize()
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def check(fmts, in_dim, out_dims, seed=0):
+    print("multi matvec", fmts, in_dim, out_dims, flush=True)
+    packed = [quant.repack_for_matvec(f, random_raw_weights(f, in_dim, n, seed=seed + 7 * i + f), in_dim, n)
+              for i, (f, n) in enumerate(zip(fmts, out_dims))]
+    xq = orc.quantize_q8(np.random.default_rng(seed).standard_normal((1, in_dim)).astype(np.float32))
+    dq = dev(xq)
+    dws = [dev(p) for p in packed]
+    # one buffer for all outputs with a guard word behind each, so a write past a matrix's rows shows
+    offs = np.concatenate([[0], np.cumsum([n + 1 for n in out_dims])])
+    host = np.full(int(offs[-1]), np.float32(-77.0), np.float32)
+    dy = dev(host)
+    runtime.matvec_multi_xq8(fmts, dws, [dy.ptr + 4 * int(o) for o in offs[:-1]], out_dims, dq, in_dim)
+    hip.synchronize()
+    got = dy.to_host(np.float32)
+    for i, (f, n) in enumerate(zip(fmts, out_dims)):
+        mine = got[int(offs[i]):int(offs[i]) + n]
+        assert got[int(offs[i]) + n] == np.float32(-77.0), f"matrix {i} wrote past its rows"
+        want = orc.matvec_q8(f, packed[i], in_dim, n, xq, 1)
+        assert_close_f32(mine.reshape(1, n), want, what=f"multi matrix {i} fmt {f} {in_dim}->{n}")
+        d1 = dev(np.full(n, np.nan, np.float32))
+        runtime.matvec_xq8(f, dws[i], dq, d1, in_dim, n)
+        hip.synchronize()
+        assert np.array_equal(bits(mine), bits(d1.to_host(np.float32))), f"matrix {i} fmt {f}: not the bits of rein_matvec_xq8"
+
+
+@pytest.mark.parametrize("fmts,in_dim,out_dims", [
+    ([rein.Q4_K, rein.Q4_K, rein.Q6_K], 2048, [2048, 512, 512]),             # Q, K, V with a Q6_K value projection
+    ([rein.Q4_K, rein.Q4_K], 1024, [2816, 2816]),                            # gate, up
+    ([rein.Q8_0, rein.Q8_0], 2048, [96, 96]),                                # two tiny projections
+    ([rein.Q5_K, rein.Q6_K, rein.Q8_0, rein.Q4_0], 512, [33, 1, 130, 67]),   # four formats, odd heights
+    ([rein.IQ4_XS, rein.IQ3_S], 768, [259, 3]),
+    ([rein.Q6_K], 2304, [517]),                                              # one matrix: the plain launch
+])
+def test_multi_matvec(fmts, in_dim, out_dims):
+    check(fmts, in_dim, out_dims)
+
+
+@pytest.mark.parametrize("rows", ["1", "2", "4"])
+@pytest.mark.parametrize("fmt", DENSE)
+def test_multi_matvec_each_rows_per_wavefront(fmt, rows, options):
+    options.set("REIN_MV_ROWS", rows)
+    check([fmt, rein.Q4_K, fmt], 1280 if fmt in (rein.Q4_0, rein.Q8_0) else 1536, [131, 66, 7], seed=3)
+    options.unset("REIN_MV_ROWS")
+
+
+def test_multi_matvec_decode_shapes():
+    """the attention and FFN projections of the 27B-class decoder (hidden 5120, 40 / 8 heads of 128, FFN 17408)"""
+    check([rein.Q4_K, rein.Q4_K, rein.Q6_K], 5120, [5120, 1024, 1024], seed=1)
+    check([rein.Q4_K, rein.Q4_K], 5120, [17408, 17408], seed=2)
+
+
+def test_multi_matvec_argument_checks():
+    dq = dev(np.zeros(40 * 8, np.uint8))
+    dw = dev(np.zeros(4096, np.uint8))
+    dy = dev(np.zeros(64, np.float32))
+    with pytest.raises(ReinError):
+        runtime.matvec_multi_xq8([], [], [], [], dq, 256)
+    with pytest.raises(ReinError):
+        runtime.matvec_multi_xq8([rein.Q4_K] * 5, [dw] * 5, [dy] * 5, [4] * 5, dq, 256)
+    with pytest.raises(ReinError):
+        runtime.matvec_multi_xq8([rein.Q4_K, rein.Q5_1], [dw, dw], [dy, dy], [4, 4], dq, 256)
+    with pytest.raises(ReinError):
+        runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, dw], [dy, dy], [4, 0], dq, 256)
+    with pytest.raises(ReinError):
+        runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, 0], [dy, dy], [4, 4], dq, 256)
+    with pytest.raises(ReinError):
+        runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, dw], [dy, dy], [4, 4], dq, 200)

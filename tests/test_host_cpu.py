@@ -259,3 +259,20 @@ def test_matvec_kernel_name_follows_the_dispatch_rules():
         name(rein.Q4_K, 5120, 0, 1)
     with pytest.raises(_lib.ReinError):
         name(99, 5120, 5120, 1)
+
+
+def test_matvec_multi_checks_its_tables_on_the_host():
+    """rein_matvec_multi_xq8 refuses bad tables before anything reaches a device"""
+    from reinstinct_amd import runtime
+    from reinstinct_amd._lib import ReinError
+    ok = dict(fmts=[rein.Q4_K, rein.Q6_K], ws=[4096, 8192], ys=[4096, 8192], out_dims=[8, 8], xq=4096, in_dim=256)
+    bad = [dict(fmts=[], ws=[], ys=[], out_dims=[]),                                   # no matrix
+           dict(fmts=[rein.Q4_K] * 5, ws=[4096] * 5, ys=[4096] * 5, out_dims=[8] * 5),  # more than four
+           dict(fmts=[rein.Q4_K, 99]),                                                 # unknown format
+           dict(fmts=[rein.Q4_K, rein.Q5_1]),                                          # an expert-only format
+           dict(ws=[4096, 0]), dict(ys=[0, 4096]), dict(ws=[4096, 4100]),              # NULL and misaligned pointers
+           dict(out_dims=[8, 0]), dict(in_dim=200), dict(xq=0)]
+    for change in bad:
+        a = dict(ok, **change)
+        with pytest.raises(ReinError):
+            runtime.matvec_multi_xq8(a["fmts"], a["ws"], a["ys"], a["out_dims"], a["xq"], a["in_dim"])
