@@ -518,10 +518,10 @@ def extras_decode_layer_separate(stream):
     def four():
         for w in layers:
             runtime.matvec_multi_xq8([fm["q"], fm["k"], fm["v"]], [w["q"], w["k"], w["v"]], [ys["q"], ys["k"], ys["v"]],
-                                     [hidden, kv, kv], dq[hidden], hidden, stream)
+                                     [hidden, kv, kv], dq[hidden], hidden, 1, stream)
             runtime.matvec_xq8(fm["o"], w["o"], dq[hidden], ys["o"], hidden, hidden, stream)
             runtime.matvec_multi_xq8([fm["gate"], fm["up"]], [w["gate"], w["up"]], [ys["gate"], ys["up"]], [ffn, ffn],
-                                     dq[hidden], hidden, stream)
+                                     dq[hidden], hidden, 1, stream)
             runtime.matvec_xq8(fm["down"], w["down"], dq[ffn], ys["down"], ffn, hidden, stream)
 
     a = time_graph(stream, seven, n_layers)

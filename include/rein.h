@@ -298,14 +298,19 @@ int rein_matvec_xq8(int fmt, const void *w, const void *xq, float *y, unsigned i
  * 448-508): y[n_rows][out_dim], 1 <= n_rows <= 8; the weights are streamed once. */
 int rein_matvec_batched_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_dim,
                             unsigned out_dim, unsigned n_rows, rein_stream_t s);
-/* The consecutive launch_matvec_prequant calls of the decode step that share one activation row --
+/* The consecutive launch_matvec_prequant calls of the decode step that share their activations --
  * attn_q / attn_k / attn_v (src/runtime/qwen35.rs:2670-2672, 3612-3614), the dense FFN's gate / up
  * (qwen35.rs:2702-2703, 3662-3663), ssm_alpha / ssm_beta (qwen35.rs:2465-2466) -- as one launch:
- * ys[i] = ws[i] . xq for i < n_mat, 1 <= n_mat <= 4.  The matrices share in_dim and may differ in
- * format and in out_dims[i]; every output is bit for bit what rein_matvec_xq8 gives for that matrix.
- * The four tables are host arrays, read before the call returns. */
+ * ys[i][n_rows][out_dims[i]] = xq[n_rows] . ws[i]^T for i < n_mat, 1 <= n_mat <= 4, 1 <= n_rows <= 4
+ * (the two to four rows of the speculative-decode verify step, prefill.rs:448-508).  The matrices
+ * share in_dim and may differ in format and in out_dims[i]; with one row every output is bit for
+ * bit what rein_matvec_xq8 gives for that matrix, with more rows what the dot4 kernels behind
+ * rein_matvec_batched_xq8 give (three and four rows against matrices of an FFN's size go out as
+ * the launches of rein_matvec_batched_xq8 one by one, which are faster there).  The four tables are
+ * host arrays, read before the call returns. */
 int rein_matvec_multi_xq8(unsigned n_mat, const int *fmts, const void *const *ws, float *const *ys,
-                          const unsigned *out_dims, const void *xq, unsigned in_dim, rein_stream_t s);
+                          const unsigned *out_dims, const void *xq, unsigned in_dim, unsigned n_rows,
+                          rein_stream_t s);
 /* Which kernel a product of few activation rows launches, given the shape and the option table
  * (host logic only, nothing is launched): 1..8 rows as rein_matvec_xq8 / rein_matvec_batched_xq8
  * dispatch them, 9..32 rows the few-row kernels behind rein_mmq_xq8, "" where that entry point

@@ -86,7 +86,7 @@ SIGNATURES = {
     "rein_matvec_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _vp]),
     "rein_matvec_batched_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_matvec_kernel_name": (_i, [_i, _u, _u, _u, C.c_char_p, _sz]),
-    "rein_matvec_multi_xq8": (_i, [_u, C.POINTER(_i), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u), _vp, _u, _vp]),
+    "rein_matvec_multi_xq8": (_i, [_u, C.POINTER(_i), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u), _vp, _u, _u, _vp]),
     "rein_mmq_xq8": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp]),
     "rein_matmul": (_i, [_i, _vp, _vp, _vp, _u, _u, _u, _vp, _vp]),
     "rein_mmq_workspace_bytes": (_sz, [_i, _u, _u]),

@@ -905,21 +905,23 @@ int rein_matvec_batched_xq8(int fmt, const void* w, const void* xq, float* y, un
     return launch_matvec("rein_matvec_batched_xq8", fmt, w, xq, y, in_dim, out_dim, n_rows, s);
 }
 
-// Up to four matvecs on one activation row in one launch (kernels/matvec_multi.hip): the wavefronts of the
-// launch are dealt over the matrices' row groups, each runs its group as rein_mv_<fmt>_r<R>_b1 would.
+// Up to four matvecs on the same activation rows in one launch (kernels/matvec_multi.hip): the wavefronts of the
+// launch are dealt over the matrices' row groups, each runs its group as rein_mv_<fmt>_r<R>_b<B> would.
 int rein_matvec_multi_xq8(unsigned n_mat, const int* fmts, const void* const* ws, float* const* ys,
-                          const unsigned* out_dims, const void* xq, unsigned in_dim, rein_stream_t s)
+                          const unsigned* out_dims, const void* xq, unsigned in_dim, unsigned n_rows,
+                          rein_stream_t s)
 {
     const char* who = "rein_matvec_multi_xq8";
     constexpr unsigned kMax = 4;
     if (n_mat == 0 || n_mat > kMax)
         return fail(REIN_E_BAD_SHAPE, std::string(who) + ": " + std::to_string(n_mat) + " matrices, 1 to " + std::to_string(kMax) + " go into one launch");
+    if (n_rows > 4) return fail(REIN_E_TOO_LARGE, std::string(who) + ": at most 4 activation rows");
     if (!fmts || !ws || !ys || !out_dims) return fail(REIN_E_BAD_POINTER, std::string(who) + ": a NULL table");
     if (int rc = check_ptr(who, xq, 8, "xq")) return rc;
     unsigned long long total = 0;
     unsigned widest = 0;
     for (unsigned i = 0; i < n_mat; i++) {
-        if (int rc = check_shape(who, fmts[i], in_dim, out_dims[i], 1)) return rc;
+        if (int rc = check_shape(who, fmts[i], in_dim, out_dims[i], n_rows)) return rc;
         if (int rc = check_dense_fmt(who, fmts[i])) return rc;
         if (int rc = check_ptr(who, ws[i], 16, "w")) return rc;
         if (int rc = check_ptr(who, ys[i], 4, "y")) return rc;
@@ -927,11 +929,23 @@ int rein_matvec_multi_xq8(unsigned n_mat, const int* fmts, const void* const* ws
         if (out_dims[i] > out_dims[widest]) widest = i;
     }
     if (total > 0x3FFFFFFFull) return fail(REIN_E_TOO_LARGE, std::string(who) + ": too many rows for one launch");
-    if (n_mat == 1) return launch_matvec(who, fmts[0], ws[0], xq, ys[0], in_dim, out_dims[0], 1, s);
-    // rows per wavefront and wavefronts per workgroup as the single-matrix launch of all the rows would take them
+    // One matrix, or three to four rows against matrices of the size of an FFN's: the launches of the matrices one by
+    // one, whose few-row kernels (activations staged in LDS, matrix instructions) are further ahead of dot4 there than
+    // a launch costs (gate + up 5120 -> 17408 at 4 rows: 34.0 us as two launches, 38.6 as one; Q + K + V 5120 -> 5120 /
+    // 1024 / 1024: 20.7 against 14.1, stays one launch; at 2 rows 26.9 against 25.7 and 15.4 against 10.1).
+    const bool one_by_one = n_mat == 1 || (n_rows >= 3 && total * in_dim >= (64ull << 20) && !opt_is_set(O_MV_ROWS));
+    if (one_by_one) {
+        for (unsigned i = 0; i < n_mat; i++)
+            if (int rc = launch_matvec(who, fmts[i], ws[i], xq, ys[i], in_dim, out_dims[i], n_rows, s)) return rc;
+        return 0;
+    }
+    // rows per wavefront and wavefronts per workgroup as the dot4 launch of all the rows in the widest matrix's
+    // format would take them
     const int lead = fmts[widest];
-    const unsigned r = pick_rows_per_wave(lead, (unsigned)total, 1);
-    unsigned wpb = (lead == REIN_TYPE_Q8_0 || lead == REIN_TYPE_Q4_K || lead == REIN_TYPE_Q5_K) ? 2 : 4;
+    const unsigned b = batch_slot(n_rows);
+    const unsigned r = pick_rows_per_wave(lead, (unsigned)total, b);
+    unsigned wpb = 4;
+    if (b == 2 || (lead == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (lead == REIN_TYPE_Q4_K || lead == REIN_TYPE_Q5_K))) wpb = 2;
     const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
     if (wpb_forced == 1 || wpb_forced == 2 || wpb_forced == 4) wpb = wpb_forced;
     struct Mat { const void* w; float* y; unsigned out_dim; int fmt; unsigned group_end; unsigned pad; };
@@ -942,8 +956,8 @@ int rein_matvec_multi_xq8(unsigned n_mat, const int* fmts, const void* const* ws
         a.m[i] = Mat{ws[i], ys[i], out_dims[i], fmts[i], groups, 0u};
     }
     for (unsigned i = n_mat; i < kMax; i++) a.m[i] = a.m[n_mat - 1];
-    void* args[] = {(void*)&a, (void*)&xq, (void*)&in_dim, (void*)&n_mat};
-    return launch("rein_mv_multi_r" + std::to_string(r), (groups + wpb - 1) / wpb, 1, 1, wpb * 64, 0, s, args);
+    void* args[] = {(void*)&a, (void*)&xq, (void*)&in_dim, (void*)&n_mat, (void*)&n_rows};
+    return launch("rein_mv_multi_r" + std::to_string(r) + "_b" + std::to_string(b), (groups + wpb - 1) / wpb, 1, 1, wpb * 64, 0, s, args);
 }
 
 int rein_matvec_kernel_name(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, char* name, size_t name_len)

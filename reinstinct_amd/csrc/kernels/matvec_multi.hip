@@ -1,4 +1,5 @@
-// Several decode matvecs that share one activation row, in one launch: rein_mv_multi_r<R>.
+// Several decode matvecs that share their activation rows (one, or the two to four of a speculative-decode
+// verify step), in one launch: rein_mv_multi_r<R>_b<B>.
 //
 // The reference's decode step launches the Q, K and V projections one after the other on the same
 // quantized activations, and likewise the gate and up projections of a dense FFN
@@ -6,9 +7,9 @@
 // that size costs one to two microseconds of gap and ramp that no kernel can win back.  Here the
 // wavefronts of one launch are dealt over up to four matrices: wavefront i belongs to the first
 // matrix whose cumulative row-group count exceeds i and runs that matrix's row group exactly as the
-// single-matrix kernel rein_mv_<fmt>_r<R>_b1 does (the same function, the same sums in the same
-// order: the outputs are the bits of the separate launches).  The matrices may differ in format and
-// in their number of rows; they share in_dim.
+// single-matrix kernel rein_mv_<fmt>_r<R>_b<B> does (the same function, the same sums in the same
+// order: the outputs are the bits of those kernels).  The matrices may differ in format and in their
+// number of rows; they share in_dim and the activation rows.
 #include "matvec_repacked.h"
 
 #define REIN_MULTI_MAX 4
@@ -25,9 +26,9 @@ struct ReinMultiArgs {
     ReinMultiMat m[REIN_MULTI_MAX];
 };
 
-template <int R>
+template <int R, int B>
 __device__ __forceinline__ void rein_matvec_multi_body(const ReinMultiArgs& a, const BlockQ8* __restrict__ xq,
-                                                       unsigned in_dim, unsigned n_mat)
+                                                       unsigned in_dim, unsigned n_mat, unsigned n_rows)
 {
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned wid = blockIdx.x * (blockDim.x >> 6) + wave;
@@ -46,24 +47,32 @@ __device__ __forceinline__ void rein_matvec_multi_body(const ReinMultiArgs& a, c
     // one row group per wavefront: first = g, and a step that ends the walk after it
     const unsigned step = 0x40000000u;
     switch (fmt) {
-    case REIN_Q4_K:   rein_matvec_span<REIN_Q4_K, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
-    case REIN_Q6_K:   rein_matvec_span<REIN_Q6_K, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
-    case REIN_Q5_K:   rein_matvec_span<REIN_Q5_K, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
-    case REIN_Q8_0:   rein_matvec_span<REIN_Q8_0, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
-    case REIN_Q4_0:   rein_matvec_span<REIN_Q4_0, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
-    case REIN_IQ4_XS: rein_matvec_span<REIN_IQ4_XS, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
-    case REIN_IQ3_S:  rein_matvec_span<REIN_IQ3_S, R, 1>(w, xq, y, in_dim, out_dim, 1u, g, step); break;
+    case REIN_Q4_K:   rein_matvec_span<REIN_Q4_K, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
+    case REIN_Q6_K:   rein_matvec_span<REIN_Q6_K, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
+    case REIN_Q5_K:   rein_matvec_span<REIN_Q5_K, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
+    case REIN_Q8_0:   rein_matvec_span<REIN_Q8_0, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
+    case REIN_Q4_0:   rein_matvec_span<REIN_Q4_0, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
+    case REIN_IQ4_XS: rein_matvec_span<REIN_IQ4_XS, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
+    case REIN_IQ3_S:  rein_matvec_span<REIN_IQ3_S, R, B>(w, xq, y, in_dim, out_dim, n_rows, g, step); break;
     default: break;
     }
 }
 
-#define REIN_DEFINE_MATVEC_MULTI(name, R)                                                                    \
+// name(table, xq[n_rows][in_dim / 32], in_dim, n_mat, n_rows): n_rows <= B; y of matrix i is [n_rows][out_dim i]
+#define REIN_DEFINE_MATVEC_MULTI(name, R, B)                                                                 \
     extern "C" __global__ __launch_bounds__(256) void name(ReinMultiArgs a, const BlockQ8* __restrict__ xq,   \
-                                                           unsigned int in_dim, unsigned int n_mat)           \
+                                                           unsigned int in_dim, unsigned int n_mat,           \
+                                                           unsigned int n_rows)                               \
     {                                                                                                        \
-        rein_matvec_multi_body<R>(a, xq, in_dim, n_mat);                                                     \
+        rein_matvec_multi_body<R, B>(a, xq, in_dim, n_mat, n_rows);                                          \
     }
 
-REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r1, 1)
-REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r2, 2)
-REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r4, 4)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r1_b1, 1, 1)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r2_b1, 2, 1)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r4_b1, 4, 1)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r1_b2, 1, 2)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r2_b2, 2, 2)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r4_b2, 4, 2)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r1_b4, 1, 4)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r2_b4, 2, 4)
+REIN_DEFINE_MATVEC_MULTI(rein_mv_multi_r4_b4, 4, 4)

@@ -61,13 +61,13 @@ def matvec_batched_xq8(fmt, w, xq, y, in_dim, out_dim, n_rows, stream=None):
     check(lib.rein_matvec_batched_xq8(fmt, _p(w), _p(xq), _p(y), in_dim, out_dim, n_rows, _s(stream)))
 
 
-def matvec_multi_xq8(fmts, ws, ys, out_dims, xq, in_dim, stream=None):
-    """the decode step's consecutive matvecs on one activation row (Q / K / V, gate / up; src/runtime/qwen35.rs:2670-2672,
-    2702-2703) as one launch: ys[i] = ws[i] . xq"""
+def matvec_multi_xq8(fmts, ws, ys, out_dims, xq, in_dim, n_rows=1, stream=None):
+    """the decode step's consecutive matvecs on the same activations (Q / K / V, gate / up; src/runtime/qwen35.rs:2670-2672,
+    2702-2703) as one launch: ys[i][n_rows][out_dims[i]] = xq . ws[i]^T, up to four matrices and four rows"""
     n = len(fmts)
     check(lib.rein_matvec_multi_xq8(n, (C.c_int * n)(*fmts), (C.c_void_p * n)(*[_p(w) for w in ws]),
                                     (C.c_void_p * n)(*[_p(y) for y in ys]), (C.c_uint * n)(*out_dims), _p(xq), in_dim,
-                                    _s(stream)))
+                                    n_rows, _s(stream)))
 
 
 def matvec_kernel_name(fmt, in_dim, out_dim, n_rows):

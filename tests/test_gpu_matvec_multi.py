@@ -1,7 +1,8 @@
-"""rein_matvec_multi_xq8: the decode step's consecutive matvecs on one activation row (Q / K / V, gate / up;
+"""rein_matvec_multi_xq8: the decode step's consecutive matvecs on the same activations (Q / K / V, gate / up;
 src/runtime/qwen35.rs:2670-2672, 2702-2703) in one launch.  Every output is compared with the oracle and, bit for
-bit, with rein_matvec_xq8 on the same matrix: mixed formats, matrices of very different heights, row counts that
-do not divide by the rows per wavefront, each rows-per-wavefront kernel, and the argument checks."""
+bit, with the launch of that matrix alone (rein_matvec_xq8; at two to four rows the dot4 kernels behind
+rein_matvec_batched_xq8): mixed formats, matrices of very different heights, row counts that do not divide by the
+rows per wavefront, each rows-per-wavefront kernel, and the argument checks."""
 import numpy as np
 import pytest
 
@@ -28,29 +29,39 @@ def bits(a):
     return np.ascontiguousarray(a).view(np.uint32)
 
 
-def check(fmts, in_dim, out_dims, seed=0):
-    print("multi matvec", fmts, in_dim, out_dims, flush=True)
+DOT4_ONLY = (("REIN_MV_LDS", "0"), ("REIN_QUAD_LDS", "0"), ("REIN_SKINNY_FROM", "99"), ("REIN_QUAD_FROM", "99"))
+
+
+def check(fmts, in_dim, out_dims, seed=0, n_rows=1, options=None, one_by_one=False):
+    print("multi matvec", fmts, in_dim, out_dims, n_rows, flush=True)
     packed = [quant.repack_for_matvec(f, random_raw_weights(f, in_dim, n, seed=seed + 7 * i + f), in_dim, n)
               for i, (f, n) in enumerate(zip(fmts, out_dims))]
-    xq = orc.quantize_q8(np.random.default_rng(seed).standard_normal((1, in_dim)).astype(np.float32))
+    xq = orc.quantize_q8(np.random.default_rng(seed).standard_normal((n_rows, in_dim)).astype(np.float32))
     dq = dev(xq)
     dws = [dev(p) for p in packed]
     # one buffer for all outputs with a guard word behind each, so a write past a matrix's rows shows
-    offs = np.concatenate([[0], np.cumsum([n + 1 for n in out_dims])])
+    offs = np.concatenate([[0], np.cumsum([n_rows * n + 1 for n in out_dims])])
     host = np.full(int(offs[-1]), np.float32(-77.0), np.float32)
     dy = dev(host)
-    runtime.matvec_multi_xq8(fmts, dws, [dy.ptr + 4 * int(o) for o in offs[:-1]], out_dims, dq, in_dim)
+    runtime.matvec_multi_xq8(fmts, dws, [dy.ptr + 4 * int(o) for o in offs[:-1]], out_dims, dq, in_dim, n_rows)
     hip.synchronize()
     got = dy.to_host(np.float32)
+    if n_rows > 1 and not one_by_one:    # the few-row launches of one matrix are compared in their dot4 form
+        for name, value in DOT4_ONLY:
+            options.set(name, value)
     for i, (f, n) in enumerate(zip(fmts, out_dims)):
-        mine = got[int(offs[i]):int(offs[i]) + n]
-        assert got[int(offs[i]) + n] == np.float32(-77.0), f"matrix {i} wrote past its rows"
-        want = orc.matvec_q8(f, packed[i], in_dim, n, xq, 1)
-        assert_close_f32(mine.reshape(1, n), want, what=f"multi matrix {i} fmt {f} {in_dim}->{n}")
-        d1 = dev(np.full(n, np.nan, np.float32))
-        runtime.matvec_xq8(f, dws[i], dq, d1, in_dim, n)
+        mine = got[int(offs[i]):int(offs[i]) + n_rows * n].reshape(n_rows, n)
+        assert got[int(offs[i]) + n_rows * n] == np.float32(-77.0), f"matrix {i} wrote past its rows"
+        want = orc.matvec_q8(f, packed[i], in_dim, n, xq, n_rows)
+        assert_close_f32(mine, want, what=f"multi matrix {i} fmt {f} {in_dim}->{n} rows {n_rows}")
+        d1 = dev(np.full(n_rows * n, np.nan, np.float32))
+        runtime.matvec_batched_xq8(f, dws[i], dq, d1, in_dim, n, n_rows)
         hip.synchronize()
-        assert np.array_equal(bits(mine), bits(d1.to_host(np.float32))), f"matrix {i} fmt {f}: not the bits of rein_matvec_xq8"
+        assert np.array_equal(bits(mine), bits(d1.to_host(np.float32).reshape(n_rows, n))), \
+            f"matrix {i} fmt {f} rows {n_rows}: not the bits of the launch of that matrix alone"
+    if n_rows > 1 and not one_by_one:
+        for name, _ in DOT4_ONLY:
+            options.unset(name)
 
 
 @pytest.mark.parametrize("fmts,in_dim,out_dims", [
@@ -73,10 +84,31 @@ def test_multi_matvec_each_rows_per_wavefront(fmt, rows, options):
     options.unset("REIN_MV_ROWS")
 
 
+@pytest.mark.parametrize("n_rows", [2, 3, 4])
+@pytest.mark.parametrize("fmts,in_dim,out_dims", [
+    ([rein.Q4_K, rein.Q4_K, rein.Q6_K], 2048, [1024, 256, 256]),
+    ([rein.Q5_K, rein.Q8_0, rein.IQ4_XS, rein.Q4_0], 768, [67, 5, 130, 33]),
+    ([rein.IQ3_S, rein.Q6_K], 1536, [259, 131]),
+])
+def test_multi_matvec_few_rows(fmts, in_dim, out_dims, n_rows, options):
+    """the two to four rows of a speculative-decode verify step"""
+    check(fmts, in_dim, out_dims, seed=n_rows, n_rows=n_rows, options=options)
+
+
 def test_multi_matvec_decode_shapes():
     """the attention and FFN projections of the 27B-class decoder (hidden 5120, 40 / 8 heads of 128, FFN 17408)"""
     check([rein.Q4_K, rein.Q4_K, rein.Q6_K], 5120, [5120, 1024, 1024], seed=1)
     check([rein.Q4_K, rein.Q4_K], 5120, [17408, 17408], seed=2)
+
+
+def test_multi_matvec_decode_shapes_four_rows(options):
+    check([rein.Q4_K, rein.Q4_K, rein.Q6_K], 5120, [5120, 1024, 1024], seed=4, n_rows=4, options=options)
+
+
+def test_multi_matvec_ffn_sized_matrices_at_four_rows():
+    """three and four rows against matrices of an FFN's size go out as the launches of the matrices one by one"""
+    check([rein.Q4_K, rein.Q4_K], 5120, [8192, 8192], seed=5, n_rows=4, one_by_one=True)
+    check([rein.Q4_K, rein.Q6_K], 5120, [8192, 8192], seed=6, n_rows=3, one_by_one=True)
 
 
 def test_multi_matvec_argument_checks():
@@ -95,3 +127,6 @@ def test_multi_matvec_argument_checks():
         runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, 0], [dy, dy], [4, 4], dq, 256)
     with pytest.raises(ReinError):
         runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, dw], [dy, dy], [4, 4], dq, 200)
+    for rows in (0, 5):
+        with pytest.raises(ReinError):
+            runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, dw], [dy, dy], [4, 4], dq, 256, rows)

@@ -271,8 +271,8 @@ def test_matvec_multi_checks_its_tables_on_the_host():
            dict(fmts=[rein.Q4_K, 99]),                                                 # unknown format
            dict(fmts=[rein.Q4_K, rein.Q5_1]),                                          # an expert-only format
            dict(ws=[4096, 0]), dict(ys=[0, 4096]), dict(ws=[4096, 4100]),              # NULL and misaligned pointers
-           dict(out_dims=[8, 0]), dict(in_dim=200), dict(xq=0)]
+           dict(out_dims=[8, 0]), dict(in_dim=200), dict(xq=0), dict(n_rows=0), dict(n_rows=5)]
     for change in bad:
-        a = dict(ok, **change)
+        a = dict(dict(ok, n_rows=1), **change)
         with pytest.raises(ReinError):
-            runtime.matvec_multi_xq8(a["fmts"], a["ws"], a["ys"], a["out_dims"], a["xq"], a["in_dim"])
+            runtime.matvec_multi_xq8(a["fmts"], a["ws"], a["ys"], a["out_dims"], a["xq"], a["in_dim"], a["n_rows"])
