@@ -941,9 +941,17 @@ int rein_matvec_multi_xq8(unsigned n_mat, const int* fmts, const void* const* ws
     }
     // rows per wavefront and wavefronts per workgroup as the dot4 launch of all the rows in the widest matrix's
     // format would take them
+    // the fewest rows any of the formats would take at this total height, and four only from 16384 rows on: the
+    // wavefronts of the heaviest format finish last (Q + K + V 5120 -> 5120 / 1024 / 1024 with a Q6_K value
+    // projection: 9.6 us at four rows per wavefront, 7.7 at two, 8.7 at one; all Q4_K: 7.7 / 6.9 / 8.1)
     const int lead = fmts[widest];
     const unsigned b = batch_slot(n_rows);
-    const unsigned r = pick_rows_per_wave(lead, (unsigned)total, b);
+    unsigned r = pick_rows_per_wave(lead, (unsigned)total, b);       // two to four rows: the widest matrix's choice (14.1 us against 17.6)
+    for (unsigned i = 0; i < n_mat && b == 1; i++) {
+        unsigned ri = pick_rows_per_wave(fmts[i], (unsigned)total, b);
+        if (ri == 4 && total < 16384 && !opt_is_set(O_MV_ROWS)) ri = 2;
+        r = std::min(r, ri);
+    }
     unsigned wpb = 4;
     if (b == 2 || (lead == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (lead == REIN_TYPE_Q4_K || lead == REIN_TYPE_Q5_K))) wpb = 2;
     const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
