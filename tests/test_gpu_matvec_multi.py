@@ -130,3 +130,18 @@ def test_multi_matvec_argument_checks():
     for rows in (0, 5):
         with pytest.raises(ReinError):
             runtime.matvec_multi_xq8([rein.Q4_K, rein.Q4_K], [dw, dw], [dy, dy], [4, 4], dq, 256, rows)
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_multi_matvec_on_random_tables(seed, options):
+    """seeded tables of two to four matrices, one to four rows, against the oracle and the launches one by one"""
+    rng = np.random.default_rng(seed)
+    for case in range(25):
+        n_mat = int(rng.integers(2, 5))
+        fmts = [DENSE[rng.integers(len(DENSE))] for _ in range(n_mat)]
+        superblocks = any(f not in (rein.Q4_0, rein.Q8_0) for f in fmts) or rng.random() < 0.5
+        in_dim = int(rng.integers(1, 9)) * 256 if superblocks else int(rng.integers(1, 40)) * 32
+        out_dims = [int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(40, 700)), int(rng.integers(700, 4000))]))
+                    for _ in range(n_mat)]
+        n_rows = int(rng.choice([1, 1, 2, 3, 4]))
+        check(fmts, in_dim, out_dims, seed=100 * seed + case, n_rows=n_rows, options=options)
