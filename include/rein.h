@@ -94,7 +94,8 @@ int rein_is_loaded(void);
  * (batched decode of 2..4 rows on the kernel that stages the activation rows in LDS: 0 never,
  * 1 whenever the rows fit), REIN_QUAD_LDS (the same for the 4x4x4 kernel, 3..8 rows),
  * REIN_QUAD_SLICES, REIN_QUAD_DEPTH (wavefronts that share a row group of that kernel, 1..8;
- * trips of weights in flight per wavefront, 1 or 2),
+ * trips of weights in flight per wavefront, 1 or 2), REIN_QUAD_WIDE32 (17..32 rows on that kernel:
+ * 1 the build for sixteen wavefronts per workgroup, 0 the build for eight),
  * REIN_SKINNY_FROM, REIN_SKINNY_KS,
  * REIN_QUAD_FROM (batched decode: row count from which the skinny MMQ / the 4x4x4 kernel run,
  * wavefronts per row tile), REIN_GROUPED_STRIDED (1: the reference-named strided grouped

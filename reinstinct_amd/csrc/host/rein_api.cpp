@@ -140,8 +140,8 @@ int check_ptr(const char* who, const void* p, size_t align, const char* what)
 // rein_set_option changes an entry, so the launch an entry point chooses depends on its arguments
 // and on this table alone.  Entries are single atomic words: setting one while another thread
 // launches is safe, the launch sees the old or the new value.
-enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_QUAD_SLICES, O_QUAD_DEPTH, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
-const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_QUAD_SLICES", "REIN_QUAD_DEPTH", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
+enum Opt : int { O_MV_ROWS, O_MV_WPB, O_MV_LDS, O_QUAD_LDS, O_QUAD_SLICES, O_QUAD_DEPTH, O_QUAD_WIDE32, O_SKINNY_KS, O_SKINNY_FROM, O_QUAD_FROM, O_GROUPED_STRIDED, O_MMQ_TM, O_MMQ_N64, O_MMQ6, O_MMQ6_N4, O_MMQ6_N2, O_MMQ6_SK_GRID, O_MMQ6_SK_SPLIT, O_MMQ6_SK, O_MMQ6_FROM, O_MMQ_SK, O_MMQ_SK_GRID, O_MMQ_SK_SPLIT, O_MMQ_SK_TM, O_MMQ16, O_TOPK_WAVE, O_MOE_SORT_SPLIT, O_MOE_GU_ROWS, O_MOE_DC_ROWS, O_MOE_CHAIN, O_MOE_FUSED, O_COUNT };
+const char* const kOptNames[O_COUNT] = {"REIN_MV_ROWS", "REIN_MV_WPB", "REIN_MV_LDS", "REIN_QUAD_LDS", "REIN_QUAD_SLICES", "REIN_QUAD_DEPTH", "REIN_QUAD_WIDE32", "REIN_SKINNY_KS", "REIN_SKINNY_FROM", "REIN_QUAD_FROM", "REIN_GROUPED_STRIDED", "REIN_MMQ_TM", "REIN_MMQ_N64", "REIN_MMQ6", "REIN_MMQ6_N4", "REIN_MMQ6_N2", "REIN_MMQ6_SK_GRID", "REIN_MMQ6_SK_SPLIT", "REIN_MMQ6_SK", "REIN_MMQ6_FROM", "REIN_MMQ_SK", "REIN_MMQ_SK_GRID", "REIN_MMQ_SK_SPLIT", "REIN_MMQ_SK_TM", "REIN_MMQ16", "REIN_TOPK_WAVE", "REIN_MOE_SORT_SPLIT", "REIN_MOE_GU_ROWS", "REIN_MOE_DC_ROWS", "REIN_MOE_CHAIN", "REIN_MOE_FUSED"};
 constexpr uint64_t kOptSet = 1ull << 63;
 std::atomic<uint64_t> g_opts[O_COUNT];          // zero = unset
 std::once_flag g_opts_env_once;
@@ -404,6 +404,15 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
 // workgroups with one group of four rows per wavefront (5120 rows: five wavefronts, 14336: fourteen); beyond,
 // 512 workgroups of eight wavefronts that stride over the row groups.
 struct QuadLdsGeometry { unsigned wpb, grid, phase_sub, slices; size_t lds; };       // lds == 0: no launch fits
+// Which build of the 32-row kernel: the one for sixteen wavefronts per workgroup (128 registers, a few spilled) lets
+// three wavefronts slice a row group's contraction and wins for every format but Q6_K, whose loop spills 328 bytes
+// there (us at 32 rows, 512-thread build / 1024-thread build: Q4_K 17408 -> 5120 69.9 / 53.3, 5120 -> 5120 25.3 / 22.2,
+// 8192 -> 8192 39.4 / 38.3; Q8_0 66.5 / 53.0, 24.3 / 24.1; Q5_K 73.0 / 55.8, 26.4 / 23.5; Q6_K 87.2 / 121.6, 30.5 / 47.9,
+// 48.7 / 90.5).
+bool mvql_wide32(int fmt)
+{
+    return opt_u(O_QUAD_WIDE32, fmt == REIN_TYPE_Q6_K ? 0u : 1u) != 0;
+}
 QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     const unsigned n_sub = in_dim / 32, t = n_rows <= 4 ? 4 : n_rows <= 8 ? 8 : n_rows <= 16 ? 16 : 32;
@@ -411,11 +420,19 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
     const unsigned groups = (out_dim + 3) / 4;
     QuadLdsGeometry g;
     g.slices = 1;
-    unsigned gpb = std::min(16u, (groups + kCUs - 1) / kCUs);          // row groups per workgroup
+    // the 32-row kernels are built for 512 threads (no spills) and, as rein_mvql_<fmt>_t32w, for 1024
+    const bool wide32 = t == 32 && mvql_wide32(fmt);
+    const unsigned max_wpb = t == 32 && !wide32 ? 8 : 16;
+    unsigned gpb = std::min(max_wpb, (groups + kCUs - 1) / kCUs);      // row groups per workgroup
+    // 32 rows: every workgroup stages all 32 activation rows (700 KB at in_dim 17408, in phases), more than its share of
+    // the weights, so fewer and fuller workgroups win as long as 160 CUs have one: 5120 rows as 160 workgroups of
+    // eight wavefronts instead of 256 of five (us: Q4_K 17408 -> 5120 67.1 -> 64.2, 5120 -> 5120 24.7 -> 24.0; Q6_K
+    // 85.6 -> 82.8, 30.6 -> 29.6)
+    if (t == 32 && !wide32 && groups >= 8 * 160) gpb = 8;
     const bool persistent = groups > kCUs * 16;
     const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
-    if (wpb_forced >= 1 && wpb_forced <= 16) gpb = wpb_forced;
-    if (persistent && !(wpb_forced >= 1 && wpb_forced <= 16)) { g.wpb = 8; g.grid = 2 * kCUs; }
+    if (wpb_forced >= 1 && wpb_forced <= max_wpb) gpb = wpb_forced;
+    if (persistent && !(wpb_forced >= 1 && wpb_forced <= max_wpb)) { g.wpb = 8; g.grid = 2 * kCUs; }
     else {
         // few row groups per CU: several wavefronts share a row group, each taking every slices-th trip
         // (us, Q4_K at 8 rows, slices 1 / 2 / 3-4: 17408 -> 5120 28.7 / 21.1 / 19.9, 14336 -> 4096 22.5 / 16.1 / 14.6,
@@ -425,7 +442,7 @@ QuadLdsGeometry mvql_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsign
         const unsigned want = opt_u(O_QUAD_SLICES, 0);
         const unsigned trips = (n_sub + 15) / 16;
         g.slices = want >= 1 && want <= 8 ? want : std::min(8u, std::max(1u, trips / 2));
-        g.slices = std::max(1u, std::min(g.slices, 16u / gpb));
+        g.slices = std::max(1u, std::min(g.slices, max_wpb / gpb));
         g.slices = std::min(g.slices, std::max(1u, trips));
         g.wpb = gpb * g.slices;
         g.grid = (groups + gpb - 1) / gpb;
@@ -511,7 +528,8 @@ int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned i
                     unsigned n_rows, rein_stream_t s)
 {
     const QuadLdsGeometry g = mvql_geometry(fmt, in_dim, out_dim, n_rows);
-    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" : "_t32");
+    const std::string name = std::string("rein_mvql_") + fmt_tag(fmt) + (n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" :
+                                                                         mvql_wide32(fmt) ? "_t32w" : "_t32");
     // Trips of weights in flight per wavefront where wavefronts stride over row groups or own a whole one (no slices,
     // no phases): two for the formats with little arithmetic per sub-block at 3-4 rows -- two register sets taking
     // turns -- (us, 5120 -> 34816 / 5120 -> 17408 / 3584 -> 18944 at 4 rows, one -> two: Q4_K 28.3 -> 26.0, 18.8 -> 17.3,
@@ -553,7 +571,7 @@ MvFamily matvec_family(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_ro
 std::string matvec_kernel_name(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     const std::string tag = fmt_tag(fmt);
-    const std::string t = n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" : "_t32";
+    const std::string t = n_rows <= 4 ? "_t4" : n_rows <= 8 ? "_t8" : n_rows <= 16 ? "_t16" : mvql_wide32(fmt) ? "_t32w" : "_t32";
     if (n_rows > 8) {
         if (n_rows <= 32 && use_mvql(fmt, in_dim, out_dim, n_rows)) return "rein_mvql_" + tag + t;
         if (n_rows <= 16 && in_dim >= 256 && skinny_from_rows(fmt) <= 16) return "rein_mmqs_" + tag + "_v8";
@@ -1526,7 +1544,7 @@ int rein_noalloc_prepare(void)
     static const int fmts[] = {REIN_TYPE_Q4_0, REIN_TYPE_Q4_K, REIN_TYPE_Q5_K, REIN_TYPE_Q6_K, REIN_TYPE_Q8_0, REIN_TYPE_IQ4_XS};
     static const char* const forms[] = {"_t32", "_t64", "_mix", "_sk", "_sk32"};
     // (up to 32 rows the entry point launches the few-row kernels)
-    static const char* const few[] = {"rein_mmqs_%s_v1", "rein_mmqs_%s_v2", "rein_mmqs_%s_v4", "rein_mmqs_%s_v8", "rein_mvql_%s_t16", "rein_mvql_%s_t32"};
+    static const char* const few[] = {"rein_mmqs_%s_v1", "rein_mmqs_%s_v2", "rein_mmqs_%s_v4", "rein_mmqs_%s_v8", "rein_mvql_%s_t16", "rein_mvql_%s_t32", "rein_mvql_%s_t32w"};
     for (int fmt : fmts) {
         for (const char* form : forms) {
             hipFunction_t f;

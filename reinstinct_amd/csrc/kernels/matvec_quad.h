@@ -269,6 +269,9 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
     constexpr bool kTwo = F::kDotParts == 2;
     constexpr int kParts = QuadRawBits<FMT>::kParts;
     constexpr unsigned T = 4u * NT;
+    // the second register set of weights (depth 2) exists for 3-8 rows only: at 16 and 32 rows the code of its loops costs
+    // the one-set loops registers (32 rows 17408 -> 5120: 57 -> 64 us for Q4_K, 131 -> 159 for Q6_K with it compiled in)
+    constexpr bool kTwoSets = NT <= 2;
     static_assert(kParts * 76 * 16 >= NT * 16 * 4, "a wavefront's partial sums go through its weight image");
     extern __shared__ uint4 rein_mvql_lds[];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wpb = blockDim.x >> 6;
@@ -391,7 +394,7 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
             const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
             rq = fmt.load(row, min(ls, n_sub - 1u));
         }
-        if (depth >= 2u) {
+        if (kTwoSets && depth >= 2u) {
             // two trips of weights in flight per wavefront: two register sets take turns, each refilled with the trip
             // after next as soon as its own has gone to LDS
             struct Pos { unsigned g, sb0; };
@@ -441,7 +444,7 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
         const unsigned g = blockIdx.x * gpb + wave / slices;
         const bool has = wave < gpb * slices && g < n_groups;    // wave-uniform
         const unsigned ahead = 16u * slices;
-        const bool two = depth >= 2u;                            // two register sets of weights taking turns
+        const bool two = kTwoSets && depth >= 2u;                // two register sets of weights taking turns
         Raw rq2;
         {
             const unsigned row = min(min(g, n_groups - 1u) * 4u + lr, out_dim - 1u);
@@ -496,8 +499,11 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
 }
 
 // name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub, slices, depth), n_rows <= 4 * NT
-#define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT)                                                \
-    extern "C" __global__ __launch_bounds__(1024) void name(                                      \
+// (32 rows: eight wavefronts per workgroup at most, so that the 32 partial sums and the eight activation tiles of a
+// trip stay in registers -- with sixteen wavefronts' 128 registers the loop spills)
+#define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT) REIN_DEFINE_MATVEC_QUAD_LDS_BOUND(name, FMT, NT, (NT >= 8 ? 512 : 1024))
+#define REIN_DEFINE_MATVEC_QUAD_LDS_BOUND(name, FMT, NT, BOUND)                                   \
+    extern "C" __global__ __launch_bounds__(BOUND) void name(                                     \
         const uint8_t* __restrict__ w, const BlockQ8* __restrict__ xq, float* __restrict__ y,    \
         unsigned int in_dim, unsigned int out_dim, unsigned int n_rows, unsigned int phase_sub,   \
         unsigned int slices, unsigned int depth)                                                  \

@@ -200,9 +200,13 @@ def test_lds_quad_nine_to_sixteen_rows(fmt, in_dim, out_dim, slices, options):
 @pytest.mark.parametrize("fmt", DENSE)
 @pytest.mark.parametrize("in_dim,out_dim", [(2048, 389), (512, 3), (5120, 130), (2304, 4099), (17408, 70)])
 @pytest.mark.parametrize("slices", ["1", None])
-def test_lds_quad_seventeen_to_thirty_two_rows(fmt, in_dim, out_dim, slices, options):
-    # rein_mvql_<fmt>_t32 behind rein_mmq_xq8 (the 32-token tile launch otherwise); 32 rows x 5120 values take two phases
+@pytest.mark.parametrize("wide", ["0", "1"])
+def test_lds_quad_seventeen_to_thirty_two_rows(fmt, in_dim, out_dim, slices, wide, options):
+    # rein_mvql_<fmt>_t32 / _t32w (the builds for eight and for sixteen wavefronts per workgroup) behind rein_mmq_xq8
+    # (the 32-token tile launch otherwise); 32 rows x 5120 values take two phases
+    options.set("REIN_QUAD_WIDE32", wide)
     check_quad_lds(options, fmt, in_dim, out_dim, rows=(17, 24, 32), slices=slices)
+    options.unset("REIN_QUAD_WIDE32")
 
 
 @pytest.mark.parametrize("fmt", DENSE)

@@ -238,7 +238,8 @@ def test_matvec_kernel_name_follows_the_dispatch_rules():
     # nine and more rows arrive through rein_mmq_xq8
     assert name(rein.Q6_K, 5120, 5120, 12) == "rein_mvql_q6k_t16"
     assert name(rein.Q4_K, 5120, 5120, 12) == "rein_mmqs_q4k_v8"
-    assert name(rein.Q4_K, 5120, 5120, 32) == "rein_mvql_q4k_t32"
+    assert name(rein.Q4_K, 5120, 5120, 32) == "rein_mvql_q4k_t32w"            # the build for sixteen wavefronts
+    assert name(rein.Q6_K, 5120, 5120, 32) == "rein_mvql_q6k_t32"             # Q6_K: the build for eight
     assert name(rein.Q4_K, 5120, 34816, 32) == ""                             # token tiles
     assert name(rein.Q4_K, 5120, 5120, 33) == ""
     # options pin a family
