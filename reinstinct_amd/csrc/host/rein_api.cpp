@@ -405,7 +405,7 @@ int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned
 // 512 workgroups of eight wavefronts that stride over the row groups.
 struct QuadLdsGeometry { unsigned wpb, grid, phase_sub, slices; size_t lds; };       // lds == 0: no launch fits
 // Which build of the 32-row kernel: the one for sixteen wavefronts per workgroup (128 registers, a few spilled) lets
-// three wavefronts slice a row group's contraction and wins for every format but Q6_K, whose loop spills 328 bytes
+// three wavefronts slice a row group's contraction and wins for every format but Q6_K, whose loop spills 204 bytes
 // there (us at 32 rows, 512-thread build / 1024-thread build: Q4_K 17408 -> 5120 69.9 / 53.3, 5120 -> 5120 25.3 / 22.2,
 // 8192 -> 8192 39.4 / 38.3; Q8_0 66.5 / 53.0, 24.3 / 24.1; Q5_K 73.0 / 55.8, 26.4 / 23.5; Q6_K 87.2 / 121.6, 30.5 / 47.9,
 // 48.7 / 90.5).

@@ -499,8 +499,9 @@ __device__ __forceinline__ void rein_matvec_quad_lds_body(const uint8_t* __restr
 }
 
 // name(w, xq[n_rows][n_sub], y[n_rows][out_dim], in_dim, out_dim, n_rows, phase_sub, slices, depth), n_rows <= 4 * NT
-// (32 rows: eight wavefronts per workgroup at most, so that the 32 partial sums and the eight activation tiles of a
-// trip stay in registers -- with sixteen wavefronts' 128 registers the loop spills)
+// (32 rows: by default for eight wavefronts per workgroup at most, so that the 32 partial sums and the eight activation
+// tiles of a trip stay in registers; REIN_DEFINE_MATVEC_QUAD_LDS_BOUND builds it for sixteen wavefronts' 128 registers as
+// well, where the heavier formats spill)
 #define REIN_DEFINE_MATVEC_QUAD_LDS(name, FMT, NT) REIN_DEFINE_MATVEC_QUAD_LDS_BOUND(name, FMT, NT, (NT >= 8 ? 512 : 1024))
 #define REIN_DEFINE_MATVEC_QUAD_LDS_BOUND(name, FMT, NT, BOUND)                                   \
     extern "C" __global__ __launch_bounds__(BOUND) void name(                                     \
