@@ -145,3 +145,29 @@ def test_multi_matvec_on_random_tables(seed, options):
                     for _ in range(n_mat)]
         n_rows = int(rng.choice([1, 1, 2, 3, 4]))
         check(fmts, in_dim, out_dims, seed=100 * seed + case, n_rows=n_rows, options=options)
+
+
+def test_multi_matvec_in_a_captured_graph():
+    """the argument table travels by value with the launch: a captured call replays with the tables of the capture,
+    whatever the host arrays hold afterwards"""
+    fmts, in_dim, out_dims = [rein.Q4_K, rein.Q6_K, rein.Q8_0], 1536, [300, 77, 129]
+    packed = [quant.repack_for_matvec(f, random_raw_weights(f, in_dim, n, seed=40 + i), in_dim, n)
+              for i, (f, n) in enumerate(zip(fmts, out_dims))]
+    xq = orc.quantize_q8(np.random.default_rng(40).standard_normal((1, in_dim)).astype(np.float32))
+    dq, dws = dev(xq), [dev(p) for p in packed]
+    dys = [dev(np.full(n, np.nan, np.float32)) for n in out_dims]
+    stream = hip.Stream()
+    stream.begin_capture()
+    runtime.matvec_multi_xq8(fmts, dws, dys, out_dims, dq, in_dim, 1, stream)
+    exe = stream.end_capture().instantiate()
+    for replay in range(3):
+        for dy, n in zip(dys, out_dims):
+            dy.copy_from_host(np.zeros(n, np.float32))
+        hip.synchronize()
+        exe.launch(stream)
+        stream.synchronize()
+        for i, (f, n) in enumerate(zip(fmts, out_dims)):
+            d1 = dev(np.full(n, np.nan, np.float32))
+            runtime.matvec_xq8(f, dws[i], dq, d1, in_dim, n)
+            hip.synchronize()
+            assert np.array_equal(bits(dys[i].to_host(np.float32)), bits(d1.to_host(np.float32))), f"replay {replay} matrix {i}"
