@@ -196,6 +196,27 @@ unsigned pick_rows_per_wave(int fmt, unsigned out_dim, unsigned batch)
 
 unsigned batch_slot(unsigned n_rows) { return n_rows <= 1 ? 1 : n_rows <= 2 ? 2 : n_rows <= 4 ? 4 : 8; }
 
+// Wavefronts per workgroup of the dot4 matvec (they share nothing): four, or two where the finer grain deals the
+// wavefronts more evenly over the CUs -- every format at two activation rows (Q4_K 17408 -> 5120: 18.5 -> 15.4 us,
+// 5120 -> 5120: 7.5 -> 6.7; IQ3_S 16.4 -> 14.5), Q8_0 also at one (19.8 -> 17.1, 7.1 -> 6.5), and one to three percent for
+// Q4_K / Q5_K at one row; Q4_0, IQ4_XS and IQ3_S at one row lose 3-10 % on 5120 -> 5120 and stay at four.
+// The workgroups of a launch this short are all resident at once, so a CU that holds three workgroups of four
+// wavefronts beside CUs that hold two ends 20 % late (5120 rows at two rows per wavefront: 640 workgroups of four, 1280
+// of two).  At one row the pairs are taken only where they even the deal out by more than 3 %; otherwise four wavefronts
+// halve the workgroups to start (us, two -> four: Q4_K 2048 -> 5632 4.17 -> 3.58, 4096 -> 6144 5.44 -> 4.94, 16384 -> 6144
+// 13.9 -> 12.9; Q5_K 4.44 -> 3.85, 6.24 -> 5.68; Q8_0 4.62 -> 4.18; 48 cells of three formats x 16 shapes then sit within
+// 3 % of the better of the two).
+unsigned pick_wpb(int fmt, unsigned groups, unsigned b)
+{
+    const unsigned forced = opt_u(O_MV_WPB, 0);
+    if (forced == 1 || forced == 2 || forced == 4) return forced;
+    const auto uneven = [&](unsigned w) { const unsigned n = (groups + w - 1) / w; return (double)((n + kCUs - 1) / kCUs * kCUs) / n; };
+    unsigned wpb = 4;
+    if (b == 2 || (fmt == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q5_K))) wpb = 2;
+    if (wpb == 2 && b == 1 && !(uneven(2) < uneven(4) - 0.03)) wpb = 4;
+    return wpb;
+}
+
 // Skinny MMQ launch: grid.x = 32-row tiles, grid.y = token groups, block = KS
 // wavefronts that split the contraction of one tile.  The kernels keep several
 // chunks of weights in flight in registers, which leaves room for two or three
@@ -614,15 +635,8 @@ int launch_matvec(const char* who, int fmt, const void* w, const void* xq, float
     if (family == MvFamily::Skinny) return launch_skinny(fmt, w, xq, y, in_dim, out_dim, n_rows, s);
     const unsigned b = batch_slot(n_rows);
     const unsigned r = pick_rows_per_wave(fmt, out_dim, b);
-    // Wavefronts per workgroup (they share nothing): four, or two where the finer grain deals the wavefronts more
-    // evenly over the CUs -- every format at two activation rows (Q4_K 17408 -> 5120: 18.5 -> 15.4 us, 5120 -> 5120:
-    // 7.5 -> 6.7; IQ3_S 16.4 -> 14.5), Q8_0 also at one (19.8 -> 17.1, 7.1 -> 6.5), and one to three percent for
-    // Q4_K / Q5_K at one row; Q4_0, IQ4_XS and IQ3_S at one row lose 3-10 % on 5120 -> 5120 and stay at four
-    unsigned wpb = 4;
-    if (b == 2 || (fmt == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q5_K))) wpb = 2;
-    const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
-    if (wpb_forced == 1 || wpb_forced == 2 || wpb_forced == 4) wpb = wpb_forced;
     const unsigned groups = (out_dim + r - 1) / r;
+    const unsigned wpb = pick_wpb(fmt, groups, b);
     const unsigned grid = (groups + wpb - 1) / wpb;
     const std::string name = std::string("rein_mv_") + fmt_tag(fmt) + "_r" + std::to_string(r) + "_b" + std::to_string(b);
     void* args[] = {(void*)&w, (void*)&xq, (void*)&y, (void*)&in_dim, (void*)&out_dim, (void*)&n_rows};
@@ -970,10 +984,6 @@ int rein_matvec_multi_xq8(unsigned n_mat, const int* fmts, const void* const* ws
         if (ri == 4 && total < 16384 && !opt_is_set(O_MV_ROWS)) ri = 2;
         r = std::min(r, ri);
     }
-    unsigned wpb = 4;
-    if (b == 2 || (lead == REIN_TYPE_Q8_0 && b <= 2) || (b == 1 && (lead == REIN_TYPE_Q4_K || lead == REIN_TYPE_Q5_K))) wpb = 2;
-    const unsigned wpb_forced = opt_u(O_MV_WPB, 0);
-    if (wpb_forced == 1 || wpb_forced == 2 || wpb_forced == 4) wpb = wpb_forced;
     struct Mat { const void* w; float* y; unsigned out_dim; int fmt; unsigned group_end; unsigned pad; };
     struct Args { Mat m[kMax]; } a{};
     unsigned groups = 0;
@@ -982,6 +992,7 @@ int rein_matvec_multi_xq8(unsigned n_mat, const int* fmts, const void* const* ws
         a.m[i] = Mat{ws[i], ys[i], out_dims[i], fmts[i], groups, 0u};
     }
     for (unsigned i = n_mat; i < kMax; i++) a.m[i] = a.m[n_mat - 1];
+    const unsigned wpb = pick_wpb(lead, groups, b);
     void* args[] = {(void*)&a, (void*)&xq, (void*)&in_dim, (void*)&n_mat, (void*)&n_rows};
     return launch("rein_mv_multi_r" + std::to_string(r) + "_b" + std::to_string(b), (groups + wpb - 1) / wpb, 1, 1, wpb * 64, 0, s, args);
 }
