@@ -1552,10 +1552,12 @@ int rein_noalloc_prepare(void)
         hipFunction_t f;
         if (int rc = get_fn(n, &f)) return rc;
     }
-    static const int fmts[] = {REIN_TYPE_Q4_0, REIN_TYPE_Q4_K, REIN_TYPE_Q5_K, REIN_TYPE_Q6_K, REIN_TYPE_Q8_0, REIN_TYPE_IQ4_XS};
+    static const int fmts[] = {REIN_TYPE_Q4_0, REIN_TYPE_Q4_K, REIN_TYPE_Q5_K, REIN_TYPE_Q6_K, REIN_TYPE_Q8_0, REIN_TYPE_IQ4_XS, REIN_TYPE_IQ3_S};
     static const char* const forms[] = {"_t32", "_t64", "_mix", "_sk", "_sk32"};
-    // (up to 32 rows the entry point launches the few-row kernels)
-    static const char* const few[] = {"rein_mmqs_%s_v1", "rein_mmqs_%s_v2", "rein_mmqs_%s_v4", "rein_mmqs_%s_v8", "rein_mvql_%s_t16", "rein_mvql_%s_t32", "rein_mvql_%s_t32w"};
+    // (up to 32 rows the entry point launches the few-row kernels: skinny MMQ, both 4x4x4 kernels, and from eight rows
+    // down the decode matvecs in every rows-per-wavefront x batch-slot instantiation there is)
+    static const char* const few[] = {"rein_mmqs_%s_v1", "rein_mmqs_%s_v2", "rein_mmqs_%s_v4", "rein_mmqs_%s_v8", "rein_mvql_%s_t4", "rein_mvql_%s_t8",
+                                      "rein_mvql_%s_t16", "rein_mvql_%s_t32", "rein_mvql_%s_t32w", "rein_mvq_%s_t4", "rein_mvq_%s_t8"};
     for (int fmt : fmts) {
         for (const char* form : forms) {
             hipFunction_t f;
@@ -1567,6 +1569,14 @@ int rein_noalloc_prepare(void)
             hipFunction_t f;
             if (int rc = get_fn(name, &f)) return rc;
         }
+        for (unsigned r = 1; r <= 4; r *= 2)
+            for (unsigned b = 1; b <= 8; b *= 2) {
+                hipFunction_t f;
+                if (r * b <= 16)
+                    if (int rc = get_fn(std::string("rein_mv_") + fmt_tag(fmt) + "_r" + std::to_string(r) + "_b" + std::to_string(b), &f)) return rc;
+                if (b == 2 || b == 4)
+                    if (int rc = get_fn(std::string("rein_mvl_") + fmt_tag(fmt) + "_r" + std::to_string(r) + "_b" + std::to_string(b), &f)) return rc;
+            }
     }
     return 0;
 }

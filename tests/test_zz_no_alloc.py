@@ -106,6 +106,41 @@ def test_no_alloc_entry_under_stream_capture_and_without_touching_device_memory(
     assert free_mid >= free_before - (4 << 20), "the graph objects aside, nothing may have been allocated"
 
 
+@pytest.mark.parametrize("fmt,p_rows,in_dim,out_dim", [(rein.IQ3_S, 4, 1536, 1030), (rein.Q5_K, 12, 2304, 520), (rein.Q6_K, 24, 1280, 2052),
+                                                        (rein.Q8_0, 2, 8192, 4100), (rein.Q4_0, 7, 1056, 16390)])
+def test_no_alloc_entry_with_few_rows_under_stream_capture(fmt, p_rows, in_dim, out_dim):
+    # up to 32 rows the entry point launches the few-row kernels (decode matvecs, skinny MMQ, the 4x4x4 kernels), whose
+    # handles rein_noalloc_prepare has looked up as well: the first call of a shape may already be a recorded one
+    init()
+    hip.set_device(0)
+    runtime.noalloc_prepare()
+    print(f"no-alloc entry, few rows under capture: fmt {fmt} P {p_rows} K {in_dim} N {out_dim}", flush=True)
+    dw = dev(quant.repack_for_matvec(fmt, random_raw_weights(fmt, in_dim, out_dim, 21), in_dim, out_dim))
+    x = np.random.default_rng(21).standard_normal((p_rows, in_dim)).astype(np.float32)
+    d_x, dq = dev(x), hip.DeviceBuf(p_rows * (in_dim // 32) * 40)
+    runtime.quantize_q8(d_x, dq, in_dim, p_rows)
+    hip.synchronize()
+    d_graph = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    stream = hip.Stream()
+    stream.begin_capture()
+    runtime.mmq_xq8_noalloc(fmt, dw, dq, d_graph, in_dim, out_dim, p_rows, stream)
+    exe = stream.end_capture().instantiate()
+    d_eager = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    d_ws = dev(np.full(p_rows * out_dim, np.nan, np.float32))
+    for replay in range(2):
+        d_graph.copy_from_host(np.zeros(p_rows * out_dim, np.float32))
+        hip.synchronize()
+        exe.launch(stream)
+        stream.synchronize()
+        # the eager call of the same entry point, and rein_mmq_xq8_ws with a workspace of the array's size, between the replays
+        runtime.mmq_xq8_noalloc(fmt, dw, dq, d_eager, in_dim, out_dim, p_rows, stream)
+        ws = hip.DeviceBuf(SCRATCH_BYTES)
+        runtime.mmq_xq8_ws(fmt, dw, dq, d_ws, in_dim, out_dim, p_rows, ws, SCRATCH_BYTES, stream)
+        stream.synchronize()
+        assert np.array_equal(d_graph.to_host(np.uint32), d_eager.to_host(np.uint32)), f"replay {replay} differs from the eager call"
+        assert np.array_equal(d_graph.to_host(np.uint32), d_ws.to_host(np.uint32)), f"replay {replay} differs from rein_mmq_xq8_ws"
+
+
 def test_no_alloc_entry_refuses_what_the_fixed_array_cannot_hold():
     init()
     hip.set_device(0)
