@@ -651,6 +651,27 @@ def read_ceiling_us(stream, weights, nbytes):
     return best * 1e6
 
 
+def extras_barrier_cost(stream):
+    """What a barrier across the workgroups of one launch costs through device memory (rein_measure_barrier, a
+    measurement kernel in the code object: one workgroup per CU, nothing but the barrier, every wait bounded),
+    per launch in a graph of 32 launches, beside an empty launch of the same shape: the price a persistent
+    kernel would pay where the graph pays a launch boundary."""
+    import ctypes as C
+    f = hip.Module.builtin().function("rein_measure_barrier")
+    out = hip.DeviceBuf.from_host(np.zeros(2, np.uint32))
+    res = {}
+    for grid, block in ((256, 1024), (256, 64), (64, 1024)):
+        for mode, name in ((0, "empty"), (1, "every_workgroup_polls_every_flag"), (2, "one_gathers_the_others_poll_a_word"),
+                           (3, "the_same_without_the_l2_write_back")):
+            sec = time_graph(stream, lambda: [f.launch((grid, 1, 1), (block, 1, 1), 0, stream,
+                                                       [C.c_uint(mode), C.c_uint(1 << 16), C.c_void_p(out.ptr)]) for _ in range(32)], 32)
+            res[f"{grid}x{block}_{name}_us"] = round(sec * 1e6, 2)
+    gave_up = int(out.to_host(np.uint32)[1])
+    res["a_wait_gave_up"] = bool(gave_up)
+    log("barrier cost", res)
+    return res
+
+
 def decode_sweep(stream, steps):
     """BASELINE configs[1] as a sweep: Q4_K and Q6_K over the three decode shapes at batch 1, 2, 4, 8, the
     other four formats at the gate+up shape; every cell over its own rotation of > 512 MB of weights.
@@ -822,7 +843,8 @@ def main():
     if args.extras:
         out["extras"] = {"fused_producers": extras_fused(stream),
                          "other_matvec_sites": extras_ondisk(stream),
-                         "decode_ffn_chain": extras_decode_ffn(stream)}
+                         "decode_ffn_chain": extras_decode_ffn(stream),
+                         "barrier_cost": extras_barrier_cost(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)

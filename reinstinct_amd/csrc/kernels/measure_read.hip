@@ -25,3 +25,61 @@ extern "C" __global__ __launch_bounds__(256) void rein_measure_read16(const rein
     }
     if (acc == 0x12345678u) sink[0] = 1u;            // keeps the loads alive; practically never taken
 }
+
+// Measurement kernel, not part of the path: what a barrier across all workgroups of a launch costs on this
+// machine when it goes through device memory (the L2s of the XCDs are not coherent with each other, so flags
+// that every CU must see are agent-scope accesses that go to memory).  Launched with one workgroup per CU
+// (all resident at once), it does nothing but the barrier; every wait is bounded by spin_limit polls, after
+// which a workgroup sets out[1] and leaves, so every wavefront ends whatever happens.  The words are never
+// reset: a launch reads the generation g, stores g + 1 to its flags, and workgroup 0 publishes g + 1 as the
+// next generation once it has seen every flag, so launches replay.
+//   mode 0  no barrier (an empty launch of the same shape)
+//   mode 1  every workgroup polls every flag
+//   mode 2  workgroup 0 gathers the flags into one word that the others poll
+//   mode 3  mode 2 without the release's L2 write-back in front of the flag store
+struct ReinMeasureSync {
+    unsigned gen, open, pad[62];
+    unsigned flag[1024];
+};
+__device__ ReinMeasureSync rein_measure_sync;
+
+extern "C" __global__ __launch_bounds__(1024) void rein_measure_barrier(unsigned int mode, unsigned int spin_limit,
+                                                                        unsigned int* __restrict__ out)
+{
+    __shared__ unsigned open_s;
+    if (mode == 0u || gridDim.x > 1024u) return;
+    ReinMeasureSync& S = rein_measure_sync;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned gen = __hip_atomic_load(&S.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0u) {
+        if (mode != 3u) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (lane == 0u) __hip_atomic_store(&S.flag[blockIdx.x], gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned open = 0u;
+        if (mode == 1u || blockIdx.x == 0u) {
+            for (unsigned s = 0; s < spin_limit; s++) {
+                bool all = true;
+                for (unsigned i = lane; i < gridDim.x; i += 64u)
+                    all = all && __hip_atomic_load(&S.flag[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gen + 1u;
+                if (__all(all)) { open = 1u; break; }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (mode != 1u && open && lane == 0u) __hip_atomic_store(&S.open, gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            for (unsigned s = 0; s < spin_limit; s++) {
+                if (__hip_atomic_load(&S.open, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gen + 1u) { open = 1u; break; }
+                __builtin_amdgcn_s_sleep(2);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (lane == 0u) open_s = open;
+    }
+    __syncthreads();
+    if (open_s == 0u) {
+        if (threadIdx.x == 0u) out[1] = 1u;
+        return;
+    }
+    if (blockIdx.x == 0u && threadIdx.x == 0u) {
+        __hip_atomic_store(&S.gen, gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        out[0] = gen + 1u;
+    }
+}

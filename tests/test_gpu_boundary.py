@@ -211,3 +211,28 @@ def test_config0_q4k_4096_by_4096():
     assert np.array_equal(dd.to_host(np.int32).reshape(dots.shape), dots)
     f32 = orc.matvec_f32(x[0], orc.dequantize_to_f32(orc.Q4_K, raw, in_dim * out_dim).reshape(out_dim, in_dim))
     assert rel_l2(got[0], f32) < 5e-2
+
+
+def test_barrier_measurement_kernel_always_ends():
+    """rein_measure_barrier (bench.py --extras): with polls allowed every workgroup passes and the generation advances by
+    one per launch; with none allowed every workgroup gives up, says so, and still ends"""
+    import ctypes as C
+    f = hip.Module.builtin().function("rein_measure_barrier")
+    out = hip.DeviceBuf.from_host(np.zeros(2, np.uint32))
+    stream = hip.Stream()
+
+    def launch(mode, spins, grid=256, block=1024):
+        f.launch((grid, 1, 1), (block, 1, 1), 0, stream, [C.c_uint(mode), C.c_uint(spins), C.c_void_p(out.ptr)])
+        stream.synchronize()
+        return out.to_host(np.uint32)
+
+    first = int(launch(1, 1 << 16)[0])
+    for i, mode in enumerate((2, 3, 1, 2), start=1):
+        got = launch(mode, 1 << 16)
+        assert int(got[0]) == first + i and int(got[1]) == 0
+    got = launch(2, 0)                                   # no poll allowed: the wait gives up at once
+    assert int(got[1]) == 1 and int(got[0]) == first + 4
+    out.copy_from_host(np.zeros(2, np.uint32))
+    # the flags of the launch that gave up hold the next generation already; the launch after it passes
+    got = launch(1, 1 << 16, grid=64)
+    assert int(got[1]) == 0
