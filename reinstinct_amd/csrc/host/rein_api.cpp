@@ -325,7 +325,9 @@ bool small_for_matrix_cores(int fmt, unsigned in_dim, unsigned out_dim, unsigned
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
     if (n_rows > 4) return weights <= (6ull << 20);
     const bool quad_family = fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS;
-    return out_dim <= 2048 || (!quad_family && weights <= (1ull << 24));
+    // (... except short contractions against 8192 rows and more, which the 4x4x4 kernel takes: 1536 -> 8960 at 4 rows Q4_K
+    // 7.3 -> 5.6 us, Q8_0 7.7 -> 6.4)
+    return out_dim <= 2048 || (!quad_family && weights <= (1ull << 24) && out_dim < 8192);
 }
 
 // LDS-staged dot4 matvec (rein_mvl_*, kernels/matvec_lds.h), 2..4 activation rows: the rows of a
@@ -391,6 +393,29 @@ void mvl_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, u
 //             more (5120 -> 34816 1.13 / 1.08 / 1.06, 5120 -> 17408 1.17 / 1.14 / 1.09, 3584 -> 18944 1.16 / 1.13 /
 //             1.05, 4096 -> 14336 1.04 / 1.08 / 1.03) and IQ3_S (1.05-1.14); Q6_K 0.91-1.10, IQ4_XS 0.97-1.06, Q8_0
 //             0.95-1.08 there.
+// Three and four rows on the 4x4x4 kernel with the rows in LDS (the shape part of use_mvql's rule, shared with use_mvl):
+//   * up to 8192 rows and from 20 * 2^20 weights, every format but Q8_0 (contraction sliced over wavefronts);
+//   * Q6_K with a long contraction against very few rows (us at 4 rows, dot4 / LDS dot4 / this: 8192 -> 1024 10.5 / 9.4 /
+//     7.0, 8960 -> 1536 14.9 / 10.6 / 9.3);
+//   * between 8192 and 14336 rows: Q4_K, Q5_K, Q6_K and their kin (5120 -> 13824 at 4 rows, 4x4x4 without LDS -> this: Q4_K
+//     14.0 -> 12.4, Q5_K 17.7 -> 14.7; 8192 -> 10240, LDS dot4 -> this: 16.8 -> 15.6, 20.0 -> 19.1, Q6_K 24.5 -> 21.9), Q8_0
+//     from 12288 rows (19.8 -> 17.1; 8192 -> 10240 21.4 on LDS dot4 against 22.9);
+//   * from 14336 rows: the formats with a cheap unpack and Q5_K.
+bool mvql_few_rows(int fmt, unsigned in_dim, unsigned out_dim)
+{
+    const unsigned long long weights = (unsigned long long)in_dim * out_dim;
+    if (fmt != REIN_TYPE_Q8_0 && out_dim <= 8192 && weights >= (20ull << 20)) return true;
+    if (fmt == REIN_TYPE_Q6_K && weights >= (6ull << 20) && in_dim >= 8192 && out_dim <= 1536) return true;
+    // (short contractions against 8192 rows and more, below 2^24 weights: 1536 -> 8960 at 4 rows, us, dot4 / 4x4x4 / this:
+    // Q4_K 7.3 / 5.6 / 5.6, Q8_0 7.7 / 6.4 / 6.4, Q6_K 10.2 / 6.9 / 6.6, IQ3_S 6.6 / 5.7 / 5.4, Q4_0 7.0 / 5.6 / 5.4)
+    if (weights >= (6ull << 20) && weights < (1ull << 24)) return out_dim >= 8192;
+    if (weights < (1ull << 24)) return false;
+    const bool light_or_q5k = fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0;
+    if (out_dim >= 14336) return light_or_q5k || fmt == REIN_TYPE_Q8_0;
+    if (out_dim > 8192) return light_or_q5k || fmt == REIN_TYPE_Q6_K || (fmt == REIN_TYPE_Q8_0 && out_dim >= 12288);
+    return false;
+}
+
 bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
 {
     if (n_rows < 2 || n_rows > 4 || mvl_lds_bytes(in_dim, n_rows) > kLdsPerCu) return false;
@@ -398,14 +423,23 @@ bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
     if (opt_is_set(O_SKINNY_FROM) || opt_is_set(O_QUAD_FROM) || opt_is_set(O_MV_ROWS) || opt_is_set(O_MV_WPB)) return false;
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
     if (n_rows >= 3) {
-        // (up to 8192 rows and from 20 * 2^20 weights the 4x4x4 kernel with its contraction sliced over wavefronts is
-        // ahead of this one for every format but Q8_0 -- use_mvql)
-        if (fmt != REIN_TYPE_Q8_0 && out_dim <= 8192 && weights >= (20ull << 20) && opt_u(O_QUAD_LDS, 1) != 0) return false;
-        return weights >= (1ull << 24) && (out_dim <= 6144 || in_dim >= 8192);
+        // (where the 4x4x4 kernel with the rows in LDS is ahead of this one, it goes first -- mvql_few_rows)
+        if (opt_u(O_QUAD_LDS, 1) != 0 && mvql_few_rows(fmt, in_dim, out_dim)) return false;
+        if (weights >= (1ull << 24)) return out_dim <= 6144 || in_dim >= 8192;
+        // Smaller matrices with a contraction of 3584 and more: ahead of the plain dot4 kernel from six million weights
+        // (us at 4 rows, dot4 -> this: 8960 -> 1536 Q4_K 9.3 -> 6.7, Q8_0 9.2 -> 7.1, Q5_K 10.0 -> 7.0; 5632 -> 2048 6.6 -> 5.2,
+        // 6.4 -> 5.7, 7.1 -> 5.5, Q6_K 9.9 -> 6.4; 3584 -> 4608 8.3 -> 6.1, 9.7 -> 6.4; 8192 -> 1024 6.2 -> 5.8, 7.4 -> 5.9;
+        // level at four million weights and with short contractions -- 2048 -> 5632 5.7 = 5.7, 1536 -> 8960 7.3 -> 6.9, where
+        // the 4x4x4 kernels take 5.6)
+        // (Q6_K, whose unpack weighs most on the plain kernel, from four million weights and at any contraction: 4096 -> 1024
+        // 6.4 -> 4.7, 2048 -> 2048 4.7 -> 4.1, 2048 -> 5632 7.2 on the 4x4x4 kernel -> 6.8)
+        if (fmt == REIN_TYPE_Q6_K) return weights >= (4ull << 20) && out_dim <= 6144;
+        return weights >= (6ull << 20) && in_dim >= 3584 && out_dim <= 6144;
     }
     if (weights < (1ull << 25)) return false;
     if (in_dim >= 8192) return true;
-    return out_dim >= 14336 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S);
+    // (5120 -> 7168 Q4_K 8.5 -> 7.7 us, Q5_K 9.5 -> 9.2; 5120 -> 13824 13.0 -> 11.6, 14.8 -> 13.2)
+    return out_dim >= 7168 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S);
 }
 
 int launch_matvec_lds(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
@@ -534,15 +568,16 @@ bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
         return weights >= (5ull << 20) && out_dim <= 4096 && (in_dim >= 14336 || out_dim <= 1536);
     }
     if (n_rows >= 5) {
-        if (weights < (5ull << 20)) return false;
+        // (from four million weights with a contraction of 4096, every format but Q5_K: 4096 -> 1024 at 8 rows Q6_K 8.6 -> 6.7 us,
+        // Q8_0 7.4 -> 6.4, IQ4_XS 8.0 -> 6.3, Q4_0 7.7 -> 6.3, IQ3_S 7.5 -> 6.2, Q4_K 6.5 -> 6.3; Q5_K 5.8 -> 6.5 and 2048 -> 2048
+        // Q4_K 5.6 -> 6.0, Q5_K 5.3 -> 6.1 stay on dot4)
+        const bool from_4m = fmt != REIN_TYPE_Q5_K && weights >= (4ull << 20) && in_dim >= 4096;
+        if (weights < (5ull << 20) && !from_4m) return false;
         if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ4_XS) return true;
         const bool phased = g.phase_sub < in_dim / 32;
         return out_dim <= 20480 && !(phased && out_dim > 6144);
     }
-    if (fmt != REIN_TYPE_Q8_0 && out_dim <= 8192 && weights >= (20ull << 20)) return true;
-    if (weights < (1ull << 24)) return false;
-    return out_dim >= 14336 && (fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K ||
-                                fmt == REIN_TYPE_Q4_0);
+    return mvql_few_rows(fmt, in_dim, out_dim);
 }
 
 int launch_quad_lds(int fmt, const void* w, const void* xq, float* y, unsigned in_dim, unsigned out_dim,
