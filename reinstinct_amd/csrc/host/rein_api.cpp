@@ -554,7 +554,10 @@ bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
         // 23, 17408 -> 5120 127 -> 56, 14336 -> 4096 104 -> 40, 8192 -> 8192 70 -> 38, 28672 -> 8192 207 -> 111, 5120 -> 1024
         // 38 -> 14; Q6_K 69 -> 50, 230 -> 127, 188 -> 91, 114 -> 92; beyond (4096 -> 14336 0.72-1.30, 2048 -> 16384
         // 0.65-1.13) the tile launch has workgroups enough
-        return weights >= (1ull << 22) && out_dim <= 8192;
+        // A sweep over 20 further shapes moved the limit: the tile launch stays short of workgroups up to 16384 rows
+        // (tile launch / this at 24-32 rows: 8192 -> 10240 1.45-1.9, 4096 -> 14336 1.06-1.36, 5120 -> 13824 1.02-1.21,
+        // 6144 -> 16384 1.05-1.21) unless the contraction is short (1536 -> 8960 0.88-1.06).
+        return weights >= (1ull << 22) && (out_dim <= 8192 || (out_dim <= 16384 && in_dim >= 4096));
     if (n_rows > 8) {
         // 9-16 rows (rein_mmq_xq8 sends them here), against the skinny MMQ at 12 and 16 rows: Q6_K and Q5_K ahead on
         // narrow and on short-and-mid matrices (5120 -> 5120 1.27 / 1.13, 17408 -> 5120 1.29 / 1.17, 14336 -> 4096 1.30 /
@@ -562,10 +565,15 @@ bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
         // 1024 1.9 / 1.6), the other formats by 1.00-1.22 against at most 4096 rows with a long contraction and 1.28-1.42
         // at 5120 -> 1024; everything behind against many rows (5120 -> 34816 0.72-0.93, 5120 -> 17408 0.69-0.85,
         // 28672 -> 8192 0.69-0.92, 5120 -> 7168 0.83-1.01)
+        // The same 20 further shapes at 12 and 16 rows (skinny MMQ / this): every format 1.27-1.48 at 8192 -> 10240, where 320
+        // tiles of 32 rows deal badly over 256 CUs; the formats of the skinny MMQ also 1.25-1.37 at 4096 -> 1024 (four million
+        // weights), 1.18-1.28 at 5632 -> 2048, 1.08-1.28 at 16384 -> 6144 (0.99-1.08 at 13824 -> 5120, 0.84-0.91 at 3584 -> 4608,
+        // 0.86-1.03 at 2048 -> 2048: they stay).
         if (weights < (1ull << 22)) return false;
+        if (in_dim >= 8192 && out_dim > 8192 && out_dim <= 10240) return true;
         if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K)
             return out_dim <= 6144 || (in_dim <= 4096 && out_dim <= 16384) || (in_dim <= 8192 && out_dim <= 8192);
-        return weights >= (5ull << 20) && out_dim <= 4096 && (in_dim >= 14336 || out_dim <= 1536);
+        return out_dim <= 1536 || (out_dim <= 2048 && in_dim >= 4096) || (out_dim <= 6144 && in_dim >= 14336);
     }
     if (n_rows >= 5) {
         // (from four million weights with a contraction of 4096, every format but Q5_K: 4096 -> 1024 at 8 rows Q6_K 8.6 -> 6.7 us,
