@@ -340,11 +340,11 @@ int rein_mmq_xq8(int fmt, const void *w, const void *xq, float *y, unsigned in_d
                  unsigned out_dim, unsigned p_rows, rein_stream_t s);
 /* The same product with a caller-provided workspace of rein_mmq_workspace_bytes(fmt, in_dim,
  * p_rows) bytes (16-byte aligned; 0 = the row count has no use for one, and NULL
- * falls back to rein_mmq_xq8).  With it Q4_K from 320 rows up runs on the block-scaled fp6
+ * falls back to rein_mmq_xq8).  With it Q4_K from 128 rows up runs on the block-scaled fp6
  * matrix instruction: the activations are first brought into operand form in the workspace
  * (one extra launch), then the GEMM streams them from there (GEMMs of less than 2.8e10 operations
- * 2 M N K, about 50 us, and GEMMs whose 128-token workgroups do not come out even over the CUs and
- * that do not take the split-tail form below stay on the int8 tile).  The reference keeps such
+ * 2 M N K, about 50 us, and GEMMs with fewer than 1.25 four-tile token groups per CU that do not
+ * take the split-tail form below stay on the int8 tile).  The reference keeps such
  * scratch in its PrefillGemm object (src/runtime/prefill.rs:479-495); here the caller owns
  * it, so nothing allocates and the call can be captured into a graph.  Calls that share a
  * workspace must be ordered on one stream.

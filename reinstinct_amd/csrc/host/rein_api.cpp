@@ -1306,12 +1306,16 @@ unsigned sk_split(unsigned in_dim, unsigned out_dim, unsigned p_rows)
     return std::max(1u, std::min(forced ? forced : std::min(8u, room), most));
 }
 // The launch wants whole 4-tile token groups (a ragged last group computes its missing tiles all the same).
-// It pays where the tail is what decides: no whole round and a tail that splits at least two ways (small
-// grids that would leave CUs idle), or one whole round and a tail that splits at least four ways (512 x 17408:
-// 167-172 us against 189-204 for the mixed launch).  With more rounds the workgroups of the mixed launch
-// drift apart and overlap their fills and stores, which this launch's lock-step rounds do not (2048 tokens:
-// 575-690 us against 586-617), and an unsplit tail is the mixed launch's all-wide plan.  REIN_MMQ6_SK = 2
-// forces the launch wherever it is valid.
+// Against the mixed launch, over 23 model shapes x 14 token counts (us, split-tail / mixed): a tail that splits
+// two ways or more wins behind one to three rounds (4096 -> 11008 at 768 tokens 0.88, 5120 -> 17408 at 512
+// 154 / 175, at 1024 289 / 308) and most without one (17408 -> 5120 at 512: 183 / 290); an unsplit tail
+// behind one to three rounds is level or just ahead (0.92-1.06, median 0.98).  Behind four rounds and more the
+// mixed launch, whose workgroups drift apart and overlap their fills and stores, is as good without the second
+// launch (0.97-1.01) and steadier (2048 tokens x 17408: 575-690 us over runs against 586-617).  Without a whole round and with more units than CUs: up
+// to 1.3 units per CU the second slots of a quarter of the CUs set the time and the mixed launch's narrower
+// groups win (320-336 units: 1.12-1.23), from there on the launch is level (400-480 units 0.97-1.03) or
+// ahead (4096 -> 6144 at 1024 tokens, 384 units, 104 / 134).  REIN_MMQ6_SK = 2 forces the launch wherever it
+// is valid.
 bool mmq6_split_tail(unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
     const unsigned mode = opt_u(O_MMQ6_SK, 1);
@@ -1320,8 +1324,11 @@ bool mmq6_split_tail(unsigned in_dim, unsigned out_dim, unsigned p_rows)
     const unsigned n_tt = (p_rows + 31) / 32, n_tg = (n_tt + 3) / 4;
     if (8 * (4 * n_tg - n_tt) > n_tt) return false;                       // more than an eighth of the tiles empty
     if (mode == 2 || opt_is_set(O_MMQ6_SK_GRID)) return true;
-    const unsigned rounds = ((out_dim + 127) / 128) * n_tg / sk_grid(), split = sk_split(in_dim, out_dim, p_rows);
-    return (rounds == 0 && split >= 2) || (rounds == 1 && split >= 4);
+    const unsigned long long units = (unsigned long long)((out_dim + 127) / 128) * n_tg;
+    const unsigned long long rounds = units / sk_grid();
+    if (units % sk_grid() == 0 || rounds > 3) return false;
+    if (sk_split(in_dim, out_dim, p_rows) >= 2) return true;
+    return rounds != 0 || units >= kSkGrid * 2 / 3;
 }
 
 // Split-tail launch of the int8 tile (rein_mmq_split_tail in mmq_gemm.h): the same scheme for every dense
@@ -1333,7 +1340,7 @@ constexpr size_t kSk8PartBytes = (size_t)2 * 16 * 256 * 4;
 struct Sk8Plan { unsigned tm, g, n_unit, n_tail, split; bool take; double cost; };
 // One unit width: units, ranges per tail unit, whether the launch pays, and a cost to compare widths by (a
 // 64-token unit costs 1.68 32-token units; workgroups that have a CU to themselves run 1.4 times faster).
-Sk8Plan sk8_width(unsigned tm, unsigned g, unsigned in_dim, unsigned out_dim, unsigned p_rows)
+Sk8Plan sk8_width(int fmt, unsigned tm, unsigned g, unsigned in_dim, unsigned out_dim, unsigned p_rows)
 {
     Sk8Plan p{tm, g, 0, 0, 1, false, 0.0};
     const unsigned n_chunk = (in_dim + 255) / 256;
@@ -1349,9 +1356,16 @@ Sk8Plan sk8_width(unsigned tm, unsigned g, unsigned in_dim, unsigned out_dim, un
         p.split = std::max(1u, std::min(std::min(forced ? forced : std::min(cap, room), g / p.n_tail), n_chunk));
     }
     // it pays where the tail decides: no whole round and a tail that splits, or one whole round and a tail that
-    // splits four ways (5120 x 17408 at 256 tokens: 117 -> 106 us Q8_0, 210 -> 184 Q6_K; with more rounds the
-    // mixed launch, whose workgroups drift apart, is level or ahead)
-    p.take = (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4);
+    // splits four ways (5120 x 17408 at 256 tokens: 117 -> 106 us Q8_0, 210 -> 184 Q6_K).  With 64-token units
+    // also behind one or two whole rounds when the tail's workgroups have a CU each, split or not: over 23 model
+    // shapes x 14 token counts Q6_K gains in all 43 such cells (1.01-1.29 x, median 1.08; 17408 -> 5120 at 1024
+    // tokens 699 -> 566 us) and Q8_0 in all 42 (1.00-1.26 x; 346 -> 274 at 13824 -> 5120), while a tail on more
+    // than half the slots loses (0.85-1.07, median 0.96) and so does Q6_K behind three rounds and more (0.89-1.00
+    // without a tail, whose workgroups the plain launch lets drift apart).  Q4_K on the int8 tile gains only with a
+    // tail that splits (0.96-1.24 against 0.88-1.04 unsplit), and the formats not measured follow it.
+    const bool any_split = fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0;
+    p.take = (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4) ||
+             (tm == 64 && (rounds == 1 || rounds == 2) && p.n_tail != 0 && p.n_tail <= g / 2 && (any_split || p.split >= 2));
     const unsigned n_seg = p.n_tail * p.split;
     const double alone = rounds || n_seg >= g ? 1.0 : n_seg <= g / 2 ? 0.71 : 0.71 + 0.29 * (n_seg - g / 2) / (g / 2);
     p.cost = (tm == 64 ? 1.68 : 1.0) * (rounds + (p.n_tail ? alone / p.split : 0.0));
@@ -1368,7 +1382,7 @@ Sk8Plan sk8_plan(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows)
     const bool force = mode == 2 || opt_is_set(O_MMQ_SK_GRID);
     const unsigned n_tt = (p_rows + 31) / 32;
     const bool half_empty = 8 * (2 * ((n_tt + 1) / 2) - n_tt) > n_tt;   // more than an eighth of the 64-token units' tiles
-    Sk8Plan w64 = sk8_width(64, g, in_dim, out_dim, p_rows), w32 = sk8_width(32, g, in_dim, out_dim, p_rows);
+    Sk8Plan w64 = sk8_width(fmt, 64, g, in_dim, out_dim, p_rows), w32 = sk8_width(fmt, 32, g, in_dim, out_dim, p_rows);
     if (const unsigned forced_tm = opt_u(O_MMQ_SK_TM, 0)) {
         Sk8Plan p = forced_tm == 32 ? w32 : w64;
         p.take = p.take || force;
@@ -1411,10 +1425,7 @@ size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows);
 
 namespace {
 // Which launch a workspace of `bytes` gets: 0 plain int8, 1 fp6 one token group per workgroup, 2 fp6 split-tail,
-// 3 int8 split-tail.  The mixed fp6 launch wants a machine full of 4-tile groups: below three 32-token tiles per
-// resident slot (Q4_K 17408 -> 5120 at 448 tokens: 289 us against 176 on the int8 tile, 5120 -> 5120: 96 against
-// 60; 5120 -> 17408 at 384 tokens, 3.2 tiles per slot: 139 against 142-152) the GEMM stays on the int8 tile, unless
-// REIN_MMQ6_FROM asks for the fp6 path by name.
+// 3 int8 split-tail.  REIN_MMQ6_FROM asks for the fp6 path by name wherever its workspace is there.
 int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t bytes)
 {
     const size_t need = rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows);
@@ -1425,15 +1436,25 @@ int mmq_form(int fmt, unsigned in_dim, unsigned out_dim, unsigned p_rows, size_t
     const bool large = 2.0 * p_rows * (double)out_dim * in_dim >= 2.8e10;
     if (need != 0 && bytes >= need && (large || asked)) {
         if (bytes >= sk_workspace_bytes(in_dim, p_rows) && mmq6_split_tail(in_dim, out_dim, p_rows)) return 2;
-        // The mixed launch wants its 128-token workgroups to come out even over the CUs' two slots: up to two per
-        // CU (from 1.5, i.e. three 32-token tiles per slot), whole multiples, or five and more.  In between, the
-        // int8 launch with its finer grain is level or ahead (units per CU -> us fp6 against int8: 2.1 184 / 168,
-        // 2.5 233 / 212 and 722 / 660, 2.7 234 / 224, 3.2 281 / 262, 3.5 324 / 289, 4.25 318 / 300; but 1.9 153 / 172,
-        // 2.0 129 / 151, 3.0 193 / 233, 5.0 385 / 399, 8.5 622 / 665, 17 1115 / 1282).
-        const unsigned long long units = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 127) / 128);
-        const unsigned long long tiles = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 31) / 32);
-        const bool even = tiles >= 3ull * kSkGrid && (units <= kSkGrid || units % kCUs == 0 || units >= 5ull * kCUs);
-        if (even || asked) return 1;
+        const unsigned n_tt = (p_rows + 31) / 32, n_tg = (n_tt + 3) / 4;
+        const unsigned long long units = (unsigned long long)((out_dim + 127) / 128) * n_tg;
+        if (8 * (4 * n_tg - n_tt) <= n_tt) {
+            // Whole 4-tile token groups: from 1.25 groups per CU the fp6 tile is ahead of the int8 launches in
+            // every measured shape but two (int8 / fp6 0.93-1.25, median 1.15, over 110 cells of 23 model shapes);
+            // below that an unsplit launch leaves too many CUs with one workgroup against the int8 launch's
+            // finer grain (258-296 groups: 0.78-0.99) and the GEMM stays there.
+            if (units >= kSkGrid * 5 / 8 || asked) return 1;
+        } else {
+            // A ragged last group: the mixed launch cuts it into narrower workgroups, and comes out even over the
+            // CUs' two slots with up to two 128-token workgroups per CU (from three 32-token tiles per slot),
+            // whole multiples, or five and more (units per CU -> us fp6 against int8: 1.9 153 / 172, 2.0 129 / 151,
+            // 3.0 193 / 233, 5.0 385 / 399, 8.5 622 / 665; in between level or behind, 3584 -> 18944 at 320 tokens
+            // 108 / 94, 5120 -> 13824 at 448 tokens 1.15 x).  Below 320 tokens a ragged count stays on the int8 tile.
+            const unsigned long long u128 = (unsigned long long)((out_dim + 127) / 128) * ((p_rows + 127) / 128);
+            const unsigned long long tiles = (unsigned long long)((out_dim + 127) / 128) * n_tt;
+            const bool even = p_rows >= 320 && tiles >= 3ull * kSkGrid && (u128 <= kSkGrid || u128 % kCUs == 0 || u128 >= 5ull * kCUs);
+            if (even || asked) return 1;
+        }
     }
     return bytes >= (size_t)kSkGrid * kSk8PartBytes && sk8_plan(fmt, in_dim, out_dim, p_rows).take ? 3 : 0;
 }
@@ -1470,14 +1491,13 @@ bool mmq16_asked(int fmt, unsigned in_dim)
 
 size_t rein_mmq_workspace_min_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
-    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < opt_u(O_MMQ6_FROM, 320)) return 0;
+    if (!mmq6_format(fmt) || in_dim == 0 || in_dim % 256 != 0 || p_rows < opt_u(O_MMQ6_FROM, 128)) return 0;
     return x6_image_bytes(in_dim / 32, p_rows);
 }
 
 size_t rein_mmq_workspace_bytes(int fmt, unsigned in_dim, unsigned p_rows)
 {
-    // below ~300 rows the int8 launch (more, smaller workgroups in flight) is the faster one:
-    // 128 rows 61 vs 93 us, 256 rows 112 vs 122 us, 512 rows 185 vs 177 us at 5120 x 17408
+    // below 128 rows the fp6 launches never paid (their 4-tile token group is then mostly empty)
     if (rein_mmq_workspace_min_bytes(fmt, in_dim, p_rows) == 0) {
         // the int8 launch needs none; with room for its partial tiles it may run as a split-tail launch
         const bool dense = fmt_tag(fmt) && fmt != REIN_TYPE_Q5_1 && in_dim != 0 && p_rows > 16;

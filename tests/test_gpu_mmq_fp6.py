@@ -222,7 +222,8 @@ def test_split_tail_needs_the_full_workspace():
 
 
 def test_workspace_launches_at_the_benchmark_shape():
-    # 5120 x 17408 at 512 tokens (one whole round + 32 tiles split eight ways) and 2048 tokens (mixed launch):
+    # 5120 x 17408 at 512 tokens (one whole round + 32 tiles split eight ways), 1024 tokens (two rounds + 64 tiles
+    # split four ways) and 2048 tokens (mixed launch):
     # every element against the int8 launch, sampled tokens against the oracle; the default row threshold applies
     set_option("REIN_MMQ6_FROM", None)
     try:
@@ -233,7 +234,7 @@ def test_workspace_launches_at_the_benchmark_shape():
         x = np.random.default_rng(32).standard_normal((2048, in_dim)).astype(np.float32)
         dw, dq = dev(packed), quantized(x)
         xq = dq.to_host(np.uint8).reshape(2048, -1)
-        for m, form in ((512, 2), (2048, 1)):
+        for m, form in ((512, 2), (1024, 2), (2048, 1)):
             print(f"mmq6 benchmark shape M {m}", flush=True)
             ws_bytes = runtime.mmq_workspace_bytes(rein.Q4_K, in_dim, m)
             assert runtime.mmq_form_ws(rein.Q4_K, in_dim, out_dim, m, ws_bytes) == form

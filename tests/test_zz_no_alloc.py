@@ -40,9 +40,9 @@ def test_no_alloc_entry_matches_the_workspace_entry_twice_in_a_row():
     # launch forms of rein_mmq_form_ws: 1 the mixed fp6 launch (activation image only), 2 the fp6 split-tail launch
     # (image + one partial tile per workgroup), 3 the int8 split-tail launch, 0 the plain launch without scratch.
     # The second call of each pair is smaller than the first and finds the first one's contents in the array.
-    big = (2304, 14336)
-    assert run_pair(rein.Q4_K, 512, *big, seed=1) == 1
-    assert run_pair(rein.Q4_K, 448, *big, seed=2) == 1
+    big = (3072, 14336)
+    assert run_pair(rein.Q4_K, 384, *big, seed=1) == 1
+    assert run_pair(rein.Q4_K, 352, *big, seed=2) == 1
     tail = (5120, 6144)
     assert run_pair(rein.Q4_K, 512, *tail, seed=7) == 2
     assert run_pair(rein.Q4_K, 480, 4096, 8192, seed=8) == 2
@@ -52,10 +52,10 @@ def test_no_alloc_entry_matches_the_workspace_entry_twice_in_a_row():
     assert run_pair(rein.Q4_K, 40, 512, 136, seed=4) == 0
     # and once more the first shapes, after the others
     assert run_pair(rein.Q4_K, 512, *tail, seed=10) == 2
-    assert run_pair(rein.Q4_K, 512, *big, seed=5) == 1
+    assert run_pair(rein.Q4_K, 384, *big, seed=5) == 1
 
 
-@pytest.mark.parametrize("shape, form", [((512, 2304, 14336), 1), ((512, 5120, 6144), 2), ((448, 2048, 264), 3)])
+@pytest.mark.parametrize("shape, form", [((384, 3072, 14336), 1), ((512, 5120, 6144), 2), ((448, 2048, 264), 3)])
 def test_no_alloc_entry_under_stream_capture_and_without_touching_device_memory(shape, form):
     # rein_noalloc_prepare places the array outside any capture; after it a call may be recorded into a graph,
     # the replays give the bits of the eager call, and the free device memory the runtime reports does not move
