@@ -1363,9 +1363,11 @@ Sk8Plan sk8_width(int fmt, unsigned tm, unsigned g, unsigned in_dim, unsigned ou
     // than half the slots loses (0.85-1.07, median 0.96) and so does Q6_K behind three rounds and more (0.89-1.00
     // without a tail, whose workgroups the plain launch lets drift apart).  Q4_K on the int8 tile gains only with a
     // tail that splits (0.96-1.24 against 0.88-1.04 unsplit), and the formats not measured follow it.
+    // Q8_0, the cheapest chunk against the same fills, stays ahead up to six rounds (1.01-1.15 x in all 19 cells).
     const bool any_split = fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0;
+    const unsigned most_rounds = fmt == REIN_TYPE_Q8_0 ? 6 : 2;
     p.take = (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4) ||
-             (tm == 64 && (rounds == 1 || rounds == 2) && p.n_tail != 0 && p.n_tail <= g / 2 && (any_split || p.split >= 2));
+             (tm == 64 && rounds >= 1 && rounds <= most_rounds && p.n_tail != 0 && p.n_tail <= g / 2 && (any_split || p.split >= 2));
     const unsigned n_seg = p.n_tail * p.split;
     const double alone = rounds || n_seg >= g ? 1.0 : n_seg <= g / 2 ? 0.71 : 0.71 + 0.29 * (n_seg - g / 2) / (g / 2);
     p.cost = (tm == 64 ? 1.68 : 1.0) * (rounds + (p.n_tail ? alone / p.split : 0.0));
