@@ -651,6 +651,60 @@ def read_ceiling_us(stream, weights, nbytes):
     return best * 1e6
 
 
+def extras_mmq_launch_forms(stream):
+    """rein_mmq_xq8_ws picks one of four launches (rein_mmq_form_ws: 0 plain int8, 1 fp6 one token group per workgroup,
+    2 fp6 split-tail, 3 int8 split-tail).  Here each is forced through the library's options on model shapes other
+    than BASELINE's and timed beside the library's own choice: `lib_over_best` is what the choice leaves behind.
+    Forced options fall back where a form is not valid for the token count (a ragged last token group), so every
+    entry carries the form that actually ran."""
+    from reinstinct_amd import _lib
+    forms = {"int8": {"REIN_MMQ6": "0", "REIN_MMQ_SK": "0"}, "int8_split_tail": {"REIN_MMQ6": "0", "REIN_MMQ_SK": "2"},
+             "fp6_mixed": {"REIN_MMQ6_FROM": "1", "REIN_MMQ6_SK": "0"}, "fp6_split_tail": {"REIN_MMQ6_FROM": "1", "REIN_MMQ6_SK": "2"}}
+    names = sorted({k for f in forms.values() for k in f})
+    shapes = {rein.Q4_K: [(5120, 17408), (17408, 5120), (4096, 14336), (14336, 4096), (8192, 28672), (8192, 10240), (4096, 6144), (5120, 13824)],
+              rein.Q6_K: [(5120, 17408), (17408, 5120), (4096, 14336), (8192, 10240)],
+              rein.Q8_0: [(5120, 17408), (17408, 5120), (4096, 14336), (8192, 10240)]}
+    out = []
+    for f, shape_list in shapes.items():
+        for k, n in shape_list:
+            packed = tiled_weights(f, k, n, seed=5)
+            ws = [hip.DeviceBuf.from_host(packed) for _ in range(max(3, min(12, (400 << 20) // packed.nbytes + 1)))]
+            for m in (128, 256, 384, 512, 768, 1024, 2048):
+                x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+                dx, dq, dy = hip.DeviceBuf.from_host(x), hip.DeviceBuf(m * (k // 32) * 40), hip.DeviceBuf(m * n * 4)
+                runtime.quantize_q8(dx, dq, k, m, stream)
+
+                def timed():
+                    wsb = runtime.mmq_workspace_bytes(f, k, m)
+                    wsp = hip.DeviceBuf(wsb) if wsb else None
+                    form = runtime.mmq_form_ws(f, k, n, m, wsb)
+                    sec = time_graph(stream, lambda: [runtime.mmq_xq8_ws(f, w_, dq, dy, k, n, m, wsp, wsb, stream) for w_ in ws], len(ws), steps=3)
+                    return round(sec * 1e6, 1), form
+
+                timed()
+                entry = {"fmt": FMT_NAME[f], "K": k, "N": n, "M": m}
+                entry["lib_us"], entry["lib_form"] = timed()
+                by_form = {}
+                try:
+                    for name, opts in forms.items():
+                        if name.startswith("fp6") and f != rein.Q4_K:
+                            continue
+                        for o in names:
+                            _lib.set_option(o, opts.get(o))
+                        us, form = timed()
+                        by_form[form] = min(us, by_form.get(form, us))
+                finally:
+                    for o in names:
+                        _lib.set_option(o, None)
+                entry["us_by_form"] = {str(a): b for a, b in sorted(by_form.items())}
+                entry["lib_over_best"] = round(by_form.get(entry["lib_form"], entry["lib_us"]) / min(by_form.values()), 3)
+                out.append(entry)
+                log("mmq forms", entry)
+                del dx, dq, dy
+            del ws
+    return out
+
+
 def extras_barrier_cost(stream):
     """What a barrier across the workgroups of one launch costs through device memory (rein_measure_barrier, a
     measurement kernel in the code object: one workgroup per CU, nothing but the barrier, every wait bounded),
@@ -844,7 +898,8 @@ def main():
         out["extras"] = {"fused_producers": extras_fused(stream),
                          "other_matvec_sites": extras_ondisk(stream),
                          "decode_ffn_chain": extras_decode_ffn(stream),
-                         "barrier_cost": extras_barrier_cost(stream)}
+                         "barrier_cost": extras_barrier_cost(stream),
+                         "mmq_launch_forms": extras_mmq_launch_forms(stream)}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)
