@@ -209,6 +209,56 @@ def test_options_table():
     assert _lib.get_option("REIN_MV_ROWS") is None
 
 
+def test_mmq_form_ws_follows_the_launch_rules():
+    # rein_mmq_form_ws: host logic only -- which of the four launches rein_mmq_xq8_ws takes for a shape and a
+    # workspace size (0 plain int8, 1 fp6 one token group per workgroup, 2 fp6 split-tail, 3 int8 split-tail)
+    _lib.reset_options()
+    Q4_K, Q6_K, Q8_0 = rein.Q4_K, rein.Q6_K, rein.Q8_0
+
+    def form(fmt, k, n, m, bytes_=None):
+        full = runtime.mmq_workspace_bytes(fmt, k, m)
+        return runtime.mmq_form_ws(fmt, k, n, m, full if bytes_ is None else bytes_)
+
+    # units = 128-row blocks x 4-tile token groups on 512 resident slots
+    assert form(Q4_K, 5120, 17408, 512) == 2        # 544 units: one round + 32 that split eight ways
+    assert form(Q4_K, 5120, 17408, 1024) == 2       # two rounds + 64 that split four ways
+    assert form(Q4_K, 5120, 17408, 2048) == 1       # four rounds: the mixed launch
+    assert form(Q4_K, 8192, 8192, 1024) == 1        # 512 units: no tail
+    assert form(Q4_K, 8192, 28672, 256) == 2        # 448 units, no round, unsplit: from 341 units split-tail
+    assert form(Q4_K, 8192, 10240, 512) == 1        # 320 units: 1.25 per CU, the mixed launch's narrower groups
+    assert form(Q4_K, 5120, 17408, 256) in (0, 3)   # 272 units: too few for an unsplit fp6 launch
+    assert form(Q4_K, 8192, 28672, 128) == 2        # from 128 rows when the GEMM is large and the tail splits
+    assert form(Q4_K, 8192, 28672, 127) in (0, 3)   # below 128 rows never
+    assert form(Q4_K, 4096, 4096, 128) in (0, 3)    # 2 M N K below 2.8e10
+    assert form(Q4_K, 3584, 18944, 320) in (0, 3)   # ragged last token group (10 tiles in three groups), not even
+    assert form(Q4_K, 5120, 17408, 1984) == 1       # ragged, but five and more 128-token workgroups per CU
+    # the image alone admits the mixed launch only; less than the image is the caller's error, not a form
+    image = runtime.mmq_workspace_min_bytes(Q4_K, 5120, 512)
+    assert 0 < image < runtime.mmq_workspace_bytes(Q4_K, 5120, 512)
+    assert form(Q4_K, 5120, 17408, 512, image) in (0, 1)
+    assert form(Q4_K, 5120, 17408, 512, 0) == 0
+    # int8 split-tail with 64-token units: behind one or two rounds when the tail has a CU per workgroup
+    assert form(Q6_K, 17408, 5120, 1024) == 3       # 640 units: one round + 128, two ranges each
+    assert form(Q6_K, 5120, 17408, 512) == 3        # 1088 units: two rounds + 64
+    assert form(Q6_K, 5120, 17408, 1024) == 0       # four rounds
+    assert form(Q6_K, 8192, 10240, 640) == 0        # one round + 288 units: more than half the slots
+    assert form(Q8_0, 5120, 17408, 1024) == 3       # Q8_0 keeps the form up to six rounds
+    assert form(Q8_0, 5120, 17408, 2048) == 0       # eight rounds
+    assert form(Q6_K, 17408, 5120, 64) == 3         # 40 units on 256 CUs
+    assert form(Q6_K, 17408, 5120, 64, 0) == 0
+    # every answer is a form, and the fp6 forms belong to Q4_K with whole superblocks from 128 rows
+    rng = np.random.default_rng(5)
+    for _ in range(3000):
+        fmt = [Q4_K, Q6_K, Q8_0, rein.Q5_K, rein.Q4_0, rein.IQ4_XS, rein.IQ3_S][rng.integers(7)]
+        k = int(rng.integers(1, 120)) * (32 if fmt in (Q8_0, rein.Q4_0) else 256)
+        n, m = int(rng.integers(1, 40000)), int(rng.integers(1, 3000))
+        got = form(fmt, k, n, m)
+        assert got in (0, 1, 2, 3)
+        if got in (1, 2):
+            assert fmt == Q4_K and k % 256 == 0 and m >= 128 and 2.0 * m * n * k >= 2.8e10
+        assert form(fmt, k, n, m, 0) == 0
+
+
 def test_matvec_kernel_name_follows_the_dispatch_rules():
     # rein_matvec_kernel_name: host logic only -- which kernel 1..32 activation rows launch for a shape, by the rules
     # beside use_mvl / use_mvql / use_quad in rein_api.cpp and the option table
