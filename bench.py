@@ -81,6 +81,22 @@ def weight_rotation(packed, min_bytes=CACHE_BYTES):
     return bufs
 
 
+CLOCK_SETTLE_S = 0.08
+
+
+def settle(launch, stream, seconds=CLOCK_SETTLE_S):
+    """Untimed repetitions of the launches about to be timed, for `seconds` of wall time.  The GPU raises its
+    clocks over tens of milliseconds of continuous work: the first 4 ms after an idle stretch (host-side
+    preparation of the next case) run the 512-token prefill GEMM at 176 us per launch, the steady state is
+    143-146 us.  Every timed region of this file starts from that steady state; the W warm-up steps follow."""
+    t_end = time.perf_counter() + seconds
+    while True:
+        launch()
+        stream.synchronize()
+        if time.perf_counter() >= t_end:
+            return
+
+
 class MatvecCase:
     """A rotation of weight buffers and a captured graph of one pass over them."""
 
@@ -118,6 +134,7 @@ class MatvecCase:
 
     def time(self, steps, warmup):
         """-> (seconds per step, seconds per launch), events on the launch stream"""
+        settle(self.step, self.stream)
         for _ in range(warmup):
             self.step()
         self.stream.synchronize()
@@ -154,6 +171,7 @@ class MmqCase:
                            self.p, self.ws, self.ws_bytes, self.stream)
 
     def time(self, launches, warmup):
+        settle(lambda: [self.launch(i) for i in range(self.n_buf)], self.stream)
         for i in range(warmup):
             self.launch(i)
         self.stream.synchronize()
@@ -230,8 +248,7 @@ def time_graph(stream, launch_all, n_launches, steps=5):
     launch_all()
     g = stream.end_capture()
     ex = g.instantiate()
-    ex.launch(stream)
-    stream.synchronize()
+    settle(lambda: ex.launch(stream), stream)
     e0, e1 = hip.Event(), hip.Event()
     e0.record(stream)
     for _ in range(steps):
@@ -777,6 +794,7 @@ def main():
     fmt = rein.FORMATS[args.fmt]
 
     cases = [MatvecCase(fmt, k, n, args.batch, stream, seed=1234 + i) for i, (k, n) in enumerate(HEADLINE_SHAPES)]
+    settle(lambda: [c.step() for c in cases], stream)
     for c in cases:
         for _ in range(args.warmup):
             c.step()
@@ -821,7 +839,7 @@ def main():
     out = {
         "metric": "Q4_K decode matvec HBM GB/s (% of peak) + MMQ pp512 int8 TOPS, 1 MI355X",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(total_s / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "clock_settle_ms": round(CLOCK_SETTLE_S * 1e3), "ms_per_step": round(total_s / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8 (int8 dot4, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.fmt} repacked-v2 decode matvec, batch {args.batch}, BASELINE configs[1] shapes "
                                "5120->5120, 5120->34816 (fused gate+up), 17408->5120; value = total algorithmic bytes "
