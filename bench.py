@@ -88,7 +88,10 @@ def settle(launch, stream, seconds=CLOCK_SETTLE_S):
     """Untimed repetitions of the launches about to be timed, for `seconds` of wall time.  The GPU raises its
     clocks over tens of milliseconds of continuous work: the first 4 ms after an idle stretch (host-side
     preparation of the next case) run the 512-token prefill GEMM at 176 us per launch, the steady state is
-    143-146 us.  Every timed region of this file starts from that steady state; the W warm-up steps follow."""
+    143-156 us.  Every timed region of this file starts from that steady state; the W warm-up steps follow.
+    `launch` issues the kernels one by one, not as a graph: rocprofv3 7.2 ends a process with a segmentation
+    fault once about 16 000 kernels have been dispatched from hipGraphs (plain launches: 43 000 and counting),
+    and this file has to run under it."""
     t_end = time.perf_counter() + seconds
     while True:
         launch()
@@ -134,7 +137,7 @@ class MatvecCase:
 
     def time(self, steps, warmup):
         """-> (seconds per step, seconds per launch), events on the launch stream"""
-        settle(self.step, self.stream)
+        settle(lambda: [self.launch(w) for w in self.weights], self.stream)
         for _ in range(warmup):
             self.step()
         self.stream.synchronize()
@@ -248,7 +251,9 @@ def time_graph(stream, launch_all, n_launches, steps=5):
     launch_all()
     g = stream.end_capture()
     ex = g.instantiate()
-    settle(lambda: ex.launch(stream), stream)
+    settle(launch_all, stream)
+    ex.launch(stream)
+    stream.synchronize()
     e0, e1 = hip.Event(), hip.Event()
     e0.record(stream)
     for _ in range(steps):
@@ -794,7 +799,7 @@ def main():
     fmt = rein.FORMATS[args.fmt]
 
     cases = [MatvecCase(fmt, k, n, args.batch, stream, seed=1234 + i) for i, (k, n) in enumerate(HEADLINE_SHAPES)]
-    settle(lambda: [c.step() for c in cases], stream)
+    settle(lambda: [c.launch(w) for c in cases for w in c.weights], stream)
     for c in cases:
         for _ in range(args.warmup):
             c.step()
