@@ -119,8 +119,9 @@ def test_row_permutation_is_bit_exact(fmt):
 @pytest.mark.parametrize("fmt", [rein.Q4_K, rein.Q6_K, rein.Q8_0])
 def test_prefill_gemm_full_size(fmt, entry):
     # "plain" is rein_mmq_xq8 (the reference's call shape), "workspace" is rein_mmq_xq8_ws with the
-    # workspace rein_mmq_workspace_bytes asks for: the entry the benchmark times (fp6 launch for Q4_K from
-    # 320 rows, split-tail launch of the int8 tile at 128 rows)
+    # workspace rein_mmq_workspace_bytes asks for: the entry the benchmark times (Q4_K: fp6 split-tail launch at
+    # 512 rows, fp6 mixed launch at 2048, split-tail launch of the int8 tile at 128; Q6_K and Q8_0: the int8
+    # split-tail launch at 128 and 512 rows, the plain launch at 2048)
     in_dim, out_dim = 5120, 17408
     raw, packed = gaussian_weights(fmt, in_dim, out_dim, seed=21)
     dw = dev(packed)
