@@ -783,6 +783,9 @@ def main():
     ap.add_argument("--no-mmq", action="store_true")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the objects of BASELINE configs[2..4] (MMQ formats x M, MoE expert FFN, decode weight stream)")
+    ap.add_argument("--configs", default="",
+                    help="comma-separated names of the `configs` objects to run instead of all of them (a profiler run that "
+                         "wants one leg: rocprofv3 cannot follow the whole line, see settle())")
     ap.add_argument("--extras", action="store_true",
                     help="also time the fused producers, the MoE decode path, the remaining matvec sites and the decode FFN chain")
     ap.add_argument("--fmt", default="q4_k")
@@ -897,10 +900,17 @@ def main():
         del mm
 
     if not args.no_configs:
-        out["configs"] = {"decode_sweep_configs1": decode_sweep(stream, args.steps), "mmq_configs2": extras_mmq(stream), "mmq_short_prompts": extras_mmq_small(stream),
-                          "moe_configs3": extras_moe(stream), "moe_configs3_one_token": extras_moe_decode(stream),
-                          "decode_stream_configs4": extras_decode_stream(stream),
-                          "decode_layer_separate_tensors": extras_decode_layer_separate(stream)}
+        legs = {"decode_sweep_configs1": lambda: decode_sweep(stream, args.steps), "mmq_configs2": lambda: extras_mmq(stream),
+                "mmq_short_prompts": lambda: extras_mmq_small(stream),
+                "moe_configs3": lambda: extras_moe(stream), "moe_configs3_one_token": lambda: extras_moe_decode(stream),
+                "decode_stream_configs4": lambda: extras_decode_stream(stream),
+                "decode_layer_separate_tensors": lambda: extras_decode_layer_separate(stream)}
+        wanted = [n for n in args.configs.split(",") if n] if args.configs else list(legs)
+        unknown = [n for n in wanted if n not in legs]
+        if unknown:
+            print(f"bench.py: --configs knows {', '.join(legs)}; got {', '.join(unknown)}", file=sys.stderr)
+            sys.exit(2)
+        out["configs"] = {n: legs[n]() for n in legs if n in wanted}
 
     if args.sweep:
         sweep = []
