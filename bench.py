@@ -786,8 +786,9 @@ def main():
     ap.add_argument("--configs", default="",
                     help="comma-separated names of the `configs` objects to run instead of all of them (a profiler run that "
                          "wants one leg: rocprofv3 cannot follow the whole line, see settle())")
-    ap.add_argument("--extras", action="store_true",
-                    help="also time the fused producers, the MoE decode path, the remaining matvec sites and the decode FFN chain")
+    ap.add_argument("--extras", nargs="?", const="all", default="",
+                    help="also time the fused producers, the remaining matvec sites, the decode FFN chain, the barrier cost and "
+                         "the launch forms of the prefill GEMM; with a comma-separated list of their names, only those")
     ap.add_argument("--fmt", default="q4_k")
     ap.add_argument("--batch", type=int, default=1)
     args = ap.parse_args()
@@ -928,11 +929,14 @@ def main():
         out["sweep"] = sweep
 
     if args.extras:
-        out["extras"] = {"fused_producers": extras_fused(stream),
-                         "other_matvec_sites": extras_ondisk(stream),
-                         "decode_ffn_chain": extras_decode_ffn(stream),
-                         "barrier_cost": extras_barrier_cost(stream),
-                         "mmq_launch_forms": extras_mmq_launch_forms(stream)}
+        legs = {"fused_producers": extras_fused, "other_matvec_sites": extras_ondisk, "decode_ffn_chain": extras_decode_ffn,
+                "barrier_cost": extras_barrier_cost, "mmq_launch_forms": extras_mmq_launch_forms}
+        wanted = list(legs) if args.extras == "all" else [n for n in args.extras.split(",") if n]
+        unknown = [n for n in wanted if n not in legs]
+        if unknown:
+            print(f"bench.py: --extras knows {', '.join(legs)}; got {', '.join(unknown)}", file=sys.stderr)
+            sys.exit(2)
+        out["extras"] = {n: legs[n](stream) for n in legs if n in wanted}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fmt, 5120, 5120, seed=1234)
