@@ -400,7 +400,8 @@ void mvl_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, u
 //   * between 8192 and 14336 rows: Q4_K, Q5_K, Q6_K and their kin (5120 -> 13824 at 4 rows, 4x4x4 without LDS -> this: Q4_K
 //     14.0 -> 12.4, Q5_K 17.7 -> 14.7; 8192 -> 10240, LDS dot4 -> this: 16.8 -> 15.6, 20.0 -> 19.1, Q6_K 24.5 -> 21.9), Q8_0
 //     from 12288 rows (19.8 -> 17.1; 8192 -> 10240 21.4 on LDS dot4 against 22.9);
-//   * from 14336 rows: the formats with a cheap unpack and Q5_K.
+//   * from 14336 rows: every format but IQ4_XS (measured again from steady clocks, 4x4x4 without LDS -> this at 4 rows: Q6_K
+//     5120 -> 34816 40.7 -> 36.7, 6144 -> 16384 23.6 -> 21.7, 3584 -> 18944 18.2 -> 17.9).
 bool mvql_few_rows(int fmt, unsigned in_dim, unsigned out_dim)
 {
     const unsigned long long weights = (unsigned long long)in_dim * out_dim;
@@ -411,7 +412,7 @@ bool mvql_few_rows(int fmt, unsigned in_dim, unsigned out_dim)
     if (weights >= (6ull << 20) && weights < (1ull << 24)) return out_dim >= 8192;
     if (weights < (1ull << 24)) return false;
     const bool light_or_q5k = fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S || fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0;
-    if (out_dim >= 14336) return light_or_q5k || fmt == REIN_TYPE_Q8_0;
+    if (out_dim >= 14336) return light_or_q5k || fmt == REIN_TYPE_Q8_0 || fmt == REIN_TYPE_Q6_K;
     if (out_dim > 8192) return light_or_q5k || fmt == REIN_TYPE_Q6_K || (fmt == REIN_TYPE_Q8_0 && out_dim >= 12288);
     return false;
 }
@@ -438,7 +439,9 @@ bool use_mvl(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
     }
     if (weights < (1ull << 25)) return false;
     if (in_dim >= 8192) return true;
-    // (5120 -> 7168 Q4_K 8.5 -> 7.7 us, Q5_K 9.5 -> 9.2; 5120 -> 13824 13.0 -> 11.6, 14.8 -> 13.2)
+    // (5120 -> 7168 Q4_K 8.5 -> 7.7 us, Q5_K 9.5 -> 9.2; 5120 -> 13824 13.0 -> 11.6, 14.8 -> 13.2; Q8_0 from 13824 rows:
+    // 5120 -> 34816 35.4 -> 32.4, 5120 -> 13824 16.1 -> 15.2, 6144 -> 16384 20.7 -> 19.6, level at 7168 rows and at 3584 -> 18944)
+    if (fmt == REIN_TYPE_Q8_0) return out_dim >= 13824 && in_dim >= 4096;
     return out_dim >= 7168 && (fmt == REIN_TYPE_Q4_K || fmt == REIN_TYPE_Q4_0 || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_IQ3_S);
 }
 

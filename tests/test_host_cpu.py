@@ -273,13 +273,16 @@ def test_matvec_kernel_name_follows_the_dispatch_rules():
     assert name(rein.Q4_K, 17408, 5120, 2) == "rein_mvl_q4k_r1_b2"
     assert name(rein.Q4_K, 5120, 34816, 2) == "rein_mvl_q4k_r2_b2"
     assert name(rein.Q6_K, 5120, 34816, 2) == "rein_mv_q6k_r2_b2"
+    assert name(rein.Q8_0, 5120, 34816, 2) == "rein_mvl_q8_0_r2_b2"
+    assert name(rein.Q8_0, 5120, 7168, 2) == "rein_mv_q8_0_r2_b2"
     assert name(rein.Q4_K, 5120, 5120, 2) == "rein_mv_q4k_r2_b2"
     # three to four rows: the sliced 4x4x4 kernel on narrow matrices (not Q8_0), LDS-staged dot4 for Q8_0 and mid sizes
     assert name(rein.Q4_K, 5120, 5120, 4) == "rein_mvql_q4k_t4"
     assert name(rein.Q8_0, 5120, 5120, 3) == "rein_mvl_q8_0_r1_b4"
     assert name(rein.Q4_K, 4096, 4096, 4) == "rein_mvl_q4k_r1_b4"
     assert name(rein.Q4_K, 5120, 34816, 4) == "rein_mvql_q4k_t4"
-    assert name(rein.Q6_K, 5120, 34816, 4) == "rein_mvq_q6k_t4"
+    assert name(rein.Q6_K, 5120, 34816, 4) == "rein_mvql_q6k_t4"
+    assert name(rein.IQ4_XS, 5120, 34816, 4) == "rein_mvq_iq4xs_t4"           # the 4x4x4 kernel without LDS
     assert name(rein.Q4_K, 2048, 1536, 4) == "rein_mv_q4k_r1_b4"            # small matrices stay on dot4
     # five to eight rows
     assert name(rein.Q4_K, 17408, 5120, 8) == "rein_mvql_q4k_t8"
