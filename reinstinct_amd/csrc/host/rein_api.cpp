@@ -576,7 +576,14 @@ bool use_mvql(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows)
         if (in_dim >= 8192 && out_dim > 8192 && out_dim <= 10240) return true;
         if (fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K)
             return out_dim <= 6144 || (in_dim <= 4096 && out_dim <= 16384) || (in_dim <= 8192 && out_dim <= 8192);
-        return out_dim <= 1536 || (out_dim <= 2048 && in_dim >= 4096) || (out_dim <= 6144 && in_dim >= 14336);
+        // Measured again with every timing from steady clocks (the sweeps above ran the families of a cell one after the
+        // other from cold clocks, the skinny MMQ last): contractions that are a multiple of 4096 -- the slices of a row
+        // group's contraction come out even -- are ahead up to 14336 rows (skinny MMQ / this at 12 / 16 rows, Q4_K and Q8_0:
+        // 4096 -> 4096 1.06 / 1.09 and 1.14 / 1.18, 4096 -> 6144 1.07 / 1.09 and 1.08 / 1.12, 4096 -> 14336 1.09 / 1.08 and
+        // 1.20 / 1.22), and 13824 -> 5120 (1.07 / 1.10, 1.07 / 1.12) joins the long contractions against at most 6144 rows;
+        // 5120 -> 5120 (0.95-1.04), 3584 -> 4608 (0.88-0.94), 5120 -> 7168 (0.81-0.88), 5120 -> 13824 (0.93-1.04) stay.
+        return out_dim <= 1536 || (out_dim <= 2048 && in_dim >= 4096) || (out_dim <= 6144 && in_dim >= 13824) ||
+               (in_dim % 4096 == 0 && out_dim <= 14336);
     }
     if (n_rows >= 5) {
         // (from four million weights with a contraction of 4096, every format but Q5_K: 4096 -> 1024 at 8 rows Q6_K 8.6 -> 6.7 us,

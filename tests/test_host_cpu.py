@@ -291,6 +291,9 @@ def test_matvec_kernel_name_follows_the_dispatch_rules():
     # nine and more rows arrive through rein_mmq_xq8
     assert name(rein.Q6_K, 5120, 5120, 12) == "rein_mvql_q6k_t16"
     assert name(rein.Q4_K, 5120, 5120, 12) == "rein_mmqs_q4k_v8"
+    assert name(rein.Q4_K, 4096, 14336, 12) == "rein_mvql_q4k_t16"            # a contraction that is a multiple of 4096
+    assert name(rein.Q4_K, 5120, 13824, 12) == "rein_mmqs_q4k_v8"
+    assert name(rein.Q8_0, 13824, 5120, 16) == "rein_mvql_q8_0_t16"           # long contraction against at most 6144 rows
     assert name(rein.Q4_K, 5120, 5120, 32) == "rein_mvql_q4k_t32w"            # the build for sixteen wavefronts
     assert name(rein.Q6_K, 5120, 5120, 32) == "rein_mvql_q6k_t32"             # Q6_K: the build for eight
     assert name(rein.Q4_K, 5120, 34816, 32) == ""                             # token tiles
