@@ -391,8 +391,8 @@ void mvl_geometry(int fmt, unsigned in_dim, unsigned out_dim, unsigned n_rows, u
 //             14336 -> 4096 0.97-1.24, 8192 -> 8192 1.03-1.16, 28672 -> 8192 1.12-1.28, 18944 -> 3584 1.10-1.63,
 //             8192 -> 28672 1.10-1.34); on shorter contractions only Q4_K, Q4_0 and Q5_K against 14336 rows and
 //             more (5120 -> 34816 1.13 / 1.08 / 1.06, 5120 -> 17408 1.17 / 1.14 / 1.09, 3584 -> 18944 1.16 / 1.13 /
-//             1.05, 4096 -> 14336 1.04 / 1.08 / 1.03) and IQ3_S (1.05-1.14); Q6_K 0.91-1.10, IQ4_XS 0.97-1.06, Q8_0
-//             0.95-1.08 there.
+//             1.05, 4096 -> 14336 1.04 / 1.08 / 1.03) and IQ3_S (1.05-1.14); Q6_K 0.91-1.10 and IQ4_XS 0.97-1.06
+//             there; Q8_0 from 13824 rows at contractions of 4096 and more (timed from steady clocks: 1.06-1.09).
 // Three and four rows on the 4x4x4 kernel with the rows in LDS (the shape part of use_mvql's rule, shared with use_mvl):
 //   * up to 8192 rows and from 20 * 2^20 weights, every format but Q8_0 (contraction sliced over wavefronts);
 //   * Q6_K with a long contraction against very few rows (us at 4 rows, dot4 / LDS dot4 / this: 8192 -> 1024 10.5 / 9.4 /
