@@ -1372,9 +1372,10 @@ Sk8Plan sk8_width(int fmt, unsigned tm, unsigned g, unsigned in_dim, unsigned ou
     // tokens 699 -> 566 us) and Q8_0 in all 42 (1.00-1.26 x; 346 -> 274 at 13824 -> 5120), while a tail on more
     // than half the slots loses (0.85-1.07, median 0.96) and so does Q6_K behind three rounds and more (0.89-1.00
     // without a tail, whose workgroups the plain launch lets drift apart).  Q4_K on the int8 tile gains only with a
-    // tail that splits (0.96-1.24 against 0.88-1.04 unsplit), and the formats not measured follow it.
+    // tail that splits (0.96-1.24 against 0.88-1.04 unsplit).  Q5_K, Q4_0 and IQ4_XS, timed from steady clocks on the same
+    // shapes: 1.13-1.16 x in the median with a tail that splits (0.95-1.28), 1.01-1.03 x unsplit (0.99-1.20); IQ3_S follows IQ4_XS.
     // Q8_0, the cheapest chunk against the same fills, stays ahead up to six rounds (1.01-1.15 x in all 19 cells).
-    const bool any_split = fmt == REIN_TYPE_Q6_K || fmt == REIN_TYPE_Q5_K || fmt == REIN_TYPE_Q8_0;
+    const bool any_split = fmt != REIN_TYPE_Q4_K;
     const unsigned most_rounds = fmt == REIN_TYPE_Q8_0 ? 6 : 2;
     p.take = (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4) ||
              (tm == 64 && rounds >= 1 && rounds <= most_rounds && p.n_tail != 0 && p.n_tail <= g / 2 && (any_split || p.split >= 2));
