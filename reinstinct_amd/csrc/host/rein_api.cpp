@@ -1376,7 +1376,8 @@ Sk8Plan sk8_width(int fmt, unsigned tm, unsigned g, unsigned in_dim, unsigned ou
     // shapes: 1.13-1.16 x in the median with a tail that splits (0.95-1.28), 1.01-1.03 x unsplit (0.99-1.20); IQ3_S follows IQ4_XS.
     // Q8_0, the cheapest chunk against the same fills, stays ahead up to six rounds (1.01-1.15 x in all 19 cells).
     const bool any_split = fmt != REIN_TYPE_Q4_K;
-    const unsigned most_rounds = fmt == REIN_TYPE_Q8_0 ? 6 : 2;
+    // Behind a third round the other formats but Q4_K are level or ahead as well (0.98-1.16, median 1.02 over 32 cells).
+    const unsigned most_rounds = fmt == REIN_TYPE_Q8_0 ? 6 : fmt == REIN_TYPE_Q4_K ? 2 : 3;
     p.take = (rounds == 0 && p.split >= 2) || (rounds == 1 && p.split >= 4) ||
              (tm == 64 && rounds >= 1 && rounds <= most_rounds && p.n_tail != 0 && p.n_tail <= g / 2 && (any_split || p.split >= 2));
     const unsigned n_seg = p.n_tail * p.split;

@@ -241,6 +241,7 @@ def test_mmq_form_ws_follows_the_launch_rules():
     assert form(Q6_K, 17408, 5120, 1024) == 3       # 640 units: one round + 128, two ranges each
     assert form(Q6_K, 5120, 17408, 512) == 3        # 1088 units: two rounds + 64
     assert form(Q6_K, 5120, 17408, 1024) == 0       # four rounds
+    assert form(Q6_K, 3584, 18944, 768) == 3        # 1776 units: three rounds + 240
     assert form(Q6_K, 8192, 10240, 640) == 0        # one round + 288 units: more than half the slots
     assert form(Q8_0, 5120, 17408, 1024) == 3       # Q8_0 keeps the form up to six rounds
     assert form(Q8_0, 5120, 17408, 2048) == 0       # eight rounds
